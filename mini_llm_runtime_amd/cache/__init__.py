@@ -1,0 +1,19 @@
+"""Paged keys and values, block tables, and per-request state slots."""
+
+from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
+from .manager import CacheManager, CacheStats, KVGroup, RequestCache, StepLayout
+from .spec import PagedKVSpec, SlotStateSpec
+
+__all__ = [
+    "BlockAllocator",
+    "BlockPoolExhaustedError",
+    "CacheManager",
+    "CacheStats",
+    "KVGroup",
+    "PagedKVSpec",
+    "RequestCache",
+    "SlotPool",
+    "SlotStateSpec",
+    "StepLayout",
+    "blocks_for",
+]

@@ -1,0 +1,492 @@
+"""The cache manager: pages of keys and values with a block table per request,
+one pool per group of execution sites with equal needs, and fixed-size state
+slots per request.
+
+It is the single owner of page ids, block tables and slots, as the reference's
+`PagedKVCacheManager` is of its allocator, storage and request registry
+(src/mini_llm_runtime/paged_kv_manager.py:53-211).  The transaction rules are the
+reference's (src/mini_llm_runtime/paged_kv_cache.py:202-243): a step begins by
+taking the pages its tokens need (all requests or none), the model writes into
+them, commit makes the tokens count, abort gives back only the pages this step
+took and leaves the written bytes as invisible garbage.
+
+Beyond the reference: several groups (each with pages and a free list of its
+own), windows (pages that every later query has passed are given back at
+commit), capacity promised by count instead of by pinning pages, and state slots.
+
+Page layout of every pool: [site, page, kv_head, offset in page, head_dim], the
+reference's inner order (src/mini_llm_runtime/paged_kv_cache.py:287-318).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
+from .spec import PagedKVSpec, SlotStateSpec
+
+SiteSpec = Union[PagedKVSpec, SlotStateSpec, None]
+
+_TORCH_DTYPES = {
+    "float32": torch.float32,
+    "bfloat16": torch.bfloat16,
+    "int32": torch.int32,
+}
+
+
+class KVGroup:
+    """Execution sites whose caches have the same shape and window share one pool."""
+
+    def __init__(
+        self,
+        index: int,
+        spec: PagedKVSpec,
+        sites: Sequence[int],
+        num_blocks: int,
+        block_size: int,
+        dtype: torch.dtype,
+        device: torch.device,
+    ) -> None:
+        self.index = index
+        self.spec = spec
+        self.sites = tuple(sites)
+        self.site_position = {site: i for i, site in enumerate(self.sites)}
+        self.allocator = BlockAllocator(num_blocks)
+        self.block_size = block_size
+        shape = (len(self.sites), num_blocks, spec.num_kv_heads, block_size, spec.head_dim)
+        # never zeroed: stale bytes must be unreachable, not clean
+        self.key = torch.empty(shape, dtype=dtype, device=device)
+        self.value = torch.empty(shape, dtype=dtype, device=device)
+
+    @property
+    def num_blocks(self) -> int:
+        return self.allocator.total_blocks
+
+    def dead_blocks(self, num_tokens: int) -> int:
+        """How many leading pages no query at position >= num_tokens can see."""
+        if self.spec.window is None:
+            return 0
+        first_visible = num_tokens - self.spec.window + 1
+        return max(0, first_visible // self.block_size)
+
+    def lifetime_blocks(self, max_tokens: int, max_step_tokens: int) -> int:
+        """Most pages a request holds at one time over its life."""
+        full = blocks_for(max_tokens, self.block_size)
+        if self.spec.window is None:
+            return full
+        # the window before the first query of a step, the step's own tokens, and
+        # one page for the misalignment of the window's start
+        bounded = blocks_for(self.spec.window - 1 + max_step_tokens, self.block_size) + 1
+        return min(full, bounded)
+
+    def storage_bytes(self) -> int:
+        return 2 * self.key.numel() * self.key.element_size()
+
+
+class StateBank:
+    """Two copies of a fixed-size state per request slot: a step reads one and
+    writes the other, commit swaps them, so an aborted step changes nothing."""
+
+    def __init__(self, site: int, spec: SlotStateSpec, num_slots: int, device: torch.device) -> None:
+        self.site = site
+        self.spec = spec
+        self.tensor = torch.zeros((num_slots * 2, *spec.shape), dtype=_TORCH_DTYPES[spec.dtype], device=device)
+
+
+@dataclass
+class RequestCache:
+    request_id: str
+    slot: int
+    num_tokens: int = 0
+    tables: list[list[int]] = field(default_factory=list)
+    reserved: list[int] = field(default_factory=list)
+    has_reservation: bool = False
+    state_parity: int = 0
+    pending_tokens: int = 0
+
+    def live_blocks(self, group: int) -> list[int]:
+        return [b for b in self.tables[group] if b >= 0]
+
+
+@dataclass
+class _PendingEntry:
+    request: RequestCache
+    num_new: int
+    new_blocks: list[list[int]]
+    from_reserved: list[int]
+
+
+@dataclass
+class StepLayout:
+    """Host-side description of one step's tokens and where their cache lives."""
+
+    request_ids: tuple[str, ...]
+    q_starts: np.ndarray  # [R] tokens already cached
+    q_lens: np.ndarray  # [R] tokens of this step
+    context_lens: np.ndarray  # [R] q_start + q_len
+    cu_q: np.ndarray  # [R+1]
+    positions: np.ndarray  # [T]
+    token_entry: np.ndarray  # [T] entry index of each token
+    block_tables: list[np.ndarray]  # per group [R, max pages], -1 where no page
+    slot_mappings: list[np.ndarray]  # per group [T] page * block_size + offset
+    state_read: np.ndarray  # [R] row of the state banks to read
+    state_write: np.ndarray  # [R] row to write
+    slots: np.ndarray  # [R] request slot
+
+    @property
+    def num_tokens(self) -> int:
+        return int(self.cu_q[-1])
+
+    @property
+    def num_entries(self) -> int:
+        return len(self.request_ids)
+
+
+@dataclass(frozen=True)
+class CacheStats:
+    """Counts as in the reference's `PagedCacheStats`
+    (src/mini_llm_runtime/paged_kv_manager.py:34-50), per group."""
+
+    group: int
+    total_blocks: int
+    free_blocks: int
+    held_blocks: int
+    reserved_blocks: int
+    block_size: int
+    allocated_slots: int
+    committed_tokens: int
+    pending_tokens: int
+    internal_fragmentation_slots: int
+    utilization: float
+    storage_bytes: int
+
+
+class CacheManager:
+    def __init__(
+        self,
+        site_specs: Sequence[SiteSpec],
+        *,
+        block_size: int,
+        num_blocks: Union[int, Sequence[int]],
+        max_requests: int,
+        dtype: torch.dtype,
+        device: Union[str, torch.device] = "cuda",
+    ) -> None:
+        if block_size <= 0:
+            raise ValueError("block_size must be > 0")
+        if max_requests <= 0:
+            raise ValueError("max_requests must be > 0")
+        self.block_size = int(block_size)
+        self.max_requests = int(max_requests)
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.site_specs = tuple(site_specs)
+
+        grouped: dict[PagedKVSpec, list[int]] = {}
+        for site, spec in enumerate(self.site_specs):
+            if isinstance(spec, PagedKVSpec):
+                grouped.setdefault(spec, []).append(site)
+        counts = [num_blocks] * len(grouped) if isinstance(num_blocks, int) else list(num_blocks)
+        if len(counts) != len(grouped):
+            raise ValueError(f"num_blocks names {len(counts)} pools, the model has {len(grouped)} groups")
+        self.groups: list[KVGroup] = [
+            KVGroup(i, spec, sites, int(counts[i]), self.block_size, dtype, self.device)
+            for i, (spec, sites) in enumerate(grouped.items())
+        ]
+        self._site_group: dict[int, KVGroup] = {s: g for g in self.groups for s in g.sites}
+        self.state_banks: dict[int, StateBank] = {
+            site: StateBank(site, spec, self.max_requests, self.device)
+            for site, spec in enumerate(self.site_specs)
+            if isinstance(spec, SlotStateSpec)
+        }
+        self.slots = SlotPool(self.max_requests)
+        self._requests: dict[str, RequestCache] = {}
+        self._pending: Optional[list[_PendingEntry]] = None
+
+    # ---- lookups ----------------------------------------------------------------
+    @property
+    def request_ids(self) -> tuple[str, ...]:
+        return tuple(self._requests)
+
+    def has_request(self, request_id: str) -> bool:
+        return request_id in self._requests
+
+    def get_request(self, request_id: str) -> RequestCache:
+        try:
+            return self._requests[request_id]
+        except KeyError:
+            raise KeyError(f"unknown request {request_id!r}") from None
+
+    def group_of_site(self, site: int) -> KVGroup:
+        return self._site_group[site]
+
+    def site_pools(self, site: int) -> tuple[torch.Tensor, torch.Tensor, int]:
+        """(key pages, value pages, group index) of one site: [page, kv_head, offset, head_dim]."""
+        group = self._site_group[site]
+        i = group.site_position[site]
+        return group.key[i], group.value[i], group.index
+
+    @property
+    def step_in_flight(self) -> bool:
+        return self._pending is not None
+
+    # ---- request lifetime ---------------------------------------------------------
+    def create_request(self, request_id: str) -> RequestCache:
+        if not request_id:
+            raise ValueError("request_id must not be empty")
+        if request_id in self._requests:
+            raise ValueError(f"request {request_id!r} already exists")
+        slot = self.slots.take()
+        request = RequestCache(
+            request_id=request_id,
+            slot=slot,
+            tables=[[] for _ in self.groups],
+            reserved=[0 for _ in self.groups],
+        )
+        for bank in self.state_banks.values():
+            bank.tensor[2 * slot : 2 * slot + 2].zero_()
+        self._requests[request_id] = request
+        return request
+
+    def lifetime_blocks(self, max_tokens: int, max_step_tokens: int) -> list[int]:
+        return [g.lifetime_blocks(max_tokens, max_step_tokens) for g in self.groups]
+
+    def can_ever_hold(self, max_tokens: int, max_step_tokens: int) -> bool:
+        need = self.lifetime_blocks(max_tokens, max_step_tokens)
+        return all(n <= g.num_blocks for n, g in zip(need, self.groups))
+
+    def try_create_reserved(self, request_id: str, max_tokens: int, max_step_tokens: int) -> bool:
+        """Create a request and promise it the pages of its whole life, or do nothing.
+
+        Returns False (no side effect) when a pool or the slots are short right now;
+        raises ValueError when the request could never fit (as the reference's
+        admission does, src/mini_llm_runtime/block_admission.py:43-49).
+        """
+        need = self.lifetime_blocks(max_tokens, max_step_tokens)
+        for n, g in zip(need, self.groups):
+            if n > g.num_blocks:
+                raise ValueError(
+                    f"request {request_id!r} can never be admitted: needs {n} pages of group {g.index}, "
+                    f"the pool has {g.num_blocks}"
+                )
+        if self.slots.free_count == 0:
+            return False
+        if any(n > g.allocator.available_count for n, g in zip(need, self.groups)):
+            return False
+        request = self.create_request(request_id)
+        for i, (n, g) in enumerate(zip(need, self.groups)):
+            g.allocator.reserve(n)
+            request.reserved[i] = n
+        request.has_reservation = True
+        return True
+
+    def release_request(self, request_id: str) -> dict[int, tuple[int, ...]]:
+        """Give back every page, promise and the slot; the request is gone afterwards."""
+        request = self.get_request(request_id)
+        if self._pending is not None and any(e.request is request for e in self._pending):
+            raise RuntimeError(f"request {request_id!r} is part of the step in flight")
+        released: dict[int, tuple[int, ...]] = {}
+        for i, g in enumerate(self.groups):
+            ids = request.live_blocks(i)
+            g.allocator.free(ids)
+            g.allocator.unreserve(request.reserved[i])
+            released[i] = tuple(ids)
+        self.slots.give_back(request.slot)
+        del self._requests[request_id]
+        return released
+
+    # ---- one step = one transaction -------------------------------------------------
+    def begin_step(self, entries: Sequence[tuple[str, int]]) -> StepLayout:
+        """Take the pages the entries' new tokens need; all entries or none."""
+        if self._pending is not None:
+            raise RuntimeError("the previous step was neither committed nor aborted")
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen: set[str] = set()
+        for rid, n in entries:
+            if rid in seen:
+                raise ValueError(f"request {rid!r} appears twice in one step")
+            seen.add(rid)
+            if isinstance(n, bool) or not isinstance(n, (int, np.integer)) or n <= 0:
+                raise ValueError(f"request {rid!r}: a step entry needs at least one token")
+            self.get_request(rid)
+
+        pending: list[_PendingEntry] = []
+        try:
+            for rid, n in entries:
+                request = self._requests[rid]
+                entry = _PendingEntry(request, int(n), [[] for _ in self.groups], [0 for _ in self.groups])
+                pending.append(entry)
+                for i, g in enumerate(self.groups):
+                    have = len(request.tables[i])
+                    need = blocks_for(request.num_tokens + int(n), self.block_size) - have
+                    if need <= 0:
+                        continue
+                    promised = min(need, request.reserved[i])
+                    ids = g.allocator.allocate(need, from_reserved=promised)
+                    request.reserved[i] -= promised
+                    request.tables[i].extend(ids)
+                    entry.new_blocks[i] = ids
+                    entry.from_reserved[i] = promised
+        except BlockPoolExhaustedError:
+            self._rollback(pending)
+            raise
+        for entry in pending:
+            entry.request.pending_tokens = entry.num_new
+        self._pending = pending
+        return self._layout(pending)
+
+    def _rollback(self, pending: list[_PendingEntry]) -> None:
+        for entry in reversed(pending):
+            request = entry.request
+            for i, g in enumerate(self.groups):
+                ids = entry.new_blocks[i]
+                if not ids:
+                    continue
+                if request.tables[i][-len(ids) :] != ids:
+                    raise RuntimeError("pages of an aborted step are no longer the table's tail")
+                del request.tables[i][-len(ids) :]
+                g.allocator.free(ids, to_reserved=entry.from_reserved[i])
+                request.reserved[i] += entry.from_reserved[i]
+            request.pending_tokens = 0
+
+    def abort_step(self) -> None:
+        if self._pending is None:
+            raise RuntimeError("no step in flight")
+        pending, self._pending = self._pending, None
+        self._rollback(pending)
+
+    def commit_step(self) -> dict[str, dict[int, tuple[int, ...]]]:
+        """Make the step's tokens count; returns the window pages given back per request."""
+        if self._pending is None:
+            raise RuntimeError("no step in flight")
+        pending, self._pending = self._pending, None
+        passed: dict[str, dict[int, tuple[int, ...]]] = {}
+        for entry in pending:
+            request = entry.request
+            request.num_tokens += entry.num_new
+            request.pending_tokens = 0
+            request.state_parity ^= 1
+            for i, g in enumerate(self.groups):
+                dead = g.dead_blocks(request.num_tokens)
+                ids = [b for b in request.tables[i][:dead] if b >= 0]
+                if not ids:
+                    continue
+                keep = len(ids) if request.has_reservation else 0
+                g.allocator.free(ids, to_reserved=keep)
+                request.reserved[i] += keep
+                for j in range(dead):
+                    request.tables[i][j] = -1
+                passed.setdefault(request.request_id, {})[i] = tuple(ids)
+        return passed
+
+    def _layout(self, pending: list[_PendingEntry]) -> StepLayout:
+        bs = self.block_size
+        count = len(pending)
+        q_starts = np.array([e.request.num_tokens for e in pending], dtype=np.int32)
+        q_lens = np.array([e.num_new for e in pending], dtype=np.int32)
+        context = q_starts + q_lens
+        cu_q = np.zeros(count + 1, dtype=np.int32)
+        np.cumsum(q_lens, out=cu_q[1:])
+        total = int(cu_q[-1])
+        positions = np.empty(total, dtype=np.int32)
+        token_entry = np.empty(total, dtype=np.int32)
+        for r in range(count):
+            a, b = int(cu_q[r]), int(cu_q[r + 1])
+            positions[a:b] = np.arange(q_starts[r], context[r], dtype=np.int32)
+            token_entry[a:b] = r
+        block_tables: list[np.ndarray] = []
+        slot_mappings: list[np.ndarray] = []
+        for i, g in enumerate(self.groups):
+            width = max(1, max(blocks_for(int(c), bs) for c in context))
+            table = np.full((count, width), -1, dtype=np.int32)
+            slots = np.empty(total, dtype=np.int32)
+            for r, e in enumerate(pending):
+                row = e.request.tables[i]
+                used = blocks_for(int(context[r]), bs)
+                table[r, :used] = row[:used]
+                a, b = int(cu_q[r]), int(cu_q[r + 1])
+                pos = positions[a:b]
+                pages = table[r, pos // bs]
+                if (pages < 0).any():
+                    raise RuntimeError(f"request {e.request.request_id!r}: a new token has no page")
+                slots[a:b] = pages * bs + pos % bs
+            block_tables.append(table)
+            slot_mappings.append(slots)
+        slot_ids = np.array([e.request.slot for e in pending], dtype=np.int32)
+        parity = np.array([e.request.state_parity for e in pending], dtype=np.int32)
+        return StepLayout(
+            request_ids=tuple(e.request.request_id for e in pending),
+            q_starts=q_starts,
+            q_lens=q_lens,
+            context_lens=context.astype(np.int32),
+            cu_q=cu_q,
+            positions=positions,
+            token_entry=token_entry,
+            block_tables=block_tables,
+            slot_mappings=slot_mappings,
+            state_read=slot_ids * 2 + parity,
+            state_write=slot_ids * 2 + (1 - parity),
+            slots=slot_ids,
+        )
+
+    # ---- bookkeeping ------------------------------------------------------------------
+    def stats(self) -> tuple[CacheStats, ...]:
+        out = []
+        for i, g in enumerate(self.groups):
+            held = g.allocator.held_count
+            committed = 0
+            pending = 0
+            for request in self._requests.values():
+                live = len(request.live_blocks(i))
+                dead_tokens = (len(request.tables[i]) - live) * self.block_size
+                committed += max(0, request.num_tokens - dead_tokens)
+                pending += request.pending_tokens
+            allocated = held * self.block_size
+            out.append(
+                CacheStats(
+                    group=i,
+                    total_blocks=g.num_blocks,
+                    free_blocks=g.allocator.free_count,
+                    held_blocks=held,
+                    reserved_blocks=g.allocator.reserved_count,
+                    block_size=self.block_size,
+                    allocated_slots=allocated,
+                    committed_tokens=committed,
+                    pending_tokens=pending,
+                    internal_fragmentation_slots=allocated - committed - pending,
+                    utilization=(committed / allocated) if allocated else 0.0,
+                    storage_bytes=g.storage_bytes(),
+                )
+            )
+        return tuple(out)
+
+    def check_invariants(self) -> None:
+        """No page lost, held twice or held by nobody; promises add up.  For tests and debugging."""
+        for i, g in enumerate(self.groups):
+            owned: list[int] = []
+            promised = 0
+            for request in self._requests.values():
+                owned.extend(request.live_blocks(i))
+                promised += request.reserved[i]
+            if len(owned) != len(set(owned)):
+                raise AssertionError(f"group {i}: a page is held by two tables")
+            if sorted(owned) != g.allocator.held_ids():
+                raise AssertionError(f"group {i}: the tables and the allocator disagree on held pages")
+            if g.allocator.free_count + len(owned) != g.num_blocks:
+                raise AssertionError(f"group {i}: pages were lost")
+            if promised != g.allocator.reserved_count:
+                raise AssertionError(f"group {i}: promised pages do not add up")
+        slots = [r.slot for r in self._requests.values()]
+        if len(slots) != len(set(slots)) or self.slots.free_count + len(slots) != self.max_requests:
+            raise AssertionError("request slots are inconsistent")
+
+    def poison(self) -> None:
+        """Fill every page with NaN so that a read of an unwritten slot shows (tests)."""
+        for g in self.groups:
+            g.key.fill_(float("nan"))
+            g.value.fill_(float("nan"))

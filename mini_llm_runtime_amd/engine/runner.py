@@ -1,0 +1,192 @@
+"""The step function: one call runs one batch of (request, its next tokens) through
+the model, from the cache, and returns the logits at the wanted places.
+
+A batch may hold portions of prompts beside single decoded tokens, cut anywhere;
+both are the same case here: a span of new tokens behind a cached prefix.  The
+reference runs two separate forwards instead, whole prompts through
+`prefill_batch` and single tokens through `decode_batch`
+(src/mini_llm_runtime/qwen_model_runner.py:296-376, 447-508; engine.py:186-248),
+and has no partial prompts.  What is kept from it: the cache transaction around the
+forward (commit only after the head succeeded, abort on any exception,
+qwen_model_runner.py:371-375, 495-503), result rows in the order of the batch
+(engine.py:256-260) and the position bound (qwen_model_runner.py:319-320, 474-475).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, StepLayout
+from ..cache.spec import PagedKVSpec, SlotStateSpec
+from ..parts.context import KVView, StateView, StepContext
+from ..parts.model import DecoderModel
+
+
+@dataclass(frozen=True)
+class StepEntry:
+    """A request's next tokens and the places among them whose logits are wanted."""
+
+    request_id: str
+    tokens: tuple[int, ...]
+    want: tuple[int, ...] = ()
+
+    @staticmethod
+    def of(request_id: str, tokens: Sequence[int], want: Sequence[int] = ()) -> "StepEntry":
+        return StepEntry(request_id, tuple(int(t) for t in tokens), tuple(int(w) for w in want))
+
+
+@dataclass
+class StepOutput:
+    """logits: [K, vocab] float32 on the device (None when nothing was wanted), in the
+    order of the entries and of each entry's `want`; `rows[i]` = (request, index)."""
+
+    logits: Optional[torch.Tensor]
+    rows: tuple[tuple[str, int], ...]
+    layout: StepLayout
+    passed_pages: dict = field(default_factory=dict)
+
+
+def _pack_int32(arrays: Sequence[np.ndarray]) -> tuple[np.ndarray, list[tuple[int, tuple[int, ...]]]]:
+    """Concatenate int32 arrays into one buffer (each start 16-byte aligned)."""
+    spans = []
+    at = 0
+    for a in arrays:
+        spans.append((at, a.shape))
+        at += (a.size + 3) // 4 * 4
+    buf = np.zeros(max(at, 4), dtype=np.int32)
+    for (start, shape), a in zip(spans, arrays):
+        buf[start : start + a.size] = a.reshape(-1)
+    return buf, spans
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, cache: CacheManager, ops: Any) -> None:
+        if model.embed_weight is None:
+            raise ValueError("the model's parameters are not loaded")
+        self.model = model
+        self.cache = cache
+        self.ops = ops
+        self.device = cache.device
+        self.dtype = cache.dtype
+        self.vocab_size = model.spec.vocab_size
+        self.max_positions = model.spec.max_position_embeddings
+        self.fail_next_step: Optional[BaseException] = None  # test hook: raise inside the forward
+        specs = model.site_cache_specs()
+        if tuple(specs) != tuple(cache.site_specs):
+            raise ValueError("the cache manager was built for another model's sites")
+        self._pinned = torch.cuda.is_available() and self.device.type == "cuda"
+
+    # -------------------------------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        for e in entries:
+            if not e.tokens:
+                raise ValueError(f"request {e.request_id!r}: no tokens in this step")
+            for t in e.tokens:
+                if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < self.vocab_size:
+                    raise ValueError(
+                        f"request {e.request_id!r}: token {t!r} is outside the vocabulary of {self.vocab_size}"
+                    )
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+            cached = self.cache.get_request(e.request_id).num_tokens
+            if cached + len(e.tokens) > self.max_positions:
+                raise ValueError(
+                    f"request {e.request_id!r}: {cached + len(e.tokens)} tokens exceed "
+                    f"max_position_embeddings={self.max_positions}"
+                )
+
+    def _upload(self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray) -> StepContext:
+        groups = len(self.cache.groups)
+        arrays = [
+            token_ids,
+            layout.positions,
+            layout.token_entry,
+            layout.cu_q,
+            layout.q_starts,
+            layout.context_lens,
+            layout.state_read,
+            layout.state_write,
+            logit_rows,
+            *layout.slot_mappings,
+            *layout.block_tables,
+        ]
+        buf, spans = _pack_int32(arrays)
+        host = torch.from_numpy(buf)
+        if self._pinned:
+            host = host.pin_memory()
+        dev = host.to(self.device, non_blocking=True)
+
+        def view(i: int) -> torch.Tensor:
+            start, shape = spans[i]
+            n = int(np.prod(shape)) if shape else 1
+            return dev[start : start + n].view(shape)
+
+        ctx = StepContext(
+            ops=self.ops,
+            dtype=self.dtype,
+            device=self.device,
+            num_tokens=layout.num_tokens,
+            num_entries=layout.num_entries,
+            token_ids=view(0),
+            positions=view(1),
+            token_entry=view(2),
+            cu_q=view(3),
+            q_starts=view(4),
+            context_lens=view(5),
+            max_q_len=int(layout.q_lens.max()),
+            max_context_len=int(layout.context_lens.max()),
+            host=layout,
+        )
+        state_read, state_write = view(6), view(7)
+        ctx.memo["logit_rows"] = view(8)
+        slot_maps = [view(9 + g) for g in range(groups)]
+        tables = [view(9 + groups + g) for g in range(groups)]
+        for site in range(self.model.num_sites):
+            source = self.model.cache_site_of(site)
+            spec = self.cache.site_specs[source]
+            if isinstance(spec, PagedKVSpec):
+                key, value, g = self.cache.site_pools(source)
+                ctx.kv_views[site] = KVView(
+                    key=key,
+                    value=value,
+                    block_table=tables[g],
+                    slot_mapping=slot_maps[g],
+                    block_size=self.cache.block_size,
+                    window=spec.window,
+                    writable=source == site,
+                )
+            elif isinstance(spec, SlotStateSpec):
+                ctx.state_views[site] = StateView(self.cache.state_banks[source].tensor, state_read, state_write)
+        return ctx
+
+    # -------------------------------------------------------------------------------------------
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
+        self._validate(entries)
+        layout = self.cache.begin_step([(e.request_id, len(e.tokens)) for e in entries])
+        try:
+            token_ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=layout.num_tokens)
+            rows: list[tuple[str, int]] = []
+            flat: list[int] = []
+            for r, e in enumerate(entries):
+                for w in e.want:
+                    rows.append((e.request_id, w))
+                    flat.append(int(layout.cu_q[r]) + w)
+            logit_rows = np.asarray(flat, dtype=np.int32)
+            ctx = self._upload(layout, token_ids, logit_rows)
+            if self.fail_next_step is not None:
+                error, self.fail_next_step = self.fail_next_step, None
+                raise error
+            logits = self.model.forward(ctx, ctx.memo["logit_rows"] if flat else None)
+        except BaseException:
+            self.cache.abort_step()
+            raise
+        passed = self.cache.commit_step()
+        return StepOutput(logits=logits, rows=tuple(rows), layout=layout, passed_pages=passed)

@@ -1,0 +1,76 @@
+"""Interfaces of the parts a layer is put together from.
+
+A part is constructed from sizes and constants only, declares its parameters
+(`param_specs`) and, for mixers, what it needs of the cache (`cache_spec`).
+`bind` hands it the loaded tensors.  `forward` computes on token-major
+activations [T, width] for whatever batch the `StepContext` describes.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Mapping, Optional
+
+import torch
+
+from .context import StepContext
+from .spec import ParamSpec
+
+
+class Part:
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, params: Mapping[str, torch.Tensor], *, dtype: torch.dtype, device: torch.device) -> None:
+        """Receive the loaded parameters (keys of `param_specs`)."""
+        for name, tensor in params.items():
+            setattr(self, name, tensor)
+
+    def children(self) -> dict[str, "Part"]:
+        """Parts nested inside this one (their parameters live under `<name>.`)."""
+        return {}
+
+
+class Norm(Part):
+    def forward(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x: float32 residual stream [T, H].  When `delta` is given, first x += delta
+        (in place, summed in 32-bit); returns norm(x) in the engine's dtype."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotation(self, ctx: StepContext) -> Optional[tuple[torch.Tensor, torch.Tensor, int]]:
+        """(cos [T, r/2], sin [T, r/2], r) when the encoding is a half-split rotation of
+        the first r dims of every head that the fused kernel can apply; else None and
+        `apply` is called instead."""
+        return None
+
+    def apply(self, ctx: StepContext, q: torch.Tensor, k: torch.Tensor) -> None:
+        """Encode positions into q [T, Hq, d] and k [T, Hkv, d] in place."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Any:
+        """PagedKVSpec, SlotStateSpec or None."""
+        return None
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, site: int) -> torch.Tensor:
+        """h: normed activations [T, H] in the engine's dtype; returns [T, H]."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of a mixer, a feed-forward and norms around the residual stream."""
+
+    def forward(
+        self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor], site: int
+    ) -> Optional[torch.Tensor]:
+        """x: float32 residual stream, updated in place.  `delta` is the previous
+        layer's output that has not been added yet (None at the first layer); the
+        return value is this layer's own not-yet-added output."""
+        raise NotImplementedError

@@ -1,0 +1,62 @@
+"""What a part sees of a step: the tokens of the batch, where they sit in their
+requests, and handles to the cache of the execution site it runs at.  It is the
+same for every mixer kind; nothing in it names a model.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Optional
+
+import torch
+
+
+@dataclass
+class KVView:
+    """Pages of one site: [page, kv_head, offset, head_dim] keys and values, the
+    block table rows of the step's entries and the slot of each new token."""
+
+    key: torch.Tensor
+    value: torch.Tensor
+    block_table: torch.Tensor  # [R, max pages] int32, -1 where there is no page
+    slot_mapping: torch.Tensor  # [T] int32: page * block_size + offset
+    block_size: int
+    window: Optional[int]
+    writable: bool  # False when the site reads another site's cache
+
+
+@dataclass
+class StateView:
+    """Fixed-size state of one site: read rows `read_rows`, write rows `write_rows`
+    of `tensor` ([2 * slots, ...]); the manager swaps them at commit."""
+
+    tensor: torch.Tensor
+    read_rows: torch.Tensor  # [R] int32
+    write_rows: torch.Tensor  # [R] int32
+
+
+@dataclass
+class StepContext:
+    ops: Any
+    dtype: torch.dtype
+    device: torch.device
+    num_tokens: int
+    num_entries: int
+    token_ids: torch.Tensor  # [T] int32
+    positions: torch.Tensor  # [T] int32 absolute position of each token in its request
+    token_entry: torch.Tensor  # [T] int32 entry index of each token
+    cu_q: torch.Tensor  # [R+1] int32 first token of each entry
+    q_starts: torch.Tensor  # [R] int32 tokens cached before this step
+    context_lens: torch.Tensor  # [R] int32 tokens visible after this step's write
+    max_q_len: int
+    max_context_len: int
+    host: Any  # the StepLayout (numpy arrays) for parts that plan on the host
+    kv_views: dict[int, KVView] = field(default_factory=dict)
+    state_views: dict[int, StateView] = field(default_factory=dict)
+    memo: dict[Any, Any] = field(default_factory=dict)
+
+    def kv(self, site: int) -> KVView:
+        return self.kv_views[site]
+
+    def state(self, site: int) -> StateView:
+        return self.state_views[site]
