@@ -1,0 +1,77 @@
+// C interface of the gfx950 kernel library.  Every entry point takes device
+// pointers, sizes, element type codes (0: float32, 1: bfloat16) and the HIP
+// stream to launch on; it checks its arguments on the host, launches, and
+// returns 0, or -1 with a message for mlr_last_error().  Nothing here
+// allocates or synchronises.
+//
+// The reference has one native op, its decode attention
+// (csrc/paged_attention_binding.cpp:16-35); everything else below stands where
+// it calls PyTorch operators (src/mini_llm_runtime/qwen_model_runner.py).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+
+const char* mlr_last_error();
+int mlr_version();
+
+// out[t, :] = float(table[ids[t], :]); an id outside [0, vocab) gives a NaN row.
+int mlr_embedding(const void* table, int dtype, const int* ids, float* out, int tokens, int hidden,
+                  int vocab, hipStream_t stream);
+
+// x (float32 [rows, hidden]) += delta (dtype, may be null), then
+// out = weight * x * rsqrt(mean(x^2) + eps) in `dtype`; weight is float32 when
+// weight_is_f32, else `dtype`.
+int mlr_rmsnorm(float* x, const void* delta, const void* weight, int weight_is_f32, void* out,
+                int dtype, int rows, int hidden, float eps, hipStream_t stream);
+
+// x (float32) += delta (dtype), count elements.
+int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t stream);
+
+// out[k, :] = src[rows[k], :]; rows are `row_bytes` wide (a multiple of 4).
+int mlr_gather_rows(const void* src, const int* rows, void* out, int count, int64_t row_bytes,
+                    int src_rows, hipStream_t stream);
+
+// out[m, i] = silu(gate_up[m, i]) * gate_up[m, inter + i].
+int mlr_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter, hipStream_t stream);
+
+// cos/sin [tokens, half] float32 of positions[t] * inv_freq[j], computed in float64.
+int mlr_rope_table(const int* positions, const double* inv_freq, float* cos, float* sin, int tokens,
+                   int half, hipStream_t stream);
+
+// Rotate q and k of qkv [tokens, (heads + 2 kv_heads) * head_dim] in place (first
+// rotary_dim dims of every head, half-split pairs; rotary_dim 0: no rotation) and,
+// when `write`, store the rotated k and the raw v at slots[t] of the pages
+// [num_pages, kv_heads, block_size, head_dim]; a negative slot writes nothing.
+int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, const int* slots,
+                      void* key_pages, void* value_pages, int tokens, int heads, int kv_heads,
+                      int head_dim, int rotary_dim, int block_size, int num_pages, int write,
+                      hipStream_t stream);
+
+// y[M, N] = x[M, K] * w[N, K]^T (+ bias[N]); x, w in `dtype`; bias float32 when
+// bias_is_f32 else `dtype` (null: none); y float32 when out_is_f32 else `dtype`.
+// Plain 32-bit FMA arithmetic on every path (no matrix-core rounding).
+int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
+                    int out_is_f32, int dtype, int m, int n, int k, hipStream_t stream);
+
+// Attention of every token over its request's pages: token t (entry
+// token_entry[t], absolute position positions[t]) sees the keys
+// max(0, p - window + 1) .. p of its entry's block table row (window 0: all).
+// q is read from q[t * q_stride + head * head_dim + i]; out is [tokens, heads * head_dim].
+// A page id outside [0, num_pages) among the visible keys gives a NaN row.
+int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_pages,
+                               const void* value_pages, const int* block_table, int table_width,
+                               const int* token_entry, const int* positions, void* out, int dtype,
+                               int tokens, int entries, int heads, int kv_heads, int head_dim,
+                               int block_size, int num_pages, float scale, int window,
+                               hipStream_t stream);
+
+// tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
+// the first index whose cumulative exp((x - max) / temperature) exceeds
+// uniform[k] * total.  temperature and uniform may be null (all greedy).
+int mlr_sample(const float* logits, const float* temperature, const float* uniform, int* tokens,
+               int rows, int vocab, hipStream_t stream);
+
+}  // extern "C"

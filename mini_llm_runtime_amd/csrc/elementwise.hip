@@ -1,0 +1,308 @@
+// Row-wise and element-wise kernels: embedding gather, RMSNorm fused with the
+// residual addition, SiLU-multiply, rotary tables, and the fused rotary encoding
+// plus paged key/value store.  All arithmetic is float32; bfloat16 only exists
+// in memory.
+#include "api.h"
+#include "common.h"
+
+namespace mlr {
+
+static thread_local std::string g_error;
+void set_error(const std::string& message) { g_error = message; }
+
+// ---- embedding -------------------------------------------------------------------
+// qwen_model_runner.py:263 (F.embedding): a row gather, no scaling.
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ table,
+                                                        const int* __restrict__ ids,
+                                                        float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* dst = out + static_cast<int64_t>(t) * hidden;
+  if (id < 0 || id >= vocab) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __builtin_nanf("");
+    return;
+  }
+  const T* src = table + static_cast<int64_t>(id) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+// ---- RMSNorm (+ residual addition) ---------------------------------------------------
+// qwen_model_runner.py:22-26: weight * x * rsqrt(mean(x^2) + eps), statistics in float32.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                                      const TW* __restrict__ weight, T* __restrict__ out,
+                                                      int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * hidden;
+  float ss = 0.f;
+  if (delta != nullptr) {
+    const T* dr = delta + row * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = xr[i] + to_f32(dr[i]);
+      xr[i] = v;
+      ss += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = xr[i];
+      ss += v * v;
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+  T* orow = out + row * hidden;
+  // each thread re-reads the elements it wrote itself
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    orow[i] = from_f32<T>(to_f32(weight[i]) * (xr[i] * inv));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void add_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                                  int64_t count) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) x[i] += to_f32(delta[i]);
+}
+
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint32_t* __restrict__ src,
+                                                          const int* __restrict__ rows,
+                                                          uint32_t* __restrict__ out, int64_t row_words,
+                                                          int src_rows) {
+  const int k = blockIdx.x;
+  const int r = rows[k];
+  uint32_t* dst = out + static_cast<int64_t>(k) * row_words;
+  if (r < 0 || r >= src_rows) {
+    for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) dst[i] = 0xffffffffu;  // NaN in both types
+    return;
+  }
+  const uint32_t* s = src + static_cast<int64_t>(r) * row_words;
+  for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) dst[i] = s[i];
+}
+
+// qwen_model_runner.py:215-216: silu(gate) * up, silu(z) = z * sigmoid(z).
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out,
+                                                       int rows, int inter) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t total = static_cast<int64_t>(rows) * inter;
+  if (i >= total) return;
+  const int64_t m = i / inter;
+  const int64_t c = i - m * inter;
+  const float g = to_f32(gate_up[m * 2 * inter + c]);
+  const float u = to_f32(gate_up[m * 2 * inter + inter + c]);
+  const float s = g / (1.0f + expf(-g));
+  out[i] = from_f32<T>(s * u);
+}
+
+// ---- rotary tables -------------------------------------------------------------------
+// qwen_model_runner.py:45-57: angle = position * inv_freq[j]; here the product and
+// its cosine and sine are evaluated in float64 and rounded once to float32.
+__global__ __launch_bounds__(256) void rope_table_kernel(const int* __restrict__ positions,
+                                                         const double* __restrict__ inv_freq,
+                                                         float* __restrict__ cos_out,
+                                                         float* __restrict__ sin_out, int tokens, int half) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= static_cast<int64_t>(tokens) * half) return;
+  const int t = static_cast<int>(i / half);
+  const int j = static_cast<int>(i - static_cast<int64_t>(t) * half);
+  const double angle = static_cast<double>(positions[t]) * inv_freq[j];
+  cos_out[i] = static_cast<float>(cos(angle));
+  sin_out[i] = static_cast<float>(sin(angle));
+}
+
+// ---- rotary encoding + paged key/value store ------------------------------------------
+// qwen_model_runner.py:56-61 (x * cos + rotate_half(x) * sin: dims j and j + r/2 are
+// a pair) and :105-109 (the cache keeps the rotated k and the raw v); page layout
+// [page, kv_head, offset, head_dim] as paged_kv_cache.py:287-291.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+    T* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ slots, T* __restrict__ key_pages, T* __restrict__ value_pages, int heads,
+    int kv_heads, int head_dim, int rotary_dim, int block_size, int num_pages, int write) {
+  const int t = blockIdx.x;
+  const int half = rotary_dim / 2;
+  const int64_t width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  T* q = qkv + t * width;
+  T* k = q + static_cast<int64_t>(heads) * head_dim;
+  T* v = k + static_cast<int64_t>(kv_heads) * head_dim;
+  const float* cs = cos_t + static_cast<int64_t>(t) * half;
+  const float* sn = sin_t + static_cast<int64_t>(t) * half;
+
+  int64_t page_base = -1;  // element offset of (page, kv_head 0, offset, 0)
+  int64_t head_stride = static_cast<int64_t>(block_size) * head_dim;
+  if (write) {
+    const int slot = slots[t];
+    if (slot >= 0) {
+      const int page = slot / block_size;
+      const int off = slot - page * block_size;
+      if (page < num_pages)
+        page_base = (static_cast<int64_t>(page) * kv_heads * block_size + off) * head_dim;
+    }
+  }
+
+  for (int i = threadIdx.x; i < heads * half; i += blockDim.x) {
+    const int h = i / half;
+    const int j = i - h * half;
+    T* p = q + h * head_dim;
+    const float a = to_f32(p[j]);
+    const float b = to_f32(p[j + half]);
+    p[j] = from_f32<T>(a * cs[j] - b * sn[j]);
+    p[j + half] = from_f32<T>(b * cs[j] + a * sn[j]);
+  }
+  for (int i = threadIdx.x; i < kv_heads * half; i += blockDim.x) {
+    const int h = i / half;
+    const int j = i - h * half;
+    T* p = k + h * head_dim;
+    const float a = to_f32(p[j]);
+    const float b = to_f32(p[j + half]);
+    const T ra = from_f32<T>(a * cs[j] - b * sn[j]);
+    const T rb = from_f32<T>(b * cs[j] + a * sn[j]);
+    p[j] = ra;
+    p[j + half] = rb;
+    if (page_base >= 0) {
+      T* dst = key_pages + page_base + h * head_stride;
+      dst[j] = ra;
+      dst[j + half] = rb;
+    }
+  }
+  if (page_base >= 0) {
+    const int tail = head_dim - rotary_dim;
+    for (int i = threadIdx.x; i < kv_heads * tail; i += blockDim.x) {
+      const int h = i / tail;
+      const int j = rotary_dim + (i - h * tail);
+      key_pages[page_base + h * head_stride + j] = k[h * head_dim + j];
+    }
+    for (int i = threadIdx.x; i < kv_heads * head_dim; i += blockDim.x) {
+      const int h = i / head_dim;
+      const int j = i - h * head_dim;
+      value_pages[page_base + h * head_stride + j] = v[h * head_dim + j];
+    }
+  }
+}
+
+}  // namespace mlr
+
+using namespace mlr;
+
+extern "C" {
+
+const char* mlr_last_error() { return g_error.c_str(); }
+
+int mlr_version() { return 1; }
+
+int mlr_embedding(const void* table, int dtype, const int* ids, float* out, int tokens, int hidden,
+                  int vocab, hipStream_t stream) {
+  MLR_REQUIRE(table && ids && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && hidden > 0 && vocab > 0, "sizes must be > 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    embedding_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
+  else
+    embedding_kernel<bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, out, hidden, vocab);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_rmsnorm(float* x, const void* delta, const void* weight, int weight_is_f32, void* out, int dtype,
+                int rows, int hidden, float eps, hipStream_t stream) {
+  MLR_REQUIRE(x && weight && out, "null pointer");
+  MLR_REQUIRE(rows > 0 && hidden > 0, "sizes must be > 0");
+  MLR_REQUIRE(eps >= 0.f, "eps must be >= 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32) {
+    MLR_REQUIRE(weight_is_f32, "a float32 engine needs float32 norm weights");
+    rmsnorm_kernel<float, float><<<rows, 256, 0, stream>>>(x, static_cast<const float*>(delta),
+                                                          static_cast<const float*>(weight),
+                                                          static_cast<float*>(out), hidden, eps);
+  } else if (weight_is_f32) {
+    rmsnorm_kernel<bf16, float><<<rows, 256, 0, stream>>>(x, static_cast<const bf16*>(delta),
+                                                         static_cast<const float*>(weight),
+                                                         static_cast<bf16*>(out), hidden, eps);
+  } else {
+    rmsnorm_kernel<bf16, bf16><<<rows, 256, 0, stream>>>(x, static_cast<const bf16*>(delta),
+                                                        static_cast<const bf16*>(weight),
+                                                        static_cast<bf16*>(out), hidden, eps);
+  }
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t stream) {
+  MLR_REQUIRE(x && delta, "null pointer");
+  MLR_REQUIRE(count > 0, "count must be > 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  const int64_t blocks = (count + 255) / 256;
+  MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
+  if (dtype == kF32)
+    add_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, static_cast<const float*>(delta), count);
+  else
+    add_kernel<bf16><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, static_cast<const bf16*>(delta), count);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_gather_rows(const void* src, const int* rows, void* out, int count, int64_t row_bytes, int src_rows,
+                    hipStream_t stream) {
+  MLR_REQUIRE(src && rows && out, "null pointer");
+  MLR_REQUIRE(count > 0 && src_rows > 0, "sizes must be > 0");
+  MLR_REQUIRE(row_bytes > 0 && row_bytes % 4 == 0, "rows must be a multiple of 4 bytes wide");
+  gather_rows_kernel<<<count, 256, 0, stream>>>(static_cast<const uint32_t*>(src), rows,
+                                                static_cast<uint32_t*>(out), row_bytes / 4, src_rows);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter, hipStream_t stream) {
+  MLR_REQUIRE(gate_up && out, "null pointer");
+  MLR_REQUIRE(rows > 0 && inter > 0, "sizes must be > 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  const int64_t total = static_cast<int64_t>(rows) * inter;
+  const int64_t blocks = (total + 255) / 256;
+  MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
+  if (dtype == kF32)
+    silu_mul_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+        static_cast<const float*>(gate_up), static_cast<float*>(out), rows, inter);
+  else
+    silu_mul_kernel<bf16><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+        static_cast<const bf16*>(gate_up), static_cast<bf16*>(out), rows, inter);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_rope_table(const int* positions, const double* inv_freq, float* cos, float* sin, int tokens, int half,
+                   hipStream_t stream) {
+  MLR_REQUIRE(positions && inv_freq && cos && sin, "null pointer");
+  MLR_REQUIRE(tokens > 0 && half > 0, "sizes must be > 0");
+  const int64_t total = static_cast<int64_t>(tokens) * half;
+  const int64_t blocks = (total + 255) / 256;
+  MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
+  rope_table_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(positions, inv_freq, cos, sin, tokens, half);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, const int* slots,
+                      void* key_pages, void* value_pages, int tokens, int heads, int kv_heads, int head_dim,
+                      int rotary_dim, int block_size, int num_pages, int write, hipStream_t stream) {
+  MLR_REQUIRE(qkv, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && head_dim > 0, "sizes must be > 0");
+  MLR_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim,
+              "rotary_dim must be even and within head_dim");
+  MLR_REQUIRE(rotary_dim == 0 || (cos && sin), "rotation needs cos and sin tables");
+  MLR_REQUIRE(!write || (slots && key_pages && value_pages && block_size > 0 && num_pages > 0),
+              "a cache write needs slots, pages and their sizes");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    rope_kv_write_kernel<float><<<tokens, 256, 0, stream>>>(
+        static_cast<float*>(qkv), cos, sin, slots, static_cast<float*>(key_pages),
+        static_cast<float*>(value_pages), heads, kv_heads, head_dim, rotary_dim, block_size, num_pages, write);
+  else
+    rope_kv_write_kernel<bf16><<<tokens, 256, 0, stream>>>(
+        static_cast<bf16*>(qkv), cos, sin, slots, static_cast<bf16*>(key_pages),
+        static_cast<bf16*>(value_pages), heads, kv_heads, head_dim, rotary_dim, block_size, num_pages, write);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,322 @@
+"""The operations the parts compute with, bound to the HIP kernel library.
+
+`HipOps` is the only implementation the product has: it loads the libraries that
+`build.py` compiles for gfx950 and calls their extern "C" entry points through
+ctypes with device pointers and the current HIP stream.  There is no CPU path;
+constructing it without a GPU or without a working hipcc build raises.
+
+Every method checks device, element type, layout and sizes of its tensors on the
+host before a kernel is launched, so that a wrong call is an exception and never
+a memory fault on the GPU.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Any, Optional, Sequence, Union
+
+import torch
+
+from . import build
+
+_VP = ctypes.c_void_p
+_I = ctypes.c_int
+_I64 = ctypes.c_int64
+_F = ctypes.c_float
+
+_SIGNATURES = {
+    "mlr_version": ([], _I),
+    "mlr_embedding": ([_VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
+    "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
+    "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
+    "mlr_gather_rows": ([_VP, _VP, _VP, _I, _I64, _I, _VP], _I),
+    "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
+    "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
+    "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_paged_attention_simple": (
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
+        _I,
+    ),
+    "mlr_sample": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
+}
+
+
+class KernelError(RuntimeError):
+    """An entry point of the kernel library refused its arguments or failed to launch."""
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return 0
+    if dtype == torch.bfloat16:
+        return 1
+    raise KernelError(f"the kernels take float32 or bfloat16, not {dtype}")
+
+
+def load_library(module: build.Module = build.CORE) -> ctypes.CDLL:
+    path = build.ensure_module(module)
+    try:
+        lib = ctypes.CDLL(str(path))
+    except OSError as e:
+        raise KernelError(f"cannot load the HIP kernel library {path}: {e}") from None
+    lib.mlr_last_error.restype = ctypes.c_char_p
+    lib.mlr_last_error.argtypes = []
+    for name, (argtypes, restype) in _SIGNATURES.items():
+        if hasattr(lib, name):
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+    return lib
+
+
+class HipOps:
+    def __init__(self, dtype: torch.dtype = torch.bfloat16, device: Union[str, torch.device] = "cuda") -> None:
+        self.dtype = dtype
+        self.code = _dtype_code(dtype)
+        device = torch.device(device)
+        if device.type != "cuda":
+            raise KernelError(
+                f"the engine computes on an AMD GPU only (device {device} asked for); there is no CPU path"
+            )
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to this process; the engine has no CPU path")
+        if device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        self.device = device
+        self.lib = load_library(build.CORE)
+        if self.lib.mlr_version() != 1:
+            raise KernelError("the built kernel library is of another version than this package")
+
+    # ---- helpers --------------------------------------------------------------------------
+    def _stream(self) -> _VP:
+        return _VP(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _call(self, name: str, *args: Any) -> None:
+        status = getattr(self.lib, name)(*args)
+        if status != 0:
+            raise KernelError(self.lib.mlr_last_error().decode("utf-8", "replace"))
+
+    def _check(
+        self,
+        t: torch.Tensor,
+        name: str,
+        dtype: Optional[Union[torch.dtype, Sequence[torch.dtype]]] = None,
+        shape: Optional[Sequence[Optional[int]]] = None,
+    ) -> torch.Tensor:
+        if not isinstance(t, torch.Tensor):
+            raise KernelError(f"{name} must be a tensor")
+        if t.device != self.device:
+            raise KernelError(f"{name} is on {t.device}, the kernels run on {self.device}")
+        if not t.is_contiguous():
+            raise KernelError(f"{name} must be contiguous")
+        if dtype is not None:
+            allowed = (dtype,) if isinstance(dtype, torch.dtype) else tuple(dtype)
+            if t.dtype not in allowed:
+                raise KernelError(f"{name} has dtype {t.dtype}, expected {' or '.join(map(str, allowed))}")
+        if shape is not None:
+            if t.dim() != len(shape) or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+                raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    @staticmethod
+    def _ptr(t: Optional[torch.Tensor]) -> _VP:
+        return _VP(None if t is None else t.data_ptr())
+
+    def _empty(self, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        return torch.empty(tuple(shape), dtype=dtype, device=self.device)
+
+    # ---- residual stream --------------------------------------------------------------------
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        self._check(table, "embedding table", self.dtype, (None, None))
+        self._check(ids, "token ids", torch.int32, (None,))
+        vocab, hidden = table.shape
+        out = self._empty((ids.shape[0], hidden), torch.float32)
+        self._call(
+            "mlr_embedding", self._ptr(table), self.code, self._ptr(ids), self._ptr(out),
+            ids.shape[0], hidden, vocab, self._stream(),
+        )
+        return out
+
+    def rmsnorm(
+        self, x: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor] = None
+    ) -> torch.Tensor:
+        self._check(x, "residual stream", torch.float32, (None, None))
+        rows, hidden = x.shape
+        self._check(weight, "norm weight", (torch.float32, self.dtype), (hidden,))
+        if delta is not None:
+            self._check(delta, "residual delta", self.dtype, (rows, hidden))
+        out = self._empty((rows, hidden), self.dtype)
+        self._call(
+            "mlr_rmsnorm", self._ptr(x), self._ptr(delta), self._ptr(weight),
+            int(weight.dtype == torch.float32), self._ptr(out), self.code, rows, hidden, float(eps), self._stream(),
+        )
+        return out
+
+    def add_(self, x: torch.Tensor, delta: torch.Tensor) -> None:
+        self._check(x, "residual stream", torch.float32)
+        self._check(delta, "residual delta", self.dtype, tuple(x.shape))
+        self._call("mlr_add", self._ptr(x), self._ptr(delta), self.code, x.numel(), self._stream())
+
+    def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        self._check(x, "rows source", (torch.float32, torch.bfloat16), (None, None))
+        self._check(rows, "row indices", torch.int32, (None,))
+        row_bytes = x.shape[1] * x.element_size()
+        if row_bytes % 4:
+            raise KernelError("gather_rows needs rows that are a multiple of 4 bytes wide")
+        out = self._empty((rows.shape[0], x.shape[1]), x.dtype)
+        self._call(
+            "mlr_gather_rows", self._ptr(x), self._ptr(rows), self._ptr(out), rows.shape[0], row_bytes,
+            x.shape[0], self._stream(),
+        )
+        return out
+
+    # ---- matrix products ----------------------------------------------------------------------
+    def linear(
+        self,
+        x: torch.Tensor,
+        weight: torch.Tensor,
+        bias: Optional[torch.Tensor] = None,
+        out_dtype: Optional[torch.dtype] = None,
+    ) -> torch.Tensor:
+        """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics."""
+        self._check(x, "linear input", self.dtype, (None, None))
+        m, k = x.shape
+        self._check(weight, "linear weight", self.dtype, (None, k))
+        n = weight.shape[0]
+        if bias is not None:
+            self._check(bias, "linear bias", (torch.float32, self.dtype), (n,))
+        out_dtype = out_dtype or self.dtype
+        if out_dtype not in (torch.float32, self.dtype):
+            raise KernelError(f"linear output must be float32 or {self.dtype}")
+        y = self._empty((m, n), out_dtype)
+        self._call(
+            "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias),
+            int(bias is not None and bias.dtype == torch.float32), self._ptr(y),
+            int(out_dtype == torch.float32), self.code, m, n, k, self._stream(),
+        )
+        return y
+
+    def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
+        self._check(gate_up, "gate_up", self.dtype, (None, None))
+        rows, width = gate_up.shape
+        if width % 2:
+            raise KernelError("gate_up must have an even width")
+        out = self._empty((rows, width // 2), self.dtype)
+        self._call("mlr_silu_mul", self._ptr(gate_up), self._ptr(out), self.code, rows, width // 2, self._stream())
+        return out
+
+    # ---- positions and cache ---------------------------------------------------------------------
+    def rope_table(self, positions: torch.Tensor, inv_freq: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        self._check(positions, "positions", torch.int32, (None,))
+        self._check(inv_freq, "inverse frequencies", torch.float64, (None,))
+        tokens, half = positions.shape[0], inv_freq.shape[0]
+        cos = self._empty((tokens, half), torch.float32)
+        sin = self._empty((tokens, half), torch.float32)
+        self._call(
+            "mlr_rope_table", self._ptr(positions), self._ptr(inv_freq), self._ptr(cos), self._ptr(sin),
+            tokens, half, self._stream(),
+        )
+        return cos, sin
+
+    def _check_pages(self, key_pages, value_pages, num_kv_heads, head_dim, block_size) -> int:
+        self._check(key_pages, "key pages", self.dtype, (None, num_kv_heads, block_size, head_dim))
+        self._check(value_pages, "value pages", self.dtype, tuple(key_pages.shape))
+        return key_pages.shape[0]
+
+    def rope_kv_write(
+        self,
+        qkv: torch.Tensor,
+        rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+        slot_mapping: torch.Tensor,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        *,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        block_size: int,
+        write: bool = True,
+    ) -> None:
+        width = (num_heads + 2 * num_kv_heads) * head_dim
+        self._check(qkv, "qkv", self.dtype, (None, width))
+        tokens = qkv.shape[0]
+        cos = sin = None
+        rotary_dim = 0
+        if rotation is not None:
+            cos, sin, rotary_dim = rotation
+            if rotary_dim <= 0 or rotary_dim % 2 or rotary_dim > head_dim:
+                raise KernelError("rotary_dim must be even and within head_dim")
+            self._check(cos, "rotary cos", torch.float32, (tokens, rotary_dim // 2))
+            self._check(sin, "rotary sin", torch.float32, (tokens, rotary_dim // 2))
+        num_pages = 0
+        if write:
+            num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
+            self._check(slot_mapping, "slot mapping", torch.int32, (tokens,))
+        self._call(
+            "mlr_rope_kv_write", self._ptr(qkv), self.code, self._ptr(cos), self._ptr(sin),
+            self._ptr(slot_mapping if write else None), self._ptr(key_pages if write else None),
+            self._ptr(value_pages if write else None), tokens, num_heads, num_kv_heads, head_dim, rotary_dim,
+            block_size, num_pages, int(write), self._stream(),
+        )
+
+    def paged_attention(
+        self,
+        qkv: torch.Tensor,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        block_table: torch.Tensor,
+        ctx: Any,
+        *,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        block_size: int,
+        scale: float,
+        window: Optional[int],
+    ) -> torch.Tensor:
+        """Causal attention of the step's tokens over their requests' pages.
+
+        qkv: [T, >= num_heads * head_dim], queries in the leading columns (already
+        position-encoded); returns [T, num_heads * head_dim].
+        """
+        self._check(qkv, "queries", self.dtype, (None, None))
+        tokens, stride = qkv.shape
+        if stride < num_heads * head_dim:
+            raise KernelError("the query rows are narrower than num_heads * head_dim")
+        num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
+        self._check(block_table, "block table", torch.int32, (ctx.num_entries, None))
+        self._check(ctx.token_entry, "token entries", torch.int32, (tokens,))
+        self._check(ctx.positions, "positions", torch.int32, (tokens,))
+        if block_table.shape[1] * block_size < ctx.max_context_len:
+            raise KernelError("the block table is narrower than the longest context")
+        out = self._empty((tokens, num_heads * head_dim), self.dtype)
+        self._call(
+            "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
+            self._ptr(block_table), block_table.shape[1], self._ptr(ctx.token_entry), self._ptr(ctx.positions),
+            self._ptr(out), self.code, tokens, ctx.num_entries, num_heads, num_kv_heads, head_dim, block_size,
+            num_pages, float(scale), int(window or 0), self._stream(),
+        )
+        return out
+
+    # ---- sampling -----------------------------------------------------------------------------------
+    def sample(
+        self,
+        logits: torch.Tensor,
+        temperature: Optional[torch.Tensor] = None,
+        uniform: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        """int32 [K]: argmax, or an inverse-CDF draw where temperature > 0."""
+        self._check(logits, "logits", torch.float32, (None, None))
+        rows, vocab = logits.shape
+        if (temperature is None) != (uniform is None):
+            raise KernelError("temperature and uniform numbers come together")
+        if temperature is not None:
+            self._check(temperature, "temperature", torch.float32, (rows,))
+            self._check(uniform, "uniform numbers", torch.float32, (rows,))
+        out = self._empty((rows,), torch.int32)
+        self._call(
+            "mlr_sample", self._ptr(logits), self._ptr(temperature), self._ptr(uniform), self._ptr(out),
+            rows, vocab, self._stream(),
+        )
+        return out

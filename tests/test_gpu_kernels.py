@@ -1,0 +1,396 @@
+"""Each HIP kernel alone against a plain float64 torch computation of the same
+operation, at sizes other than the tiny models': widths and vocabularies that are
+no power of two, head sizes in steps of 16, MQA/GQA/MHA, fragmented block tables,
+NaN-filled pages (a read of an unwritten or foreign slot poisons the result).
+"""
+
+from __future__ import annotations
+
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+    # one rounding to bfloat16 is 2^-9 relative; float32 kernels differ from float64 by ~1e-6
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=1e-2, rtol=1.6e-2)
+
+
+@pytest.fixture(scope="module")
+def ops_for(gpu_device):
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    cache = {}
+
+    def get(dtype):
+        if dtype not in cache:
+            cache[dtype] = HipOps(dtype, gpu_device)
+        return cache[dtype]
+
+    return get
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+# ---- embedding, norm, elementwise -----------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(ops_for, dtype):
+    ops = ops_for(dtype)
+    table = _rand((517, 96), dtype, 1)
+    ids = torch.tensor([0, 516, 3, 3, 200], dtype=torch.int32)
+    out = ops.embedding(table.cuda(), ids.cuda()).cpu()
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table[ids.long()].float())
+    bad = ops.embedding(table.cuda(), torch.tensor([517, -1], dtype=torch.int32).cuda()).cpu()
+    assert torch.isnan(bad).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [64, 96, 896, 1000, 5120])
+@pytest.mark.parametrize("weight_f32", [False, True])
+def test_rmsnorm(ops_for, dtype, hidden, weight_f32):
+    ops = ops_for(dtype)
+    x = _rand((5, hidden), torch.float32, 2, 3.0)
+    delta = _rand((5, hidden), dtype, 3)
+    w = (1 + _rand((hidden,), torch.float32, 4, 0.1)).to(torch.float32 if weight_f32 or dtype == torch.float32 else dtype)
+    eps = 1e-5
+    ref = plain.rms_norm(x.double(), w.double(), eps)
+    got = ops.rmsnorm(x.cuda().clone(), w.cuda(), eps).cpu()
+    assert got.dtype == dtype
+    torch.testing.assert_close(got.double(), ref, **_tol(dtype))
+    xd = x.cuda().clone()
+    got = ops.rmsnorm(xd, w.cuda(), eps, delta=delta.cuda()).cpu()
+    summed = x.double() + delta.double()
+    torch.testing.assert_close(xd.cpu().double(), summed, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(got.double(), plain.rms_norm(summed, w.double(), eps), **_tol(dtype))
+
+
+def test_rmsnorm_vectors(ops_for):
+    """x=[3,4], w=[2,0.5], eps=0 and ones-stay-ones (reference tests/test_manual_qwen_decoder_layer.py:8-18)."""
+    ops = ops_for(torch.float32)
+    x = torch.tensor([[3.0, 4.0]]).cuda()
+    got = ops.rmsnorm(x, torch.tensor([2.0, 0.5]).cuda(), 0.0).cpu()
+    rms = math.sqrt(12.5)
+    torch.testing.assert_close(got, torch.tensor([[2 * 3 / rms, 0.5 * 4 / rms]]))
+    ones = ops.rmsnorm(torch.ones(1, 8).cuda(), torch.ones(8).cuda(), 0.0).cpu()
+    torch.testing.assert_close(ones, torch.ones(1, 8))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_gather_silu(ops_for, dtype):
+    ops = ops_for(dtype)
+    x = _rand((7, 100), torch.float32, 5)
+    d = _rand((7, 100), dtype, 6)
+    xd = x.cuda().clone()
+    ops.add_(xd, d.cuda())
+    torch.testing.assert_close(xd.cpu(), x + d.float())
+    rows = torch.tensor([6, 0, 3, 3], dtype=torch.int32)
+    assert torch.equal(ops.gather_rows(x.cuda(), rows.cuda()).cpu(), x[rows.long()])
+    assert torch.equal(ops.gather_rows(d.cuda(), rows.cuda()).cpu(), d[rows.long()])
+    gu = _rand((9, 2 * 352), dtype, 7, 2.0)
+    g, u = gu[:, :352].double(), gu[:, 352:].double()
+    ref = g * torch.sigmoid(g) * u
+    torch.testing.assert_close(ops.silu_mul(gu.cuda()).cpu().double(), ref, **_tol(dtype))
+    # identity-weight SwiGLU vector: silu(x) * 2x (reference tests/test_manual_qwen_decoder_layer.py:21-36)
+    xv = torch.tensor([[-1.0, 0.5, 2.0]])
+    both = torch.cat([xv, 2 * xv], dim=1).to(dtype)
+    ref = torch.nn.functional.silu(both[:, :3].double()) * both[:, 3:].double()
+    torch.testing.assert_close(ops.silu_mul(both.cuda()).cpu().double(), ref, **_tol(dtype))
+
+
+# ---- matrix product -----------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 17, 8), (5, 64, 96), (63, 352, 129), (65, 517, 96), (200, 130, 1000), (2, 1152, 896)])
+def test_linear(ops_for, dtype, m, n, k):
+    ops = ops_for(dtype)
+    x = _rand((m, k), dtype, 8)
+    w = _rand((n, k), dtype, 9, 0.1)
+    for bias_dtype in (None, dtype, torch.float32):
+        b = None if bias_dtype is None else _rand((n,), bias_dtype, 10)
+        ref = x.double() @ w.double().t() + (0 if b is None else b.double())
+        for out_dtype in {dtype, torch.float32}:
+            got = ops.linear(x.cuda(), w.cuda(), None if b is None else b.cuda(), out_dtype=out_dtype).cpu()
+            assert got.dtype == out_dtype and got.shape == (m, n)
+            tol = _tol(out_dtype if dtype == torch.bfloat16 else dtype)
+            if dtype == torch.float32:
+                tol = dict(atol=1e-4, rtol=1e-5)  # k-long float32 sums against float64
+            torch.testing.assert_close(got.double(), ref, **tol)
+
+
+# ---- rotary encoding and cache write ----------------------------------------------------------------
+def test_rope_table(ops_for):
+    ops = ops_for(torch.float32)
+    pos = torch.tensor([0, 1, 2, 17, 4095, 32767, 131071], dtype=torch.int32)
+    inv = 1.0 / (1e6 ** (torch.arange(0, 64, 2, dtype=torch.float64) / 64))
+    cos, sin = ops.rope_table(pos.cuda(), inv.cuda())
+    ang = pos.double()[:, None] * inv[None]
+    torch.testing.assert_close(cos.cpu().double(), ang.cos(), atol=1e-7, rtol=0)
+    torch.testing.assert_close(sin.cpu().double(), ang.sin(), atol=1e-7, rtol=0)
+    assert torch.equal(cos[0].cpu(), torch.ones(32)) and torch.equal(sin[0].cpu(), torch.zeros(32))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary", [(4, 2, 16, 16), (3, 1, 32, 32), (14, 2, 64, 64), (8, 8, 128, 64), (2, 1, 48, 48)])
+def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
+    ops = ops_for(dtype)
+    tokens, bs, pages = 11, 8, 9
+    width = (heads + 2 * kv_heads) * head_dim
+    qkv = _rand((tokens, width), dtype, 11)
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 7, 8, 9, 100, 5], dtype=torch.int32)
+    theta = 10000.0
+    inv = 1.0 / (theta ** (torch.arange(0, rotary, 2, dtype=torch.float64) / rotary))
+    cos, sin = ops.rope_table(positions.cuda(), inv.cuda())
+    g = torch.Generator().manual_seed(12)
+    slots = torch.randperm(pages * bs, generator=g)[:tokens].to(torch.int32)
+    slots[4] = -1  # writes nothing
+    kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=dtype).cuda()
+    vp = kp.clone()
+    dev = qkv.cuda().clone()
+    ops.rope_kv_write(dev, (cos, sin, rotary), slots.cuda(), kp, vp, num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs)
+    out = dev.cpu()
+
+    def rot(x):  # [T, H, d] float64 -> rotated first `rotary` dims
+        y = x.clone()
+        part = x[..., :rotary].transpose(0, 1)  # [H, T, r]
+        y[..., :rotary] = plain.apply_rope(part, positions, theta).transpose(0, 1)
+        return y
+
+    q_ref = rot(qkv[:, : heads * head_dim].double().view(tokens, heads, head_dim))
+    k_ref = rot(qkv[:, heads * head_dim : (heads + kv_heads) * head_dim].double().view(tokens, kv_heads, head_dim))
+    v_ref = qkv[:, (heads + kv_heads) * head_dim :].double().view(tokens, kv_heads, head_dim)
+    tol = _tol(dtype)
+    torch.testing.assert_close(out[:, : heads * head_dim].double().view(tokens, heads, head_dim), q_ref, **tol)
+    kc, vc = kp.cpu().double(), vp.cpu().double()
+    written = torch.zeros(pages, bs, dtype=torch.bool)
+    for t in range(tokens):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        page, off = divmod(s, bs)
+        written[page, off] = True
+        torch.testing.assert_close(kc[page, :, off], k_ref[t], **tol)
+        torch.testing.assert_close(vc[page, :, off], v_ref[t], atol=0, rtol=0)
+    untouched = ~written[:, None, :, None].expand_as(kc)
+    assert torch.isnan(kc[untouched]).all() and torch.isnan(vc[untouched]).all()
+    # position 0 is the identity (reference tests/test_manual_qwen_attention.py:35-42)
+    assert torch.equal(out[0, : heads * head_dim], qkv[0, : heads * head_dim])
+
+
+# ---- attention ----------------------------------------------------------------------------------------
+def _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, seed, extra_pages=3, spike=False):
+    """entries: list of (context_len, q_len).  Returns device inputs and the float64 expectation."""
+    g = torch.Generator().manual_seed(seed)
+    need = [-(-c // bs) for c, _ in entries]
+    pages = sum(need) + extra_pages
+    perm = torch.randperm(pages, generator=g).tolist()
+    width = max(need)
+    table = torch.full((len(entries), width), -1, dtype=torch.int32)
+    kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=dtype)
+    vp = kp.clone()
+    dense = []
+    for r, (ctx_len, _) in enumerate(entries):
+        ids = [perm.pop() for _ in range(need[r])]
+        table[r, : need[r]] = torch.tensor(ids, dtype=torch.int32)
+        k = torch.randn(ctx_len, kv_heads, head_dim, generator=g).to(dtype)
+        v = torch.randn(ctx_len, kv_heads, head_dim, generator=g).to(dtype)
+        if spike and ctx_len > 3:
+            k[1] *= 6.0  # a far key that must dominate when the query points at it
+        for p in range(ctx_len):
+            kp[ids[p // bs], :, p % bs] = k[p]
+            vp[ids[p // bs], :, p % bs] = v[p]
+        dense.append((k.double(), v.double()))
+    token_entry, positions = [], []
+    for r, (ctx_len, q_len) in enumerate(entries):
+        for i in range(q_len):
+            token_entry.append(r)
+            positions.append(ctx_len - q_len + i)
+    tokens = len(positions)
+    q = torch.randn(tokens, heads * head_dim + 24, generator=g).to(dtype)  # wider rows: a strided q
+    if spike:
+        for t, r in enumerate(token_entry):
+            if entries[r][0] > 3:
+                k1 = dense[r][0][1]  # [kv_heads, d]
+                rep = k1.repeat_interleave(heads // kv_heads, dim=0).reshape(-1)
+                q[t, : heads * head_dim] = (rep * 0.5).to(dtype)
+    ctx = SimpleNamespace(
+        num_entries=len(entries),
+        token_entry=torch.tensor(token_entry, dtype=torch.int32).cuda(),
+        positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+        max_context_len=max(c for c, _ in entries),
+        max_q_len=max(ql for _, ql in entries),
+    )
+    return q, kp, vp, table, ctx, dense, token_entry, positions
+
+
+def _attention_reference(q, dense, token_entry, positions, heads, kv_heads, head_dim, scale, window):
+    group = heads // kv_heads
+    out = torch.zeros(len(positions), heads, head_dim, dtype=torch.float64)
+    for t, (r, p) in enumerate(zip(token_entry, positions)):
+        k, v = dense[r]
+        first = 0 if not window else max(0, p - window + 1)
+        kk = k[first : p + 1].repeat_interleave(group, dim=1)  # [n, H, d]
+        vv = v[first : p + 1].repeat_interleave(group, dim=1)
+        qq = q[t, : heads * head_dim].double().view(heads, head_dim)
+        s = torch.einsum("hd,nhd->hn", qq, kk) * scale
+        out[t] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+    return out.reshape(len(positions), heads * head_dim)
+
+
+ATTN_SHAPES = [(14, 2, 64), (4, 1, 32), (3, 3, 16), (8, 2, 128), (6, 2, 48), (5, 1, 80)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim", ATTN_SHAPES)
+@pytest.mark.parametrize("bs", [8, 16])
+def test_paged_attention_mixed_batch(ops_for, dtype, heads, kv_heads, head_dim, bs):
+    ops = ops_for(dtype)
+    # (context, new tokens): decode tokens, whole prompts, portions behind a cached prefix, page edges
+    entries = [(1, 1), (bs, 1), (bs + 1, 1), (37, 37), (70, 5), (4 * bs + 1, 2), (130, 1), (2 * bs, bs)]
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 21)
+    scale = head_dim**-0.5
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
+    ).cpu()
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
+    assert torch.isfinite(got).all(), "a NaN page slot was read"
+    torch.testing.assert_close(got.double(), ref, **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 16, 50])
+def test_paged_attention_window(ops_for, dtype, window):
+    ops = ops_for(dtype)
+    heads, kv_heads, head_dim, bs = 4, 2, 32, 8
+    entries = [(1, 1), (16, 16), (60, 3), (75, 1)]
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 22)
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=0.2, window=window,
+    ).cpu()
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, 0.2, window)
+    torch.testing.assert_close(got.double(), ref, **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_far_key_among_hundreds(ops_for, dtype):
+    """Queries aligned with key 1 of a long context: that key's value must dominate."""
+    ops = ops_for(dtype)
+    heads, kv_heads, head_dim, bs = 4, 2, 64, 16
+    entries = [(700, 1), (515, 3), (2049, 1)]
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 23, spike=True)
+    scale = head_dim**-0.5
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
+    ).cpu()
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
+    torch.testing.assert_close(got.double(), ref, **_tol(dtype))
+    v1 = dense[0][1][1].repeat_interleave(heads // kv_heads, dim=0).reshape(-1)
+    assert (got[0].double() - v1).abs().max() < 0.2, "the far key did not dominate"
+
+
+def test_paged_attention_merge_needs_global_weights(ops_for):
+    """Two keys with scores +-large and values 7 and -3: the answer is 7, not the mean 2
+    (reference tests/test_split_kv_attention.py:62-73)."""
+    ops = ops_for(torch.float32)
+    bs = 4
+    kp = torch.zeros(2, 1, bs, 16)
+    vp = torch.zeros(2, 1, bs, 16)
+    kp[0, 0, 0, 0] = 40.0
+    kp[1, 0, 0, 0] = -40.0
+    vp[0, 0, 0] = 7.0
+    vp[1, 0, 0] = -3.0
+    # context of 5 tokens: positions 0..3 in page 0 (1..3 neutral), position 4 in page 1
+    q = torch.zeros(1, 16)
+    q[0, 0] = 1.0
+    ctx = SimpleNamespace(
+        num_entries=1,
+        token_entry=torch.zeros(1, dtype=torch.int32).cuda(),
+        positions=torch.tensor([4], dtype=torch.int32).cuda(),
+        max_context_len=5,
+        max_q_len=1,
+    )
+    table = torch.tensor([[0, 1]], dtype=torch.int32)
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=1, num_kv_heads=1, head_dim=16, block_size=bs, scale=1.0, window=None,
+    ).cpu()
+    torch.testing.assert_close(got, torch.full((1, 16), 7.0), atol=1e-5, rtol=0)
+
+
+def test_paged_attention_bad_page_poisons(ops_for):
+    """A used table entry of -1 must never be read as a page (reference tests/test_paged_attention.py:158-171)."""
+    ops = ops_for(torch.float32)
+    entries = [(20, 1)]
+    q, kp, vp, table, ctx, *_ = _paged_case(entries, 2, 1, 16, 8, torch.float32, 24)
+    table[0, 1] = -1
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=2, num_kv_heads=1, head_dim=16, block_size=8, scale=0.25, window=None,
+    ).cpu()
+    assert torch.isnan(got).all()
+
+
+def test_attention_matches_library_special_case(ops_for):
+    """No rotation, whole prompt, MHA: equals torch's scaled_dot_product_attention(is_causal=True)."""
+    ops = ops_for(torch.float32)
+    heads, head_dim, bs, n = 3, 32, 8, 29
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case([(n, n)], heads, heads, head_dim, bs, torch.float32, 25)
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=heads, head_dim=head_dim, block_size=bs, scale=head_dim**-0.5, window=None,
+    ).cpu()
+    k, v = dense[0]
+    qq = q[:, : heads * head_dim].double().view(n, heads, head_dim).transpose(0, 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(qq, k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+    torch.testing.assert_close(got.double(), ref.transpose(0, 1).reshape(n, -1), atol=2e-5, rtol=2e-5)
+
+
+# ---- sampling ---------------------------------------------------------------------------------------------
+def test_sample_greedy_first_maximum(ops_for):
+    ops = ops_for(torch.float32)
+    logits = _rand((6, 1000), torch.float32, 30)
+    logits[0, 17] = logits[0, 900] = 50.0  # tie: the first wins
+    logits[1, 999] = 60.0
+    logits[2, 0] = 60.0
+    got = ops.sample(logits.cuda()).cpu()
+    assert got.dtype == torch.int32
+    assert got.tolist() == torch.argmax(logits, dim=-1).tolist()
+    assert got[0] == 17
+    big = _rand((3, 151936), torch.float32, 31)
+    assert ops.sample(big.cuda()).cpu().tolist() == torch.argmax(big, -1).tolist()
+
+
+def test_sample_temperature_inverse_cdf(ops_for):
+    ops = ops_for(torch.float32)
+    rows, vocab = 64, 517
+    logits = _rand((rows, vocab), torch.float32, 32, 3.0)
+    g = torch.Generator().manual_seed(33)
+    u = torch.rand(rows, generator=g)
+    u[0], u[1] = 0.0, 0.99999994
+    temp = torch.full((rows,), 0.8)
+    temp[2] = 0.0  # greedy row inside a sampled batch
+    got = ops.sample(logits.cuda(), temp.cuda(), u.cuda()).cpu().long()
+    assert got[2] == torch.argmax(logits[2])
+    for i in range(rows):
+        if temp[i] == 0:
+            continue
+        cdf = torch.cumsum(plain.temperature_probabilities(logits[i], float(temp[i])), 0)
+        lo = 0.0 if got[i] == 0 else float(cdf[got[i] - 1])
+        hi = float(cdf[got[i]])
+        assert lo - 1e-5 <= float(u[i]) <= hi + 1e-5, (i, lo, float(u[i]), hi)
+    # the same uniform number gives the same token whatever else is in the batch
+    alone = ops.sample(logits[5:6].cuda(), temp[5:6].cuda(), u[5:6].cuda()).cpu()
+    assert int(alone[0]) == int(got[5])

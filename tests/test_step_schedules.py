@@ -1,0 +1,146 @@
+"""The step function against the plain implementation under every way of cutting
+and batching: whole, bulk + one by one, changing portions, and mixed with pages
+that are used again.  Runs with the torch stand-in for the kernels on the CPU and
+with the HIP kernels on the GPU (`-m gpu`), in 32-bit and in bfloat16.
+"""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+import mini_llm_runtime_amd.models  # noqa: F401
+import plain_qwen2 as plain
+import schedules
+from helpers import BLOCK_SIZE, TINY, make_model_dir, make_runner, random_tokens, read_weights
+from kernel_doubles import TorchOps
+
+LENGTHS = {"A": (5, 17, 33, 70, 41, 52), "B": (1, 9, 24, 40, 63, 37)}
+
+# float32: the engine and the plain implementation (float64) differ by float32
+# rounding only.  bfloat16: activations between kernels are rounded to 8 bits of
+# mantissa (2^-9 relative per rounding); the error is judged relative to the size
+# of the logits.
+FP32_MAX_ABS = 1e-4
+BF16_REL_L2 = 2e-2
+
+
+def _ops(backend: str, dtype: torch.dtype):
+    if backend == "double":
+        return TorchOps(dtype, "cpu")
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    return HipOps(dtype, "cuda")
+
+
+def _sharpen(tensors: dict[str, torch.Tensor], factor: float) -> dict[str, torch.Tensor]:
+    """Scale the query and key projections so that attention is peaked: with small
+    random weights every key gets nearly the same weight, which would hide a key
+    that is read from the wrong place."""
+    out = {}
+    for name, t in tensors.items():
+        if ".q_proj." in name or ".k_proj." in name:
+            t = (t.float() * factor).to(t.dtype)
+        out[name] = t
+    return out
+
+
+def _setup(tmp_path, which: str, backend: str, dtype: torch.dtype, steps, sharp: float = 0.0):
+    from mini_llm_runtime_amd.weights import save_state_dict
+
+    model_dir = make_model_dir(tmp_path, which, seed=11)
+    cfg, weights = read_weights(model_dir)
+    if sharp:
+        weights = _sharpen(weights, sharp)
+        save_state_dict(model_dir / "model.safetensors", weights)
+    bs = BLOCK_SIZE[which]
+    ops = _ops(backend, dtype)
+    _, _, cache, runner = make_runner(
+        model_dir, ops, block_size=bs, num_blocks=schedules.pages_needed(steps, bs), max_requests=4
+    )
+    cache.poison()
+    return cfg, weights, cache, runner
+
+
+def _requests(which: str) -> dict[str, list[int]]:
+    vocab = TINY[which]["vocab_size"]
+    return {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[which])}
+
+
+def _compare(got, requests, weights, cfg, dtype):
+    assert got, "no logits came back"
+    worst_abs = 0.0
+    num = 0.0
+    den = 0.0
+    for rid, toks in requests.items():
+        ref = plain.forward(toks, weights, cfg)
+        for pos in range(len(toks)):
+            row = got[(rid, pos)].double()
+            assert torch.isfinite(row).all(), f"{rid}:{pos} is not finite"
+            diff = row - ref[pos]
+            worst_abs = max(worst_abs, float(diff.abs().max()))
+            num += float((diff**2).sum())
+            den += float((ref[pos] ** 2).sum())
+    rel = (num / den) ** 0.5
+    if dtype == torch.float32:
+        assert worst_abs < FP32_MAX_ABS, f"max abs error {worst_abs:.3e}, rel L2 {rel:.3e}"
+    else:
+        assert rel < BF16_REL_L2, f"rel L2 error {rel:.3e}, max abs {worst_abs:.3e}"
+
+
+FAMILIES = {
+    "whole": schedules.whole,
+    "bulk_then_tail": schedules.bulk_then_tail,
+    "portions": schedules.portions,
+    "mixed": schedules.mixed,
+}
+
+CASES = [
+    pytest.param("double", torch.float32, id="double-f32"),
+    pytest.param("hip", torch.float32, id="hip-f32", marks=pytest.mark.gpu),
+    pytest.param("hip", torch.bfloat16, id="hip-bf16", marks=pytest.mark.gpu),
+]
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("family", list(FAMILIES))
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_schedule_matches_plain(tmp_path, which, family, backend, dtype):
+    requests = _requests(which)
+    steps = FAMILIES[family](requests)
+    if family == "mixed":
+        assert schedules.most_live(steps) == 4
+        total = sum(schedules.blocks_for(len(t), BLOCK_SIZE[which]) for t in requests.values())
+        assert schedules.pages_needed(steps, BLOCK_SIZE[which]) < total, "pages would not be used again"
+    cfg, weights, cache, runner = _setup(tmp_path, which, backend, dtype, steps)
+    got = schedules.run_schedule(runner, cache, steps)
+    _compare(got, requests, weights, cfg, dtype)
+    cache.check_invariants()
+    assert cache.request_ids == ()
+    assert all(g.allocator.free_count == g.num_blocks for g in cache.groups)
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_peaked_attention_mixed(tmp_path, which, backend, dtype):
+    """Same as the mixed family, with query/key projections scaled up so that single
+    keys dominate: a key read from a wrong slot or page changes the logits visibly."""
+    requests = _requests(which)
+    steps = schedules.mixed(requests, seed=5)
+    cfg, weights, cache, runner = _setup(tmp_path, which, backend, dtype, steps, sharp=12.0)
+    got = schedules.run_schedule(runner, cache, steps)
+    _compare(got, requests, weights, cfg, dtype)
+
+
+@pytest.mark.parametrize("backend,dtype", CASES[:2])
+def test_schedules_agree_with_each_other(tmp_path, backend, dtype):
+    """In 32-bit the families agree with each other far below the plain-implementation bound."""
+    requests = _requests("B")
+    results = []
+    for family in FAMILIES.values():
+        steps = family(requests)
+        _, _, cache, runner = _setup(tmp_path, "B", backend, dtype, steps)
+        results.append(schedules.run_schedule(runner, cache, steps))
+    for other in results[1:]:
+        for key, row in results[0].items():
+            assert torch.allclose(row, other[key], atol=2e-5, rtol=0), key
