@@ -62,6 +62,11 @@ CORE = Module(
 )
 
 
+def all_modules() -> list[Module]:
+    """Every module a default build compiles."""
+    return [CORE]
+
+
 def log(message: str) -> None:
     print(f"[mini_llm_runtime_amd] {message}", file=sys.stderr, flush=True)
 
