@@ -14,8 +14,11 @@ Beyond the reference: several groups (each with pages and a free list of its
 own), windows (pages that every later query has passed are given back at
 commit), capacity promised by count instead of by pinning pages, and state slots.
 
-Page layout of every pool: [site, page, kv_head, offset in page, head_dim], the
-reference's inner order (src/mini_llm_runtime/paged_kv_cache.py:287-318).
+Page layout: keys [site, page, kv_head, offset in page, head_dim], the reference's
+inner order (src/mini_llm_runtime/paged_kv_cache.py:287-318); values are kept
+transposed inside a page, [site, page, kv_head, head_dim, offset in page], because
+the matrix cores want the index that is summed over (the key position, for the
+probability-times-value product) to be the fastest one of both operands.
 """
 
 from __future__ import annotations
@@ -60,7 +63,9 @@ class KVGroup:
         shape = (len(self.sites), num_blocks, spec.num_kv_heads, block_size, spec.head_dim)
         # never zeroed: stale bytes must be unreachable, not clean
         self.key = torch.empty(shape, dtype=dtype, device=device)
-        self.value = torch.empty(shape, dtype=dtype, device=device)
+        self.value = torch.empty(
+            (len(self.sites), num_blocks, spec.num_kv_heads, spec.head_dim, block_size), dtype=dtype, device=device
+        )
 
     @property
     def num_blocks(self) -> int:
@@ -225,7 +230,8 @@ class CacheManager:
         return self._site_group[site]
 
     def site_pools(self, site: int) -> tuple[torch.Tensor, torch.Tensor, int]:
-        """(key pages, value pages, group index) of one site: [page, kv_head, offset, head_dim]."""
+        """(key pages [page, kv_head, offset, head_dim], value pages [page, kv_head, head_dim, offset],
+        group index) of one site."""
         group = self._site_group[site]
         i = group.site_position[site]
         return group.key[i], group.value[i], group.index

@@ -43,8 +43,9 @@ int mlr_rope_table(const int* positions, const double* inv_freq, float* cos, flo
 
 // Rotate q and k of qkv [tokens, (heads + 2 kv_heads) * head_dim] in place (first
 // rotary_dim dims of every head, half-split pairs; rotary_dim 0: no rotation) and,
-// when `write`, store the rotated k and the raw v at slots[t] of the pages
-// [num_pages, kv_heads, block_size, head_dim]; a negative slot writes nothing.
+// when `write`, store the rotated k and the raw v at slots[t] of the key pages
+// [num_pages, kv_heads, block_size, head_dim] and the value pages
+// [num_pages, kv_heads, head_dim, block_size]; a negative slot writes nothing.
 int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, const int* slots,
                       void* key_pages, void* value_pages, int tokens, int heads, int kv_heads,
                       int head_dim, int rotary_dim, int block_size, int num_pages, int write,
@@ -56,10 +57,16 @@ int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, 
 int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                     int out_is_f32, int dtype, int m, int n, int k, hipStream_t stream);
 
+// The same product in bfloat16 on the matrix cores (float32 accumulation).  Needs
+// k % 8 == 0 and 16-byte aligned x and w; any m and n.
+int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
+                  int out_is_f32, int m, int n, int k, hipStream_t stream);
+
 // Attention of every token over its request's pages: token t (entry
 // token_entry[t], absolute position positions[t]) sees the keys
 // max(0, p - window + 1) .. p of its entry's block table row (window 0: all).
-// q is read from q[t * q_stride + head * head_dim + i]; out is [tokens, heads * head_dim].
+// q is read from q[t * q_stride + head * head_dim + i]; out is [tokens, heads * head_dim];
+// pages are laid out as for mlr_rope_kv_write.
 // A page id outside [0, num_pages) among the visible keys gives a NaN row.
 int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_pages,
                                const void* value_pages, const int* block_table, int table_width,

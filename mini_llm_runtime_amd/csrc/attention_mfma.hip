@@ -1,0 +1,531 @@
+// bfloat16 paged attention on the matrix cores for one head size (MLR_HEAD_DIM,
+// a multiple of 16 up to 256); one shared library per head size.
+//
+// Both kernels compute scores transposed, S^T[key, row] = K[key, :] . Q[row, :],
+// so that the accumulator layout of the first product (a lane holds 4 consecutive
+// keys of one row) is exactly the operand layout of the second product
+// O^T[dim, row] = V^T[dim, key] . P^T[key, row]: probabilities go from one MFMA
+// to the next in registers.  Keys are read from pages [page, kv_head, offset, dim]
+// (dim fastest: operand of the first product), values from pages
+// [page, kv_head, dim, offset] (key position fastest: operand of the second).
+// Softmax is the online form with float32 max, sum and accumulator
+// (csrc/paged_attention_cuda.cu:87-105 of the reference); a lane's column is one
+// row (a query head, or a query token), so max and sum are per lane.
+//
+//  * attn_decode: entries with ONE new token.  A workgroup takes one (entry,
+//    KV head, partition of the keys); the g query heads that share the KV head
+//    are the 16 columns of the MFMA tile, so keys and values are read once per
+//    KV head (the reference's kernel reads them once per query head,
+//    csrc/paged_attention_cuda.cu:44-46).  Four wavefronts take 16-key tiles in
+//    turn and merge through LDS; partitions merge in attn_decode_merge with the
+//    reference's rule m = max m_j, O = sum w_j a_j / sum w_j l_j, w_j = exp(m_j - m)
+//    (csrc/paged_attention_split_cuda.cu:66-88).
+//  * attn_prefill: entries with several new tokens (prompt portions), in tiles of
+//    64 queries of one head; key and value tiles of 64 positions are staged in LDS
+//    and shared by the four wavefronts (16 queries each).  A query at position p
+//    sees keys first..p of its request, read from the pages after the step's own
+//    keys were written, so a portion behind a cached prefix needs nothing special.
+#define MLR_ERROR_CHANNEL
+#include "common.h"
+#include "mfma.h"
+
+#ifndef MLR_HEAD_DIM
+#error "compile with -DMLR_HEAD_DIM=<multiple of 16>"
+#endif
+
+namespace mlr {
+
+constexpr int D = MLR_HEAD_DIM;
+static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 within 16..256");
+constexpr int kSteps32 = D / 32;       // full 16x16x32 steps over the head dims
+constexpr bool kTail16 = (D % 32) != 0;  // one 16x16x16 step for the last 16 dims
+constexpr int kDimTiles = D / 16;
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4_t mfma_16x16x16(s16x4_t a, s16x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ s16x4_t pack_bf16x4(float a, float b, float c, float d) {
+  s16x4_t r;
+  r[0] = static_cast<short>(f32_to_bf16(a).bits);
+  r[1] = static_cast<short>(f32_to_bf16(b).bits);
+  r[2] = static_cast<short>(f32_to_bf16(c).bits);
+  r[3] = static_cast<short>(f32_to_bf16(d).bits);
+  return r;
+}
+
+// The query operand of one row: D dims as 16-byte chunks (and an 8-byte tail).
+struct QueryOperand {
+  bf16x8_t full[kSteps32 > 0 ? kSteps32 : 1];
+  s16x4_t tail;
+};
+
+__device__ __forceinline__ QueryOperand load_query(const bf16* row, bool valid, int quarter) {
+  QueryOperand q;
+#pragma unroll
+  for (int s = 0; s < kSteps32; ++s)
+    q.full[s] = valid ? load_bf16x8(row + s * 32 + quarter * 8) : zero_bf16x8();
+  q.tail = s16x4_t{0, 0, 0, 0};
+  if (kTail16 && valid) q.tail = *reinterpret_cast<const s16x4_t*>(row + kSteps32 * 32 + quarter * 4);
+  return q;
+}
+
+// S^T tile [16 keys x 16 rows]: `krow` points at this lane's key row (dim 0), in
+// global memory or LDS.
+__device__ __forceinline__ f32x4_t score_tile(const bf16* krow, bool valid, const QueryOperand& q, int quarter) {
+  f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < kSteps32; ++st) {
+    const bf16x8_t a = valid ? load_bf16x8(krow + st * 32 + quarter * 8) : zero_bf16x8();
+    s = mfma_16x16x32(a, q.full[st], s);
+  }
+  if (kTail16) {
+    s16x4_t a = {0, 0, 0, 0};
+    if (valid) a = *reinterpret_cast<const s16x4_t*>(krow + kSteps32 * 32 + quarter * 4);
+    s = mfma_16x16x16(a, q.tail, s);
+  }
+  return s;
+}
+
+// Running softmax state of one column (row of the attention problem) in a lane.
+struct Softmax {
+  float m;
+  float l;  // this lane's share of the sum (its own 4 keys of every tile)
+};
+
+// Fold a tile of 4 scores into the state; returns the probabilities as the B
+// operand of the value product and the factor the accumulator must be scaled by.
+__device__ __forceinline__ s16x4_t softmax_tile(Softmax& st, f32x4_t s, const bool (&ok)[4], float scale,
+                                                float& alpha) {
+  float v[4];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[i] = ok[i] ? s[i] * scale : -INFINITY;
+    tmax = fmaxf(tmax, v[i]);
+  }
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+  const float m_new = fmaxf(st.m, tmax);
+  alpha = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+  float p[4];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    p[i] = (v[i] == -INFINITY) ? 0.f : __expf(v[i] - m_new);
+    sum += p[i];
+  }
+  st.l = st.l * alpha + sum;
+  st.m = m_new;
+  return pack_bf16x4(p[0], p[1], p[2], p[3]);
+}
+
+// ---- decode ---------------------------------------------------------------------------------
+constexpr int kDecodeWaves = D > 128 ? 2 : 4;  // bounded by the LDS the merge needs
+constexpr int kPartialStride = D + 2;  // numerator[D], max, denominator
+
+__global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
+    const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
+    const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
+    float* __restrict__ partial, int heads, int kv_heads, int head_tiles, int block_size, int num_pages,
+    float scale, int window, int part, int splits) {
+  __shared__ float sm_acc[kDecodeWaves][16][D];
+  __shared__ float sm_m[kDecodeWaves][16];
+  __shared__ float sm_l[kDecodeWaves][16];
+  __shared__ int sm_bad;
+
+  const int entry = blockIdx.x;
+  const int kvh = blockIdx.y / head_tiles;
+  const int htile = blockIdx.y % head_tiles;
+  const int split = blockIdx.z;
+  const int t = cu_q[entry];
+  if (cu_q[entry + 1] - t != 1) return;  // not a single-token entry: the prefill kernel owns it
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int col = lane % 16;      // query head within the tile
+  const int quarter = lane / 16;  // which 4 keys of a tile / which chunk of the dims
+  const int group = heads / kv_heads;
+  const int head_in_group = htile * 16 + col;
+  const bool head_ok = head_in_group < group;
+  const int head = kvh * group + head_in_group;
+
+  const int ctx = context_lens[entry];
+  const int p = ctx - 1;
+  const int first = window > 0 ? max(0, p - window + 1) : 0;
+  const int base = (first / 16) * 16;
+  const int kb = base + split * part;
+  const int ke = min(kb + part, ctx);
+  const int* table = block_table + static_cast<int64_t>(entry) * table_width;
+  if (tid == 0) sm_bad = 0;
+  __syncthreads();
+
+  const QueryOperand qo =
+      load_query(q + t * q_stride + static_cast<int64_t>(head_ok ? head : 0) * D, head_ok, quarter);
+
+  Softmax sm{-INFINITY, 0.f};
+  f32x4_t acc[kDimTiles];
+#pragma unroll
+  for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  bool bad = false;
+
+  for (int ts = kb + wave * 16; ts < ke; ts += kDecodeWaves * 16) {
+    // key operand: this lane's row is key ts + col
+    const int key_a = ts + col;
+    bool valid_a = key_a < ke;
+    const bf16* krow = key_pages;
+    if (valid_a) {
+      const int logical = key_a / block_size;
+      const int page = table[logical];
+      if (page < 0 || page >= num_pages) {
+        bad = bad || key_a >= first;
+        valid_a = false;
+      } else {
+        krow = key_pages +
+               ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size + (key_a - logical * block_size)) * D;
+      }
+    }
+    // value operand: this lane's 4 keys are ts + quarter * 4 .. + 3, inside one page
+    const int key_v = ts + quarter * 4;
+    bool valid_v = key_v < ke;
+    const bf16* vbase = value_pages;
+    if (valid_v) {
+      const int logical = key_v / block_size;
+      const int page = table[logical];
+      if (page < 0 || page >= num_pages) {
+        valid_v = false;
+      } else {
+        vbase = value_pages + (static_cast<int64_t>(page) * kv_heads + kvh) * D * block_size +
+                (key_v - logical * block_size);
+      }
+    }
+    s16x4_t vt[kDimTiles];
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt) {
+      vt[dt] = s16x4_t{0, 0, 0, 0};
+      if (valid_v) vt[dt] = *reinterpret_cast<const s16x4_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size);
+    }
+
+    const f32x4_t s = score_tile(krow, valid_a, qo, quarter);
+    bool ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = key_v + i;
+      ok[i] = key >= first && key < ke;
+      if (!ok[i]) {
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt) vt[dt][i] = 0;  // unwritten slots may hold NaN
+      }
+    }
+    float alpha;
+    const s16x4_t pb = softmax_tile(sm, s, ok, scale, alpha);
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+      acc[dt] = mfma_16x16x16(vt[dt], pb, acc[dt]);
+    }
+  }
+
+  // the column's sum is spread over the four lanes that share it
+  sm.l += __shfl_xor(sm.l, 16, kWave);
+  sm.l += __shfl_xor(sm.l, 32, kWave);
+  if (bad) atomicOr(&sm_bad, 1);
+  if (quarter == 0) {
+    sm_m[wave][col] = sm.m;
+    sm_l[wave][col] = sm.l;
+  }
+#pragma unroll
+  for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sm_acc[wave][col][dt * 16 + quarter * 4 + i] = acc[dt][i];
+  __syncthreads();
+
+  const bool poisoned = sm_bad != 0;
+  for (int idx = tid; idx < 16 * D; idx += kDecodeWaves * kWave) {
+    const int c = idx / D;
+    const int d = idx - c * D;
+    const int hig = htile * 16 + c;
+    if (hig >= group) continue;
+    float mstar = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kDecodeWaves; ++w) mstar = fmaxf(mstar, sm_m[w][c]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < kDecodeWaves; ++w) {
+      const float wgt = (sm_m[w][c] == -INFINITY) ? 0.f : __expf(sm_m[w][c] - mstar);
+      num += wgt * sm_acc[w][c][d];
+      den += wgt * sm_l[w][c];
+    }
+    const int h = kvh * group + hig;
+    if (splits == 1) {
+      const float v = poisoned ? __builtin_nanf("") : num / den;
+      out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(v);
+    } else {
+      float* dst = partial + ((static_cast<int64_t>(entry) * heads + h) * splits + split) * kPartialStride;
+      dst[d] = poisoned ? __builtin_nanf("") : num;
+      if (d == 0) {
+        dst[D] = mstar;
+        dst[D + 1] = den;
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* __restrict__ partial,
+                                                                  const int* __restrict__ cu_q,
+                                                                  bf16* __restrict__ out, int heads, int splits) {
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int t = cu_q[entry];
+  if (cu_q[entry + 1] - t != 1) return;
+  const float* src = partial + (static_cast<int64_t>(entry) * heads + h) * splits * kPartialStride;
+  float mstar = -INFINITY;
+  for (int s = 0; s < splits; ++s) mstar = fmaxf(mstar, src[s * kPartialStride + D]);
+  float den = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = src[s * kPartialStride + D];
+    if (ms != -INFINITY) den += __expf(ms - mstar) * src[s * kPartialStride + D + 1];
+  }
+  for (int d = threadIdx.x; d < D; d += kWave) {
+    float num = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = src[s * kPartialStride + D];
+      if (ms != -INFINITY) num += __expf(ms - mstar) * src[s * kPartialStride + d];
+    }
+    out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(num / den);
+  }
+}
+
+// ---- prefill ----------------------------------------------------------------------------------
+constexpr int kTileQ = 64;   // queries per workgroup (16 per wavefront)
+constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounded by LDS)
+constexpr int kKLd = D + 8;  // padded key row in LDS (elements)
+constexpr int kVLd = kTileK + 8;
+
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
+    const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
+    bf16* __restrict__ out, int heads, int kv_heads, int block_size, int num_pages, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) bf16 ks[kTileK * kKLd];
+  __shared__ __attribute__((aligned(16))) bf16 vs[D * kVLd];
+  __shared__ int sm_bad;
+
+  const int entry = tiles[2 * blockIdx.x];
+  const int q0 = tiles[2 * blockIdx.x + 1];
+  const int head = blockIdx.y;
+  const int kvh = head / (heads / kv_heads);
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int col = lane % 16;
+  const int quarter = lane / 16;
+
+  const int t_first = cu_q[entry];
+  const int q_len = cu_q[entry + 1] - t_first;
+  const int ctx = context_lens[entry];
+  const int pos0 = ctx - q_len;  // position of the entry's first new token
+  const int* table = block_table + static_cast<int64_t>(entry) * table_width;
+  if (tid == 0) sm_bad = 0;
+  __syncthreads();
+
+  // this lane's query (a column of S^T)
+  const int qi = q0 + wave * 16 + col;
+  const bool q_ok = qi < q_len;
+  const int pq = pos0 + qi;  // its absolute position
+  const int pq_first = window > 0 ? max(0, pq - window + 1) : 0;
+  const QueryOperand qo = load_query(
+      q + static_cast<int64_t>(t_first + (q_ok ? qi : 0)) * q_stride + static_cast<int64_t>(head) * D, q_ok, quarter);
+
+  // key range of the workgroup: from the first query's window start to the last query's position
+  const int last_q = min(q0 + kTileQ, q_len) - 1;
+  const int k_end = pos0 + last_q + 1;
+  const int k_begin_raw = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
+  const int k_begin = (k_begin_raw / kTileK) * kTileK;
+  // the wavefront's own range (uniform within the wavefront)
+  const int w_last = pos0 + min(q0 + wave * 16 + 15, q_len - 1);
+  const int w_first = window > 0 ? max(0, pos0 + q0 + wave * 16 - window + 1) : 0;
+  const bool wave_has_queries = q0 + wave * 16 < q_len;
+
+  Softmax sm{-INFINITY, 0.f};
+  f32x4_t acc[kDimTiles];
+#pragma unroll
+  for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  bool bad = false;
+
+  for (int kt0 = k_begin; kt0 < k_end; kt0 += kTileK) {
+    __syncthreads();  // the previous tile has been consumed
+    // keys: kTileK rows of D dims, 16-byte chunks
+    for (int c = tid; c < kTileK * (D / 8); c += 256) {
+      const int row = c / (D / 8);
+      const int ch = c - row * (D / 8);
+      const int key = kt0 + row;
+      bf16x8_t val = zero_bf16x8();
+      if (key < k_end) {
+        const int logical = key / block_size;
+        const int page = table[logical];
+        if (page < 0 || page >= num_pages) {
+          bad = bad || key >= k_begin_raw;
+        } else {
+          val = load_bf16x8(key_pages +
+                            ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size +
+                             (key - logical * block_size)) * D + ch * 8);
+        }
+      }
+      *reinterpret_cast<bf16x8_t*>(ks + row * kKLd + ch * 8) = val;
+    }
+    // values: per page a contiguous [D][block_size] block; 8-byte chunks of 4 key positions
+    {
+      const int per_row = block_size / 4;      // chunks per dim row of a page
+      const int per_page = D * per_row;        // chunks per page
+      const int pages_in_tile = kTileK / block_size;
+      for (int c = tid; c < pages_in_tile * per_page; c += 256) {
+        const int pg = c / per_page;
+        const int rem = c - pg * per_page;
+        const int d = rem / per_row;
+        const int kg = rem - d * per_row;
+        const int key = kt0 + pg * block_size + kg * 4;
+        s16x4_t val = {0, 0, 0, 0};
+        if (key < k_end) {
+          const int page = table[key / block_size];
+          if (page >= 0 && page < num_pages) {
+            val = *reinterpret_cast<const s16x4_t*>(
+                value_pages + ((static_cast<int64_t>(page) * kv_heads + kvh) * D + d) * block_size + kg * 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (key + i >= k_end) val[i] = 0;  // beyond the last visible key: may be unwritten
+          }
+        }
+        *reinterpret_cast<s16x4_t*>(vs + d * kVLd + pg * block_size + kg * 4) = val;
+      }
+    }
+    __syncthreads();
+    if (!wave_has_queries) continue;
+#pragma unroll
+    for (int sub = 0; sub < kTileK / 16; ++sub) {
+      const int ts = kt0 + sub * 16;
+      if (ts > w_last || ts + 15 < w_first) continue;  // nothing visible to this wavefront
+      const f32x4_t s = score_tile(ks + (sub * 16 + col) * kKLd, true, qo, quarter);
+      bool ok[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = ts + quarter * 4 + i;
+        ok[i] = q_ok && key <= pq && key >= pq_first;
+      }
+      float alpha;
+      const s16x4_t pb = softmax_tile(sm, s, ok, scale, alpha);
+#pragma unroll
+      for (int dt = 0; dt < kDimTiles; ++dt) {
+        const s16x4_t va =
+            *reinterpret_cast<const s16x4_t*>(vs + (dt * 16 + col) * kVLd + sub * 16 + quarter * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+        acc[dt] = mfma_16x16x16(va, pb, acc[dt]);
+      }
+    }
+  }
+
+  if (bad) atomicOr(&sm_bad, 1);
+  __syncthreads();
+  const bool poisoned = sm_bad != 0;
+  sm.l += __shfl_xor(sm.l, 16, kWave);
+  sm.l += __shfl_xor(sm.l, 32, kWave);
+  if (q_ok) {
+    const float inv = 1.0f / sm.l;
+    bf16* orow = out + (static_cast<int64_t>(t_first + qi) * heads + head) * D;
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt) {
+      u16x4_t packed;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        packed[i] = f32_to_bf16(poisoned ? __builtin_nanf("") : acc[dt][i] * inv).bits;
+      *reinterpret_cast<u16x4_t*>(orow + dt * 16 + quarter * 4) = packed;
+    }
+  }
+}
+
+}  // namespace mlr
+
+using namespace mlr;
+
+extern "C" {
+
+int mlr_attention_head_dim() { return D; }
+
+// Key positions per LDS tile of the prefill kernel; block_size must divide it.
+int mlr_attention_key_tile() { return kTileK; }
+
+// Floats of scratch the decode kernel needs for `splits` partitions.
+int64_t mlr_attention_decode_scratch(int entries, int heads, int splits) {
+  return splits <= 1 ? 0 : static_cast<int64_t>(entries) * heads * splits * kPartialStride;
+}
+
+// Attention of every single-token entry (entries with more tokens are skipped).
+// Keys of an entry are cut into `splits` partitions of `part` positions (a
+// multiple of 64); with more than one partition `partial` must hold
+// mlr_attention_decode_scratch floats.
+int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
+                         const int* block_table, int table_width, const int* cu_q, const int* context_lens,
+                         void* out, float* partial, int entries, int heads, int kv_heads, int block_size,
+                         int num_pages, float scale, int window, int part, int splits, hipStream_t stream) {
+  MLR_REQUIRE(q && key_pages && value_pages && block_table && cu_q && context_lens && out, "null pointer");
+  MLR_REQUIRE(entries > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
+  MLR_REQUIRE(block_size > 0 && block_size % 4 == 0, "block_size must be a multiple of 4");
+  MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
+  MLR_REQUIRE(part > 0 && part % 64 == 0, "part must be a positive multiple of 64");
+  MLR_REQUIRE(splits >= 1 && splits <= 65535, "splits out of range");
+  MLR_REQUIRE(splits == 1 || partial != nullptr, "several partitions need scratch memory");
+  MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * D && q_stride % 8 == 0, "q_stride must cover a row and keep 16-byte alignment");
+  MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(value_pages) % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
+              "operands must be 16-byte aligned");
+  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
+  const int group = heads / kv_heads;
+  const int head_tiles = (group + 15) / 16;
+  MLR_REQUIRE(kv_heads * head_tiles <= 65535, "too many heads for one launch");
+  dim3 grid(entries, kv_heads * head_tiles, splits);
+  attn_decode_kernel<<<grid, kDecodeWaves * kWave, 0, stream>>>(
+      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
+      static_cast<const bf16*>(value_pages), block_table, table_width, cu_q, context_lens,
+      static_cast<bf16*>(out), partial, heads, kv_heads, head_tiles, block_size, num_pages, scale, window, part,
+      splits);
+  MLR_LAUNCH_CHECK();
+  if (splits > 1) {
+    attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, static_cast<bf16*>(out),
+                                                                         heads, splits);
+    MLR_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// Attention of the query tiles listed in `tiles` ([num_tiles][2]: entry, first
+// query of the tile within the entry's new tokens; 64 queries per tile).
+int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
+                          const int* block_table, int table_width, const int* tiles, int num_tiles,
+                          const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
+                          int block_size, int num_pages, float scale, int window, hipStream_t stream) {
+  MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
+  MLR_REQUIRE(num_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad sizes");
+  MLR_REQUIRE(block_size >= 4 && block_size % 4 == 0 && kTileK % block_size == 0,
+              "block_size must be a multiple of 4 that divides the key tile");
+  MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
+  MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * D && q_stride % 8 == 0, "q_stride must cover a row and keep 16-byte alignment");
+  MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(value_pages) % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
+              "operands must be 16-byte aligned");
+  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
+  MLR_REQUIRE(heads <= 65535, "too many heads for one launch");
+  attn_prefill_kernel<<<dim3(num_tiles, heads), 256, 0, stream>>>(
+      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
+      static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,
+      static_cast<bf16*>(out), heads, kv_heads, block_size, num_pages, scale, window);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -25,6 +25,7 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[kWave];
   __shared__ int64_t offs[kWave];
+  __shared__ int64_t voffs[kWave];
 
   const int t = blockIdx.x;
   const int h = blockIdx.y;
@@ -53,14 +54,17 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const int kpos = k0 + lane;
     float s = -INFINITY;
     int64_t off = -1;
+    int64_t voff = -1;
     if (kpos <= p) {
       const int logical = kpos / block_size;
       const int page = logical < table_width ? table[logical] : -1;
       if (page < 0 || page >= num_pages) {
         bad = true;
       } else {
-        off = ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size + (kpos - logical * block_size)) *
-              head_dim;
+        const int in_page = kpos - logical * block_size;
+        const int64_t head_base = (static_cast<int64_t>(page) * kv_heads + kvh) * block_size * head_dim;
+        off = head_base + static_cast<int64_t>(in_page) * head_dim;  // keys: [offset][dim]
+        voff = head_base + in_page;                                   // values: [dim][offset]
         const T* kp = key_pages + off;
         float dot = 0.f;
         for (int i = 0; i < head_dim; ++i) dot = fmaf(qs[i], to_f32(kp[i]), dot);
@@ -74,19 +78,19 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     m = m_new;
     ps[lane] = pr;
     offs[lane] = off;
+    voffs[lane] = voff;
     __syncthreads();
     const int count = min(kWave, p - k0 + 1);
 #pragma unroll
     for (int j = 0; j < kMaxHeadDim / kWave; ++j) acc[j] *= alpha;
     for (int i = 0; i < count; ++i) {
-      const int64_t o = offs[i];
-      if (o < 0) continue;
+      if (offs[i] < 0) continue;
       const float pi = ps[i];
-      const T* vp = value_pages + o;
+      const T* vp = value_pages + voffs[i];
 #pragma unroll
       for (int j = 0; j < kMaxHeadDim / kWave; ++j) {
         const int dim = lane + j * kWave;
-        if (dim < head_dim) acc[j] = fmaf(pi, to_f32(vp[dim]), acc[j]);
+        if (dim < head_dim) acc[j] = fmaf(pi, to_f32(vp[static_cast<int64_t>(dim) * block_size]), acc[j]);
       }
     }
     __syncthreads();

@@ -108,12 +108,17 @@ __device__ inline float block_max(float v, float* scratch) {
 
 void set_error(const std::string& message);
 
-inline bool fail(const std::string& message) {
-  set_error(message);
-  return false;
-}
+// Each shared library defines MLR_ERROR_CHANNEL in exactly one of its sources.
+#ifdef MLR_ERROR_CHANNEL
+static thread_local std::string g_error;
+void set_error(const std::string& message) { g_error = message; }
+#endif
 
 }  // namespace mlr
+
+#ifdef MLR_ERROR_CHANNEL
+extern "C" const char* mlr_last_error() { return mlr::g_error.c_str(); }
+#endif
 
 // Entry points return 0 on success and -1 after storing a message for
 // mlr_last_error().

@@ -2,13 +2,11 @@
 // residual addition, SiLU-multiply, rotary tables, and the fused rotary encoding
 // plus paged key/value store.  All arithmetic is float32; bfloat16 only exists
 // in memory.
+#define MLR_ERROR_CHANNEL
 #include "api.h"
 #include "common.h"
 
 namespace mlr {
-
-static thread_local std::string g_error;
-void set_error(const std::string& message) { g_error = message; }
 
 // ---- embedding -------------------------------------------------------------------
 // qwen_model_runner.py:263 (F.embedding): a row gather, no scaling.
@@ -113,8 +111,9 @@ __global__ __launch_bounds__(256) void rope_table_kernel(const int* __restrict__
 
 // ---- rotary encoding + paged key/value store ------------------------------------------
 // qwen_model_runner.py:56-61 (x * cos + rotate_half(x) * sin: dims j and j + r/2 are
-// a pair) and :105-109 (the cache keeps the rotated k and the raw v); page layout
-// [page, kv_head, offset, head_dim] as paged_kv_cache.py:287-291.
+// a pair) and :105-109 (the cache keeps the rotated k and the raw v).  Key pages are
+// [page, kv_head, offset, head_dim] as paged_kv_cache.py:287-291; value pages are
+// transposed inside a page, [page, kv_head, head_dim, offset].
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
@@ -129,15 +128,18 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   const float* cs = cos_t + static_cast<int64_t>(t) * half;
   const float* sn = sin_t + static_cast<int64_t>(t) * half;
 
-  int64_t page_base = -1;  // element offset of (page, kv_head 0, offset, 0)
+  int64_t page_base = -1;   // element offset of key (page, kv_head 0, offset, 0)
+  int64_t value_base = -1;  // element offset of value (page, kv_head 0, dim 0, offset)
   int64_t head_stride = static_cast<int64_t>(block_size) * head_dim;
   if (write) {
     const int slot = slots[t];
     if (slot >= 0) {
       const int page = slot / block_size;
       const int off = slot - page * block_size;
-      if (page < num_pages)
+      if (page < num_pages) {
         page_base = (static_cast<int64_t>(page) * kv_heads * block_size + off) * head_dim;
+        value_base = static_cast<int64_t>(page) * kv_heads * head_stride + off;
+      }
     }
   }
 
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     for (int i = threadIdx.x; i < kv_heads * head_dim; i += blockDim.x) {
       const int h = i / head_dim;
       const int j = i - h * head_dim;
-      value_pages[page_base + h * head_stride + j] = v[h * head_dim + j];
+      value_pages[value_base + h * head_stride + static_cast<int64_t>(j) * block_size] = v[h * head_dim + j];
     }
   }
 }
@@ -186,8 +188,6 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
 using namespace mlr;
 
 extern "C" {
-
-const char* mlr_last_error() { return g_error.c_str(); }
 
 int mlr_version() { return 1; }
 

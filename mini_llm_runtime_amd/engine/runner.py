@@ -25,6 +25,8 @@ from ..cache.spec import PagedKVSpec, SlotStateSpec
 from ..parts.context import KVView, StateView, StepContext
 from ..parts.model import DecoderModel
 
+QUERY_TILE = 64  # queries per tile of the attention plan
+
 
 @dataclass(frozen=True)
 class StepEntry:
@@ -104,6 +106,9 @@ class ModelRunner:
 
     def _upload(self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray) -> StepContext:
         groups = len(self.cache.groups)
+        single = layout.q_lens == 1
+        tiles = [(r, q0) for r, n in enumerate(layout.q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
+        tile_array = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
         arrays = [
             token_ids,
             layout.positions,
@@ -114,6 +119,7 @@ class ModelRunner:
             layout.state_read,
             layout.state_write,
             logit_rows,
+            tile_array,
             *layout.slot_mappings,
             *layout.block_tables,
         ]
@@ -143,11 +149,15 @@ class ModelRunner:
             max_q_len=int(layout.q_lens.max()),
             max_context_len=int(layout.context_lens.max()),
             host=layout,
+            query_tiles=view(9) if tiles else None,
+            num_query_tiles=len(tiles),
+            num_decode_entries=int(single.sum()),
+            max_decode_context=int(layout.context_lens[single].max()) if single.any() else 0,
         )
         state_read, state_write = view(6), view(7)
         ctx.memo["logit_rows"] = view(8)
-        slot_maps = [view(9 + g) for g in range(groups)]
-        tables = [view(9 + groups + g) for g in range(groups)]
+        slot_maps = [view(10 + g) for g in range(groups)]
+        tables = [view(10 + groups + g) for g in range(groups)]
         for site in range(self.model.num_sites):
             source = self.model.cache_site_of(site)
             spec = self.cache.site_specs[source]

@@ -56,15 +56,27 @@ CORE = Module(
     (
         "elementwise.hip",
         "gemm_simple.hip",
+        "gemm_mfma.hip",
         "attention_simple.hip",
         "sampling.hip",
     ),
 )
 
 
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
+
+
+def attention_module(head_dim: int) -> Module:
+    """The MFMA attention kernels for one head size (a multiple of 16 within 16..256)."""
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise ValueError("the MFMA attention kernels take head sizes in steps of 16 up to 256")
+    return Module(f"attention_d{head_dim}", ("attention_mfma.hip",), (f"MLR_HEAD_DIM={head_dim}",))
+
+
 def all_modules() -> list[Module]:
-    """Every module a default build compiles."""
-    return [CORE]
+    """Every module a default build compiles: the core library and the attention
+    kernels of the usual head sizes (other sizes are compiled when a model needs them)."""
+    return [CORE] + [attention_module(d) for d in DEFAULT_HEAD_DIMS]
 
 
 def log(message: str) -> None:

@@ -13,6 +13,7 @@ a memory fault on the GPU.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Any, Optional, Sequence, Union
 
 import torch
@@ -34,12 +35,34 @@ _SIGNATURES = {
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
         _I,
     ),
     "mlr_sample": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
+    "mlr_attention_head_dim": ([], _I),
+    "mlr_attention_key_tile": ([], _I),
+    "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
+    "mlr_attention_decode": (
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _VP],
+        _I,
+    ),
+    "mlr_attention_prefill": (
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
+        _I,
+    ),
 }
+
+QUERY_TILE = 64  # queries per workgroup of the prefill attention kernel
+
+
+def query_tiles(q_lens) -> "np.ndarray":
+    """[num_tiles, 2] int32 (entry, first query) covering every entry with more than one new token."""
+    import numpy as np
+
+    tiles = [(r, q0) for r, n in enumerate(q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
+    return np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
 
 
 class KernelError(RuntimeError):
@@ -87,15 +110,28 @@ class HipOps:
         self.lib = load_library(build.CORE)
         if self.lib.mlr_version() != 1:
             raise KernelError("the built kernel library is of another version than this package")
+        self._attention_libs: dict[int, ctypes.CDLL] = {}
+        self.decode_partition = int(os.environ.get("MLR_DECODE_PARTITION", "256"))
+
+    def attention_library(self, head_dim: int) -> ctypes.CDLL:
+        """The MFMA attention kernels of one head size, compiled on first use."""
+        lib = self._attention_libs.get(head_dim)
+        if lib is None:
+            lib = load_library(build.attention_module(head_dim))
+            if lib.mlr_attention_head_dim() != head_dim:
+                raise KernelError(f"the attention library for head size {head_dim} was built for another size")
+            self._attention_libs[head_dim] = lib
+        return lib
 
     # ---- helpers --------------------------------------------------------------------------
     def _stream(self) -> _VP:
         return _VP(torch.cuda.current_stream(self.device).cuda_stream)
 
-    def _call(self, name: str, *args: Any) -> None:
-        status = getattr(self.lib, name)(*args)
+    def _call(self, name: str, *args: Any, lib: Optional[ctypes.CDLL] = None) -> None:
+        lib = lib or self.lib
+        status = getattr(lib, name)(*args)
         if status != 0:
-            raise KernelError(self.lib.mlr_last_error().decode("utf-8", "replace"))
+            raise KernelError(lib.mlr_last_error().decode("utf-8", "replace"))
 
     def _check(
         self,
@@ -178,8 +214,13 @@ class HipOps:
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
         out_dtype: Optional[torch.dtype] = None,
+        kernel: str = "auto",
     ) -> torch.Tensor:
-        """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics."""
+        """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
+
+        bfloat16 products run on the matrix cores when k is a multiple of 8; float32
+        products, and everything with kernel="fma", run as plain 32-bit FMA arithmetic.
+        """
         self._check(x, "linear input", self.dtype, (None, None))
         m, k = x.shape
         self._check(weight, "linear weight", self.dtype, (None, k))
@@ -190,6 +231,15 @@ class HipOps:
         if out_dtype not in (torch.float32, self.dtype):
             raise KernelError(f"linear output must be float32 or {self.dtype}")
         y = self._empty((m, n), out_dtype)
+        if kernel not in ("auto", "fma"):
+            raise KernelError("kernel must be 'auto' or 'fma'")
+        if kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0:
+            self._call(
+                "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias),
+                int(bias is not None and bias.dtype == torch.float32), self._ptr(y),
+                int(out_dtype == torch.float32), m, n, k, self._stream(),
+            )
+            return y
         self._call(
             "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias),
             int(bias is not None and bias.dtype == torch.float32), self._ptr(y),
@@ -221,7 +271,7 @@ class HipOps:
 
     def _check_pages(self, key_pages, value_pages, num_kv_heads, head_dim, block_size) -> int:
         self._check(key_pages, "key pages", self.dtype, (None, num_kv_heads, block_size, head_dim))
-        self._check(value_pages, "value pages", self.dtype, tuple(key_pages.shape))
+        self._check(value_pages, "value pages", self.dtype, (key_pages.shape[0], num_kv_heads, head_dim, block_size))
         return key_pages.shape[0]
 
     def rope_kv_write(
@@ -274,29 +324,89 @@ class HipOps:
         block_size: int,
         scale: float,
         window: Optional[int],
+        kernel: str = "auto",
     ) -> torch.Tensor:
         """Causal attention of the step's tokens over their requests' pages.
 
         qkv: [T, >= num_heads * head_dim], queries in the leading columns (already
-        position-encoded); returns [T, num_heads * head_dim].
+        position-encoded); returns [T, num_heads * head_dim].  `ctx` describes the
+        batch (StepContext).  bfloat16 with a head size in steps of 16 and a block
+        size that is a multiple of 4 runs on the matrix cores: single-token entries
+        through the split-KV decode kernel, the others through the tiled prefill
+        kernel.  Everything else (float32, other sizes, kernel="fma") runs the plain
+        32-bit kernel.
         """
         self._check(qkv, "queries", self.dtype, (None, None))
         tokens, stride = qkv.shape
         if stride < num_heads * head_dim:
             raise KernelError("the query rows are narrower than num_heads * head_dim")
+        if num_heads % num_kv_heads:
+            raise KernelError("query heads must be a multiple of KV heads")
         num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
-        self._check(block_table, "block table", torch.int32, (ctx.num_entries, None))
+        entries = ctx.num_entries
+        self._check(block_table, "block table", torch.int32, (entries, None))
         self._check(ctx.token_entry, "token entries", torch.int32, (tokens,))
         self._check(ctx.positions, "positions", torch.int32, (tokens,))
         if block_table.shape[1] * block_size < ctx.max_context_len:
             raise KernelError("the block table is narrower than the longest context")
+        if kernel not in ("auto", "fma"):
+            raise KernelError("kernel must be 'auto' or 'fma'")
         out = self._empty((tokens, num_heads * head_dim), self.dtype)
-        self._call(
-            "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
-            self._ptr(block_table), block_table.shape[1], self._ptr(ctx.token_entry), self._ptr(ctx.positions),
-            self._ptr(out), self.code, tokens, ctx.num_entries, num_heads, num_kv_heads, head_dim, block_size,
-            num_pages, float(scale), int(window or 0), self._stream(),
+        width = block_table.shape[1]
+        use_mfma = (
+            kernel == "auto"
+            and self.dtype == torch.bfloat16
+            and head_dim % 16 == 0
+            and 16 <= head_dim <= 256
+            and block_size % 4 == 0
+            and stride % 8 == 0
         )
+        num_tiles = int(getattr(ctx, "num_query_tiles", 0))
+        num_decode = int(getattr(ctx, "num_decode_entries", 0))
+        if use_mfma and num_tiles + num_decode == 0:
+            use_mfma = False  # a caller that planned nothing (kernel tests of the plain path)
+        lib = None
+        if use_mfma:
+            lib = self.attention_library(head_dim)
+            if num_tiles and lib.mlr_attention_key_tile() % block_size:
+                use_mfma = False
+        if not use_mfma:
+            self._call(
+                "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
+                self._ptr(block_table), width, self._ptr(ctx.token_entry), self._ptr(ctx.positions),
+                self._ptr(out), self.code, tokens, entries, num_heads, num_kv_heads, head_dim, block_size,
+                num_pages, float(scale), int(window or 0), self._stream(),
+            )
+            return out
+        self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
+        self._check(ctx.context_lens, "context lengths", torch.int32, (entries,))
+        if num_decode:
+            span = int(ctx.max_decode_context)
+            if window:
+                span = min(span, int(window) + 15)
+            group_tiles = -(-(num_heads // num_kv_heads) // 16)
+            base = num_decode * num_kv_heads * group_tiles
+            part = max(64, self.decode_partition // 64 * 64)
+            splits = max(1, min(-(-span // part), -(-1024 // base)))
+            part = -(-(-(-span // splits)) // 64) * 64
+            splits = -(-span // part)
+            partial = None
+            if splits > 1:
+                partial = self._empty((lib.mlr_attention_decode_scratch(entries, num_heads, splits),), torch.float32)
+            self._call(
+                "mlr_attention_decode", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
+                self._ptr(block_table), width, self._ptr(ctx.cu_q), self._ptr(ctx.context_lens), self._ptr(out),
+                self._ptr(partial), entries, num_heads, num_kv_heads, block_size, num_pages, float(scale),
+                int(window or 0), part, splits, self._stream(), lib=lib,
+            )
+        if num_tiles:
+            self._check(ctx.query_tiles, "query tiles", torch.int32, (num_tiles, 2))
+            self._call(
+                "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
+                self._ptr(block_table), width, self._ptr(ctx.query_tiles), num_tiles, self._ptr(ctx.cu_q),
+                self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
+                float(scale), int(window or 0), self._stream(), lib=lib,
+            )
         return out
 
     # ---- sampling -----------------------------------------------------------------------------------

@@ -13,8 +13,9 @@ import torch
 
 @dataclass
 class KVView:
-    """Pages of one site: [page, kv_head, offset, head_dim] keys and values, the
-    block table rows of the step's entries and the slot of each new token."""
+    """Pages of one site: keys [page, kv_head, offset, head_dim], values
+    [page, kv_head, head_dim, offset], the block table rows of the step's entries
+    and the slot of each new token."""
 
     key: torch.Tensor
     value: torch.Tensor
@@ -51,6 +52,12 @@ class StepContext:
     max_q_len: int
     max_context_len: int
     host: Any  # the StepLayout (numpy arrays) for parts that plan on the host
+    # plan for attention kernels: tiles of 64 queries over entries with several new
+    # tokens ([num_tiles, 2]: entry, first query), and the single-token entries
+    query_tiles: Optional[torch.Tensor] = None
+    num_query_tiles: int = 0
+    num_decode_entries: int = 0
+    max_decode_context: int = 0
     kv_views: dict[int, KVView] = field(default_factory=dict)
     state_views: dict[int, StateView] = field(default_factory=dict)
     memo: dict[Any, Any] = field(default_factory=dict)

@@ -90,7 +90,7 @@ class TorchOps:
             page = slots[ok] // block_size
             off = slots[ok] % block_size
             key_pages[page, :, off, :] = k[ok]
-            value_pages[page, :, off, :] = v[ok]
+            value_pages[page, :, :, off] = v[ok]
 
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window
@@ -109,7 +109,7 @@ class TorchOps:
             page = table[r, idx // block_size]
             assert (page >= 0).all(), "attention would read a page that is not there"
             k = key_pages[page, :, idx % block_size, :].float()  # [n, Hkv, d]
-            v = value_pages[page, :, idx % block_size, :].float()
+            v = value_pages[page, :, :, idx % block_size].float()
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)
             s = torch.einsum("hd,nhd->hn", q[t], k) * scale

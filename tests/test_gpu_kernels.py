@@ -128,6 +128,28 @@ def test_linear(ops_for, dtype, m, n, k):
             torch.testing.assert_close(got.double(), ref, **tol)
 
 
+@pytest.mark.parametrize(
+    "m,n,k",
+    [(1, 1152, 896), (8, 896, 4864), (3, 17, 8), (16, 130, 136), (17, 64, 96), (33, 517, 2056), (64, 9728, 896),
+     (65, 100, 64), (128, 128, 64), (200, 352, 1000), (300, 1152, 896), (2048, 896, 4864), (129, 151936, 96)],
+)
+def test_linear_bf16_matrix_cores(ops_for, m, n, k):
+    """The MFMA kernels (skinny for up to 64 tokens, tiled above) against float64 and against the FMA kernel."""
+    ops = ops_for(torch.bfloat16)
+    x = _rand((m, k), torch.bfloat16, 40)
+    w = _rand((n, k), torch.bfloat16, 41, 0.05)
+    b = _rand((n,), torch.float32, 42)
+    ref = x.double() @ w.double().t() + b.double()
+    xd, wd, bd = x.cuda(), w.cuda(), b.cuda()
+    got32 = ops.linear(xd, wd, bd, out_dtype=torch.float32).cpu().double()
+    # exact bfloat16 products, float32 accumulation: only the order of the k-long sums differs
+    torch.testing.assert_close(got32, ref, atol=1e-3 * (k / 1000) ** 0.5 + 1e-4, rtol=1e-4)
+    fma = ops.linear(xd, wd, bd, out_dtype=torch.float32, kernel="fma").cpu().double()
+    torch.testing.assert_close(got32, fma, atol=1e-3 * (k / 1000) ** 0.5 + 1e-4, rtol=1e-4)
+    got16 = ops.linear(xd, wd, None).cpu().double()
+    torch.testing.assert_close(got16, ref - b.double(), **_tol(torch.bfloat16))
+
+
 # ---- rotary encoding and cache write ----------------------------------------------------------------
 def test_rope_table(ops_for):
     ops = ops_for(torch.float32)
@@ -155,7 +177,7 @@ def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
     slots = torch.randperm(pages * bs, generator=g)[:tokens].to(torch.int32)
     slots[4] = -1  # writes nothing
     kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=dtype).cuda()
-    vp = kp.clone()
+    vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=dtype).cuda()
     dev = qkv.cuda().clone()
     ops.rope_kv_write(dev, (cos, sin, rotary), slots.cuda(), kp, vp, num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs)
     out = dev.cpu()
@@ -171,7 +193,7 @@ def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
     v_ref = qkv[:, (heads + kv_heads) * head_dim :].double().view(tokens, kv_heads, head_dim)
     tol = _tol(dtype)
     torch.testing.assert_close(out[:, : heads * head_dim].double().view(tokens, heads, head_dim), q_ref, **tol)
-    kc, vc = kp.cpu().double(), vp.cpu().double()
+    kc, vc = kp.cpu().double(), vp.cpu().double().transpose(2, 3)  # values are transposed inside a page
     written = torch.zeros(pages, bs, dtype=torch.bool)
     for t in range(tokens):
         s = int(slots[t])
@@ -197,7 +219,7 @@ def _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, seed, extra_pages
     width = max(need)
     table = torch.full((len(entries), width), -1, dtype=torch.int32)
     kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=dtype)
-    vp = kp.clone()
+    vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=dtype)  # transposed inside a page
     dense = []
     for r, (ctx_len, _) in enumerate(entries):
         ids = [perm.pop() for _ in range(need[r])]
@@ -208,7 +230,7 @@ def _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, seed, extra_pages
             k[1] *= 6.0  # a far key that must dominate when the query points at it
         for p in range(ctx_len):
             kp[ids[p // bs], :, p % bs] = k[p]
-            vp[ids[p // bs], :, p % bs] = v[p]
+            vp[ids[p // bs], :, :, p % bs] = v[p]
         dense.append((k.double(), v.double()))
     token_entry, positions = [], []
     for r, (ctx_len, q_len) in enumerate(entries):
@@ -223,14 +245,33 @@ def _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, seed, extra_pages
                 k1 = dense[r][0][1]  # [kv_heads, d]
                 rep = k1.repeat_interleave(heads // kv_heads, dim=0).reshape(-1)
                 q[t, : heads * head_dim] = (rep * 0.5).to(dtype)
-    ctx = SimpleNamespace(
+    ctx = _plan(entries, token_entry, positions)
+    return q, kp, vp, table, ctx, dense, token_entry, positions
+
+
+def _plan(entries, token_entry, positions):
+    """What the step function hands to the attention kernels about a batch."""
+    from mini_llm_runtime_amd.kernels.ops import query_tiles
+
+    q_lens = [ql for _, ql in entries]
+    cu = [0]
+    for n in q_lens:
+        cu.append(cu[-1] + n)
+    tiles = query_tiles(q_lens)
+    singles = [c for c, ql in entries if ql == 1]
+    return SimpleNamespace(
         num_entries=len(entries),
         token_entry=torch.tensor(token_entry, dtype=torch.int32).cuda(),
         positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+        cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
+        context_lens=torch.tensor([c for c, _ in entries], dtype=torch.int32).cuda(),
         max_context_len=max(c for c, _ in entries),
-        max_q_len=max(ql for _, ql in entries),
+        max_q_len=max(q_lens),
+        query_tiles=torch.from_numpy(tiles).cuda() if len(tiles) else None,
+        num_query_tiles=len(tiles),
+        num_decode_entries=len(singles),
+        max_decode_context=max(singles, default=0),
     )
-    return q, kp, vp, table, ctx, dense, token_entry, positions
 
 
 def _attention_reference(q, dense, token_entry, positions, heads, kv_heads, head_dim, scale, window):
@@ -307,21 +348,15 @@ def test_paged_attention_merge_needs_global_weights(ops_for):
     ops = ops_for(torch.float32)
     bs = 4
     kp = torch.zeros(2, 1, bs, 16)
-    vp = torch.zeros(2, 1, bs, 16)
+    vp = torch.zeros(2, 1, 16, bs)
     kp[0, 0, 0, 0] = 40.0
     kp[1, 0, 0, 0] = -40.0
-    vp[0, 0, 0] = 7.0
-    vp[1, 0, 0] = -3.0
+    vp[0, 0, :, 0] = 7.0
+    vp[1, 0, :, 0] = -3.0
     # context of 5 tokens: positions 0..3 in page 0 (1..3 neutral), position 4 in page 1
     q = torch.zeros(1, 16)
     q[0, 0] = 1.0
-    ctx = SimpleNamespace(
-        num_entries=1,
-        token_entry=torch.zeros(1, dtype=torch.int32).cuda(),
-        positions=torch.tensor([4], dtype=torch.int32).cuda(),
-        max_context_len=5,
-        max_q_len=1,
-    )
+    ctx = _plan([(5, 1)], [0], [4])
     table = torch.tensor([[0, 1]], dtype=torch.int32)
     got = ops.paged_attention(
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
@@ -356,6 +391,47 @@ def test_attention_matches_library_special_case(ops_for):
     qq = q[:, : heads * head_dim].double().view(n, heads, head_dim).transpose(0, 1)
     ref = torch.nn.functional.scaled_dot_product_attention(qq, k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
     torch.testing.assert_close(got.double(), ref.transpose(0, 1).reshape(n, -1), atol=2e-5, rtol=2e-5)
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim", ATTN_SHAPES + [(40, 2, 64), (2, 2, 256)])
+@pytest.mark.parametrize("partition", [64, 256, 4096])
+def test_decode_attention_partitions(ops_for, heads, kv_heads, head_dim, partition):
+    """The split-KV decode kernel with one, a few and many partitions, at context lengths around
+    page and tile edges (reference tests/test_split_kv_attention.py:37-59: 1, 15, 16, 17, 65, 2048, 2049),
+    against float64 and against the plain 32-bit kernel."""
+    ops = ops_for(torch.bfloat16)
+    old = ops.decode_partition
+    ops.decode_partition = partition
+    try:
+        entries = [(n, 1) for n in (1, 15, 16, 17, 65, 300, 2048, 2049)]
+        q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, 16, torch.bfloat16, 26)
+        scale = head_dim**-0.5
+        args = (q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx)
+        kw = dict(num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=16, scale=scale, window=None)
+        got = ops.paged_attention(*args, **kw).cpu()
+        fma = ops.paged_attention(*args, kernel="fma", **kw).cpu()
+    finally:
+        ops.decode_partition = old
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.double(), ref, **_tol(torch.bfloat16))
+    torch.testing.assert_close(got.double(), fma.double(), **_tol(torch.bfloat16))
+
+
+def test_prefill_attention_long_prompt_and_portion(ops_for):
+    """The tiled prefill kernel on a 2,048-token prompt and on a 300-token portion behind 1,500 cached tokens."""
+    ops = ops_for(torch.bfloat16)
+    heads, kv_heads, head_dim, bs = 14, 2, 64, 16
+    entries = [(2048, 2048), (1800, 300), (77, 77)]
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 27, spike=True)
+    scale = head_dim**-0.5
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
+    ).cpu()
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.double(), ref, **_tol(torch.bfloat16))
 
 
 # ---- sampling ---------------------------------------------------------------------------------------------
