@@ -54,13 +54,24 @@ int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, 
 // y[M, N] = x[M, K] * w[N, K]^T (+ bias[N]); x, w in `dtype`; bias float32 when
 // bias_is_f32 else `dtype` (null: none); y float32 when out_is_f32 else `dtype`.
 // Plain 32-bit FMA arithmetic on every path (no matrix-core rounding).
+// With `swiglu` the rows of w come in groups (gate 2j, gate 2j+1, up 2j, up 2j+1),
+// there is no bias, n is a multiple of 4 and y[M, N / 2] = silu(gate) * up.
 int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                    int out_is_f32, int dtype, int m, int n, int k, hipStream_t stream);
+                    int out_is_f32, int swiglu, int dtype, int m, int n, int k, hipStream_t stream);
 
 // The same product in bfloat16 on the matrix cores (float32 accumulation).  Needs
 // k % 8 == 0 and 16-byte aligned x and w; any m and n.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                  int out_is_f32, int m, int n, int k, hipStream_t stream);
+                  int out_is_f32, int swiglu, int m, int n, int k, hipStream_t stream);
+
+// mlr_gemm_bf16 with the RMSNorm of its input fused in, for up to 64 tokens: the
+// input is norm(x + delta) with x float32 [m, k], delta bfloat16 (may be null) and
+// norm weight [k] (float32 when norm_weight_is_f32, else bfloat16); x + delta is
+// written to x_out (float32 [m, k]; may be null; must not alias x).
+int mlr_gemm_bf16_norm(const float* x, const void* delta, const void* norm_weight,
+                       int norm_weight_is_f32, float eps, float* x_out, const void* w,
+                       const void* bias, int bias_is_f32, void* y, int out_is_f32, int swiglu, int m,
+                       int n, int k, hipStream_t stream);
 
 // Attention of every token over its request's pages: token t (entry
 // token_entry[t], absolute position positions[t]) sees the keys
@@ -77,8 +88,10 @@ int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_
 
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
 // the first index whose cumulative exp((x - max) / temperature) exceeds
-// uniform[k] * total.  temperature and uniform may be null (all greedy).
+// uniform[k] * total.  temperature and uniform may be null (all greedy).  `scratch`
+// holds mlr_sample_scratch(rows, vocab) floats.
+int64_t mlr_sample_scratch(int rows, int vocab);
 int mlr_sample(const float* logits, const float* temperature, const float* uniform, int* tokens,
-               int rows, int vocab, hipStream_t stream);
+               float* scratch, int rows, int vocab, hipStream_t stream);
 
 }  // extern "C"

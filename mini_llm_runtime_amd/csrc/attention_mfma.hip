@@ -37,8 +37,11 @@ namespace mlr {
 
 constexpr int D = MLR_HEAD_DIM;
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 within 16..256");
-constexpr int kSteps32 = D / 32;       // full 16x16x32 steps over the head dims
-constexpr bool kTail16 = (D % 32) != 0;  // one 16x16x16 step for the last 16 dims
+// The score product runs over the head dims in 16x16x32 steps.  When D is an odd
+// multiple of 16 the last step covers 16 dims only: lanes of quarters 2 and 3 (k 16..31
+// of that step) feed zeros on both sides.
+constexpr int kSteps = (D + 31) / 32;
+constexpr bool kHalfLast = (D % 32) != 0;
 constexpr int kDimTiles = D / 16;
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -56,36 +59,27 @@ __device__ __forceinline__ s16x4_t pack_bf16x4(float a, float b, float c, float 
   return r;
 }
 
-// The query operand of one row: D dims as 16-byte chunks (and an 8-byte tail).
-struct QueryOperand {
-  bf16x8_t full[kSteps32 > 0 ? kSteps32 : 1];
-  s16x4_t tail;
+// One row of D dims (a query, or a key) as the operand chunks of the score product.
+struct RowOperand {
+  bf16x8_t step[kSteps];
 };
 
-__device__ __forceinline__ QueryOperand load_query(const bf16* row, bool valid, int quarter) {
-  QueryOperand q;
+// `row` points at dim 0 of this lane's row, in global memory or LDS.
+__device__ __forceinline__ RowOperand load_row(const bf16* row, bool valid, int quarter) {
+  RowOperand r;
 #pragma unroll
-  for (int s = 0; s < kSteps32; ++s)
-    q.full[s] = valid ? load_bf16x8(row + s * 32 + quarter * 8) : zero_bf16x8();
-  q.tail = s16x4_t{0, 0, 0, 0};
-  if (kTail16 && valid) q.tail = *reinterpret_cast<const s16x4_t*>(row + kSteps32 * 32 + quarter * 4);
-  return q;
+  for (int s = 0; s < kSteps; ++s) {
+    const bool inside = valid && !(kHalfLast && s == kSteps - 1 && quarter >= 2);
+    r.step[s] = inside ? load_bf16x8(row + s * 32 + quarter * 8) : zero_bf16x8();
+  }
+  return r;
 }
 
-// S^T tile [16 keys x 16 rows]: `krow` points at this lane's key row (dim 0), in
-// global memory or LDS.
-__device__ __forceinline__ f32x4_t score_tile(const bf16* krow, bool valid, const QueryOperand& q, int quarter) {
+// S^T tile [16 keys x 16 rows].
+__device__ __forceinline__ f32x4_t score_tile(const RowOperand& k, const RowOperand& q) {
   f32x4_t s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int st = 0; st < kSteps32; ++st) {
-    const bf16x8_t a = valid ? load_bf16x8(krow + st * 32 + quarter * 8) : zero_bf16x8();
-    s = mfma_16x16x32(a, q.full[st], s);
-  }
-  if (kTail16) {
-    s16x4_t a = {0, 0, 0, 0};
-    if (valid) a = *reinterpret_cast<const s16x4_t*>(krow + kSteps32 * 32 + quarter * 4);
-    s = mfma_16x16x16(a, q.tail, s);
-  }
+  for (int st = 0; st < kSteps; ++st) s = mfma_16x16x32(k.step[st], q.step[st], s);
   return s;
 }
 
@@ -126,6 +120,59 @@ __device__ __forceinline__ s16x4_t softmax_tile(Softmax& st, f32x4_t s, const bo
 constexpr int kDecodeWaves = D > 128 ? 2 : 4;  // bounded by the LDS the merge needs
 constexpr int kPartialStride = D + 2;  // numerator[D], max, denominator
 
+// Operands of one 16-key tile, loaded ahead of their use.
+struct DecodeTile {
+  RowOperand k;
+  s16x4_t v[kDimTiles];
+  bool bad;
+};
+
+__device__ __forceinline__ DecodeTile load_decode_tile(const bf16* __restrict__ key_pages,
+                                                       const bf16* __restrict__ value_pages,
+                                                       const int* __restrict__ table, int ts, int ke, int first,
+                                                       int kvh, int kv_heads, int block_size, int num_pages,
+                                                       int col, int quarter) {
+  DecodeTile t;
+  t.bad = false;
+  // key operand: this lane's row is key ts + col
+  const int key_a = ts + col;
+  bool valid_a = key_a < ke;
+  const bf16* krow = key_pages;
+  if (valid_a) {
+    const int logical = key_a / block_size;
+    const int page = table[logical];
+    if (page < 0 || page >= num_pages) {
+      t.bad = key_a >= first;
+      valid_a = false;
+    } else {
+      krow = key_pages +
+             ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size + (key_a - logical * block_size)) * D;
+    }
+  }
+  t.k = load_row(krow, valid_a, quarter);
+  // value operand: this lane's 4 keys are ts + quarter * 4 .. + 3, inside one page
+  const int key_v = ts + quarter * 4;
+  bool valid_v = key_v < ke;
+  const bf16* vbase = value_pages;
+  if (valid_v) {
+    const int logical = key_v / block_size;
+    const int page = table[logical];
+    if (page < 0 || page >= num_pages) {
+      valid_v = false;
+    } else {
+      vbase = value_pages + (static_cast<int64_t>(page) * kv_heads + kvh) * D * block_size +
+              (key_v - logical * block_size);
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < kDimTiles; ++dt) {
+    t.v[dt] = s16x4_t{0, 0, 0, 0};
+    if (valid_v)
+      t.v[dt] = *reinterpret_cast<const s16x4_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size);
+  }
+  return t;
+}
+
 __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
@@ -164,8 +211,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   if (tid == 0) sm_bad = 0;
   __syncthreads();
 
-  const QueryOperand qo =
-      load_query(q + t * q_stride + static_cast<int64_t>(head_ok ? head : 0) * D, head_ok, quarter);
+  const RowOperand qo =
+      load_row(q + t * q_stride + static_cast<int64_t>(head_ok ? head : 0) * D, head_ok, quarter);
 
   Softmax sm{-INFINITY, 0.f};
   f32x4_t acc[kDimTiles];
@@ -173,52 +220,28 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   bool bad = false;
 
-  for (int ts = kb + wave * 16; ts < ke; ts += kDecodeWaves * 16) {
-    // key operand: this lane's row is key ts + col
-    const int key_a = ts + col;
-    bool valid_a = key_a < ke;
-    const bf16* krow = key_pages;
-    if (valid_a) {
-      const int logical = key_a / block_size;
-      const int page = table[logical];
-      if (page < 0 || page >= num_pages) {
-        bad = bad || key_a >= first;
-        valid_a = false;
-      } else {
-        krow = key_pages +
-               ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size + (key_a - logical * block_size)) * D;
-      }
-    }
-    // value operand: this lane's 4 keys are ts + quarter * 4 .. + 3, inside one page
-    const int key_v = ts + quarter * 4;
-    bool valid_v = key_v < ke;
-    const bf16* vbase = value_pages;
-    if (valid_v) {
-      const int logical = key_v / block_size;
-      const int page = table[logical];
-      if (page < 0 || page >= num_pages) {
-        valid_v = false;
-      } else {
-        vbase = value_pages + (static_cast<int64_t>(page) * kv_heads + kvh) * D * block_size +
-                (key_v - logical * block_size);
-      }
-    }
-    s16x4_t vt[kDimTiles];
-#pragma unroll
-    for (int dt = 0; dt < kDimTiles; ++dt) {
-      vt[dt] = s16x4_t{0, 0, 0, 0};
-      if (valid_v) vt[dt] = *reinterpret_cast<const s16x4_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size);
-    }
-
-    const f32x4_t s = score_tile(krow, valid_a, qo, quarter);
+  constexpr int kStride = kDecodeWaves * 16;
+  int ts = kb + wave * 16;
+  DecodeTile cur;
+  if (ts < ke)
+    cur = load_decode_tile(key_pages, value_pages, table, ts, ke, first, kvh, kv_heads, block_size, num_pages, col,
+                           quarter);
+  while (ts < ke) {
+    DecodeTile nxt;
+    const bool more = ts + kStride < ke;
+    if (more)  // the next tile's loads are in flight while this one is computed
+      nxt = load_decode_tile(key_pages, value_pages, table, ts + kStride, ke, first, kvh, kv_heads, block_size,
+                             num_pages, col, quarter);
+    bad = bad || cur.bad;
+    const f32x4_t s = score_tile(cur.k, qo);
     bool ok[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = key_v + i;
+      const int key = ts + quarter * 4 + i;
       ok[i] = key >= first && key < ke;
       if (!ok[i]) {
 #pragma unroll
-        for (int dt = 0; dt < kDimTiles; ++dt) vt[dt][i] = 0;  // unwritten slots may hold NaN
+        for (int dt = 0; dt < kDimTiles; ++dt) cur.v[dt][i] = 0;  // unwritten slots may hold NaN
       }
     }
     float alpha;
@@ -227,8 +250,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     for (int dt = 0; dt < kDimTiles; ++dt) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
-      acc[dt] = mfma_16x16x16(vt[dt], pb, acc[dt]);
+      acc[dt] = mfma_16x16x16(cur.v[dt], pb, acc[dt]);
     }
+    if (more) cur = nxt;
+    ts += kStride;
   }
 
   // the column's sum is spread over the four lanes that share it
@@ -245,12 +270,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     for (int i = 0; i < 4; ++i) sm_acc[wave][col][dt * 16 + quarter * 4 + i] = acc[dt][i];
   __syncthreads();
 
+  // merge the wavefronts; with one partition this is the result
   const bool poisoned = sm_bad != 0;
-  for (int idx = tid; idx < 16 * D; idx += kDecodeWaves * kWave) {
+  const int tile_heads = min(16, group - htile * 16);
+  for (int idx = tid; idx < tile_heads * D; idx += kDecodeWaves * kWave) {
     const int c = idx / D;
     const int d = idx - c * D;
-    const int hig = htile * 16 + c;
-    if (hig >= group) continue;
     float mstar = -INFINITY;
 #pragma unroll
     for (int w = 0; w < kDecodeWaves; ++w) mstar = fmaxf(mstar, sm_m[w][c]);
@@ -261,7 +286,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
       num += wgt * sm_acc[w][c][d];
       den += wgt * sm_l[w][c];
     }
-    const int h = kvh * group + hig;
+    const int h = kvh * group + htile * 16 + c;
     if (splits == 1) {
       const float v = poisoned ? __builtin_nanf("") : num / den;
       out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(v);
@@ -276,28 +301,50 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   }
 }
 
+// Merge of the partitions of one (entry, query head): m = max m_j, w_j = exp(m_j - m),
+// O = sum w_j a_j / sum w_j l_j (csrc/paged_attention_split_cuda.cu:66-88 of the
+// reference).  Lane j holds partition j's max and sum, so the weights come from two
+// wavefront reductions; every lane then sums its output dims over the partitions
+// with independent loads.
 __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* __restrict__ partial,
                                                                   const int* __restrict__ cu_q,
                                                                   bf16* __restrict__ out, int heads, int splits) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
+  const int lane = threadIdx.x;
   const int t = cu_q[entry];
   if (cu_q[entry + 1] - t != 1) return;
   const float* src = partial + (static_cast<int64_t>(entry) * heads + h) * splits * kPartialStride;
   float mstar = -INFINITY;
-  for (int s = 0; s < splits; ++s) mstar = fmaxf(mstar, src[s * kPartialStride + D]);
   float den = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ms = src[s * kPartialStride + D];
-    if (ms != -INFINITY) den += __expf(ms - mstar) * src[s * kPartialStride + D + 1];
+  // more than 64 partitions: several rounds of the same two reductions
+  for (int s0 = 0; s0 < splits; s0 += kWave) {
+    const int sp = s0 + lane;
+    const float ms = sp < splits ? src[sp * kPartialStride + D] : -INFINITY;
+    const float ls = sp < splits ? src[sp * kPartialStride + D + 1] : 0.f;
+    const float round_max = wave_max(ms);
+    const float m_new = fmaxf(mstar, round_max);
+    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m_new);
+    const float rescale = (mstar == -INFINITY) ? 0.f : __expf(mstar - m_new);
+    den = den * rescale + wave_sum(w * ls);
+    mstar = m_new;
   }
-  for (int d = threadIdx.x; d < D; d += kWave) {
-    float num = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = src[s * kPartialStride + D];
-      if (ms != -INFINITY) num += __expf(ms - mstar) * src[s * kPartialStride + d];
+  float num[(D + kWave - 1) / kWave];
+#pragma unroll
+  for (int j = 0; j < (D + kWave - 1) / kWave; ++j) num[j] = 0.f;
+  for (int sp = 0; sp < splits; ++sp) {
+    const float ms = src[sp * kPartialStride + D];
+    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - mstar);
+#pragma unroll
+    for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
+      const int d = lane + j * kWave;
+      if (d < D) num[j] += w * src[sp * kPartialStride + d];
     }
-    out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(num / den);
+  }
+#pragma unroll
+  for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
+    const int d = lane + j * kWave;
+    if (d < D) out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(num[j] / den);
   }
 }
 
@@ -339,7 +386,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const bool q_ok = qi < q_len;
   const int pq = pos0 + qi;  // its absolute position
   const int pq_first = window > 0 ? max(0, pq - window + 1) : 0;
-  const QueryOperand qo = load_query(
+  const RowOperand qo = load_row(
       q + static_cast<int64_t>(t_first + (q_ok ? qi : 0)) * q_stride + static_cast<int64_t>(head) * D, q_ok, quarter);
 
   // key range of the workgroup: from the first query's window start to the last query's position
@@ -410,7 +457,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int sub = 0; sub < kTileK / 16; ++sub) {
       const int ts = kt0 + sub * 16;
       if (ts > w_last || ts + 15 < w_first) continue;  // nothing visible to this wavefront
-      const f32x4_t s = score_tile(ks + (sub * 16 + col) * kKLd, true, qo, quarter);
+      const f32x4_t s = score_tile(load_row(ks + (sub * 16 + col) * kKLd, true, quarter), qo);
       bool ok[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {

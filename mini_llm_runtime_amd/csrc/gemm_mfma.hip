@@ -16,6 +16,18 @@
 //    K in slices of 64 staged through double-buffered LDS, four wavefronts of
 //    64 x 64 each, 32x32x16 MFMA.
 // K must be a multiple of 8 (16-byte rows); other shapes take the FMA kernel.
+//
+// Fusions (they save whole kernels in a decode step, which is a chain of very
+// short ones):
+//  * norm prologue (skinny only): the input is the float32 residual stream plus
+//    a not-yet-added delta; the kernel adds them, writes the sum out once,
+//    multiplies by the norm weight while building its operand, collects the sum
+//    of squares on the way and scales the finished sums by rsqrt(mean + eps).
+//    RMSNorm commutes with the product because its statistic is one scalar per
+//    token (formula: src/mini_llm_runtime/qwen_model_runner.py:22-26).
+//  * SwiGLU epilogue: with gate and up rows interleaved in pairs
+//    (g0 g1 u0 u1 g2 g3 u2 u3 ...) a lane holds two gate sums and their two up
+//    sums and stores silu(gate) * up (qwen_model_runner.py:215-216) directly.
 #include "api.h"
 #include "common.h"
 #include "mfma.h"
@@ -27,12 +39,40 @@ struct GemmEpilogue {
   int bias_is_f32;
   void* y;
   int out_is_f32;
+  int swiglu;  // store silu(v0) * v2, silu(v1) * v3 into a row of N / 2
 };
 
-// Store four consecutive output features n..n+3 of token m.
+struct NormPrologue {
+  const float* x;      // residual stream [M, K]
+  const bf16* delta;   // not-yet-added delta [M, K], may be null
+  const void* weight;  // norm weight [K]
+  int weight_is_f32;
+  float* x_out;        // x + delta [M, K], may be null
+  float eps;
+};
+
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+// Store four consecutive output features n..n+3 of token m (n is a multiple of 4).
 __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n, int N, float v0, float v1,
                                        float v2, float v3) {
   float v[4] = {v0, v1, v2, v3};
+  if (ep.swiglu) {
+    // n..n+3 = gate 2j, gate 2j+1, up 2j, up 2j+1 with j = n / 4; N is a multiple of 4
+    const int64_t at = m * (N / 2) + n / 2;
+    const float a = silu(v[0]) * v[2];
+    const float b = silu(v[1]) * v[3];
+    if (ep.out_is_f32) {
+      float* y = static_cast<float*>(ep.y) + at;
+      y[0] = a;
+      y[1] = b;
+    } else {
+      const uint32_t packed =
+          static_cast<uint32_t>(f32_to_bf16(a).bits) | (static_cast<uint32_t>(f32_to_bf16(b).bits) << 16);
+      *reinterpret_cast<uint32_t*>(static_cast<bf16*>(ep.y) + at) = packed;
+    }
+    return;
+  }
   if (ep.bias != nullptr) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -62,13 +102,53 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
   }
 }
 
+// Eight consecutive elements of the normed-but-not-yet-scaled input of token row
+// `m` at chunk c: (x + delta) * weight, rounded to bfloat16; adds their squares
+// to `ssq` and, when asked, writes x + delta out.
+__device__ __forceinline__ bf16x8_t norm_chunk(const NormPrologue& np, int64_t row_offset, int c, bool write_out,
+                                               float& ssq) {
+  const f32x4_t* xp = reinterpret_cast<const f32x4_t*>(np.x + row_offset) + 2 * c;
+  f32x4_t lo = xp[0];
+  f32x4_t hi = xp[1];
+  float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  if (np.delta != nullptr) {
+    const u16x8_t d = *(reinterpret_cast<const u16x8_t*>(np.delta + row_offset) + c);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] += to_f32(bf16{d[i]});
+  }
+  if (write_out) {
+    f32x4_t* op = reinterpret_cast<f32x4_t*>(np.x_out + row_offset) + 2 * c;
+    op[0] = f32x4_t{v[0], v[1], v[2], v[3]};
+    op[1] = f32x4_t{v[4], v[5], v[6], v[7]};
+  }
+  float w[8];
+  if (np.weight_is_f32) {
+    const f32x4_t* wp = reinterpret_cast<const f32x4_t*>(np.weight) + 2 * c;
+    const f32x4_t a = wp[0], b = wp[1];
+    w[0] = a[0]; w[1] = a[1]; w[2] = a[2]; w[3] = a[3];
+    w[4] = b[0]; w[5] = b[1]; w[6] = b[2]; w[7] = b[3];
+  } else {
+    const u16x8_t ww = *(reinterpret_cast<const u16x8_t*>(np.weight) + c);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = to_f32(bf16{ww[i]});
+  }
+  u16x8_t out;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    ssq += v[i] * v[i];
+    out[i] = f32_to_bf16(v[i] * w[i]).bits;
+  }
+  return __builtin_bit_cast(bf16x8_t, out);
+}
+
 // ---- skinny: M <= 16 * MT ---------------------------------------------------------------
-template <int MT, int WAVES>
+template <int MT, int WAVES, bool NORM>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
-                                                                 const bf16* __restrict__ w, GemmEpilogue ep,
-                                                                 int M, int N, int K) {
-  constexpr int U = 4;  // k-steps in flight per wavefront
+                                                                 const bf16* __restrict__ w, NormPrologue np,
+                                                                 GemmEpilogue ep, int M, int N, int K) {
+  constexpr int U = NORM ? 4 : 8;  // k-steps in flight per wavefront
   __shared__ float red[WAVES][MT][kWave][4];
+  __shared__ float red_ssq[NORM ? WAVES : 1][MT][16];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int r = lane % 16;
@@ -79,46 +159,74 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   const int ksteps = (chunks + 3) / 4;  // one MFMA consumes 4 chunks (32 elements of k)
   const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(wrow) * K);
   const bf16x8_t* xp[MT];
+  int64_t xoff[MT];
   bool xok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
     xok[mt] = m < M;
-    xp[mt] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(m, M - 1)) * K);
+    xoff[mt] = static_cast<int64_t>(min(m, M - 1)) * K;
+    xp[mt] = NORM ? nullptr : reinterpret_cast<const bf16x8_t*>(x + xoff[mt]);
   }
+  const bool write_out = NORM && np.x_out != nullptr && blockIdx.x == 0;
   f32x4_t acc[MT];
+  float ssq[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt) {
+    acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    ssq[mt] = 0.f;
+  }
 
   for (int s0 = wave; s0 < ksteps; s0 += WAVES * U) {
     bf16x8_t a[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int c = (s0 + u * WAVES) * 4 + q;
-      a[u] = c < chunks ? wp[c] : zero_bf16x8();
+      a[u] = c < chunks ? __builtin_nontemporal_load(wp + c) : zero_bf16x8();
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int c = (s0 + u * WAVES) * 4 + q;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8_t b = (xok[mt] && c < chunks) ? xp[mt][c] : zero_bf16x8();
+        bf16x8_t b = zero_bf16x8();
+        if (xok[mt] && c < chunks) {
+          if (NORM)
+            b = norm_chunk(np, xoff[mt], c, write_out, ssq[mt]);
+          else
+            b = xp[mt][c];
+        }
         acc[mt] = mfma_16x16x32(a[u], b, acc[mt]);
       }
     }
   }
 
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][mt][lane][i] = acc[mt][i];
+    if (NORM) {
+      float s = ssq[mt];
+      s += __shfl_xor(s, 16, kWave);
+      s += __shfl_xor(s, 32, kWave);
+      if (q == 0) red_ssq[wave][mt][r] = s;
+    }
+  }
   __syncthreads();
+  // wavefront w < MT finishes token tile w (MT <= WAVES)
   if (wave < MT) {
     const int mt = wave;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] += red[ww][mt][lane][i];
+    if (NORM) {
+      float total = 0.f;
+      for (int ww = 0; ww < WAVES; ++ww) total += red_ssq[ww][mt][r];
+      const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + np.eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= inv;
+    }
     const int m = mt * 16 + r;
     const int n = n0 + q * 4;
     if (m < M && n < N) store4(ep, m, n, N, v[0], v[1], v[2], v[3]);
@@ -236,51 +344,97 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 }
 
 template <int MT, int WAVES>
-static void launch_skinny(const bf16* x, const bf16* w, const GemmEpilogue& ep, int m, int n, int k,
-                          hipStream_t stream) {
-  gemm_skinny_kernel<MT, WAVES><<<(n + 15) / 16, WAVES * 64, 0, stream>>>(x, w, ep, m, n, k);
+static void launch_skinny(const bf16* x, const bf16* w, const NormPrologue* np, const GemmEpilogue& ep, int m,
+                          int n, int k, hipStream_t stream) {
+  const unsigned grid = (n + 15) / 16;
+  if (np != nullptr)
+    gemm_skinny_kernel<MT, WAVES, true><<<grid, WAVES * 64, 0, stream>>>(x, w, *np, ep, m, n, k);
+  else
+    gemm_skinny_kernel<MT, WAVES, false><<<grid, WAVES * 64, 0, stream>>>(x, w, NormPrologue{}, ep, m, n, k);
 }
 
-}  // namespace mlr
-
-using namespace mlr;
-
-// y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
-// argument meanings.  Requires k % 8 == 0 and 16-byte aligned x and w.
-extern "C" int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                             int out_is_f32, int m, int n, int k, hipStream_t stream) {
-  MLR_REQUIRE(x && w && y, "null pointer");
-  MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
-  MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
-  MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
-              "x and w must be 16-byte aligned");
-  const bf16* xb = static_cast<const bf16*>(x);
-  const bf16* wb = static_cast<const bf16*>(w);
-  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32};
+static int gemm_bf16(const bf16* xb, const bf16* wb, const NormPrologue* np, const GemmEpilogue& ep, int m, int n,
+                     int k, hipStream_t stream) {
   if (m <= 64) {
     const bool deep = k >= 2048;
     if (m <= 16) {
-      if (deep) launch_skinny<1, 8>(xb, wb, ep, m, n, k, stream);
-      else launch_skinny<1, 4>(xb, wb, ep, m, n, k, stream);
+      if (deep) launch_skinny<1, 16>(xb, wb, np, ep, m, n, k, stream);
+      else launch_skinny<1, 4>(xb, wb, np, ep, m, n, k, stream);
     } else if (m <= 32) {
-      if (deep) launch_skinny<2, 8>(xb, wb, ep, m, n, k, stream);
-      else launch_skinny<2, 4>(xb, wb, ep, m, n, k, stream);
+      if (deep) launch_skinny<2, 8>(xb, wb, np, ep, m, n, k, stream);
+      else launch_skinny<2, 4>(xb, wb, np, ep, m, n, k, stream);
     } else {
-      if (deep) launch_skinny<4, 8>(xb, wb, ep, m, n, k, stream);
-      else launch_skinny<4, 4>(xb, wb, ep, m, n, k, stream);
+      if (deep) launch_skinny<4, 8>(xb, wb, np, ep, m, n, k, stream);
+      else launch_skinny<4, 4>(xb, wb, np, ep, m, n, k, stream);
     }
   } else {
     static bool configured = false;
     if (!configured) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, kTiledLds);
-      MLR_REQUIRE(e == hipSuccess, std::string("cannot raise the LDS limit: ") + hipGetErrorString(e));
+      if (e != hipSuccess) {
+        set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
+        return -1;
+      }
       configured = true;
     }
     dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
-    MLR_REQUIRE(grid.y < 65536u, "too many rows for one launch");
+    if (grid.y >= 65536u) {
+      set_error("mlr_gemm_bf16: too many rows for one launch");
+      return -1;
+    }
     gemm_tiled_kernel<<<grid, 256, kTiledLds, stream>>>(xb, wb, ep, m, n, k);
   }
+  return 0;
+}
+
+}  // namespace mlr
+
+using namespace mlr;
+
+extern "C" {
+
+// y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
+// argument meanings.  Requires k % 8 == 0 and 16-byte aligned x and w.  With
+// `swiglu` the rows of w are (gate, gate, up, up) groups, there is no bias, n is
+// a multiple of 4 and y is [m, n / 2].
+int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
+                  int swiglu, int m, int n, int k, hipStream_t stream) {
+  MLR_REQUIRE(x && w && y, "null pointer");
+  MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
+  MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
+  MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
+  MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
+              "x and w must be 16-byte aligned");
+  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
+  if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), nullptr, ep, m, n, k, stream) != 0)
+    return -1;
   MLR_LAUNCH_CHECK();
   return 0;
 }
+
+// The same product with the RMSNorm of its input fused in, for up to 64 tokens:
+// input = norm(x + delta) with x float32 [m, k], delta bfloat16 (may be null),
+// norm weight [k] (float32 when norm_weight_is_f32, else bfloat16); x + delta is
+// written to x_out (float32 [m, k], may be null; must not alias x).
+int mlr_gemm_bf16_norm(const float* x, const void* delta, const void* norm_weight, int norm_weight_is_f32,
+                       float eps, float* x_out, const void* w, const void* bias, int bias_is_f32, void* y,
+                       int out_is_f32, int swiglu, int m, int n, int k, hipStream_t stream) {
+  MLR_REQUIRE(x && norm_weight && w && y, "null pointer");
+  MLR_REQUIRE(m > 0 && m <= 64 && n > 0 && k > 0, "sizes must be > 0 and m <= 64");
+  MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
+  MLR_REQUIRE(eps >= 0.f, "eps must be >= 0");
+  MLR_REQUIRE(x_out != x, "x_out must not alias x");
+  MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
+  MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(norm_weight) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(x_out) % 16 == 0,
+              "operands must be 16-byte aligned");
+  NormPrologue np{x, static_cast<const bf16*>(delta), norm_weight, norm_weight_is_f32, x_out, eps};
+  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
+  if (gemm_bf16(nullptr, static_cast<const bf16*>(w), &np, ep, m, n, k, stream) != 0) return -1;
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -18,8 +18,8 @@ constexpr int kTK = 16;
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const void* __restrict__ bias, int bias_is_f32,
-                                                          void* __restrict__ y, int out_is_f32, int M, int N,
-                                                          int K) {
+                                                          void* __restrict__ y, int out_is_f32, int swiglu,
+                                                          int M, int N, int K) {
   __shared__ float xs[kTK][kTM + 4];
   __shared__ float ws[kTK][kTN + 4];
   const int tid = threadIdx.x;
@@ -66,6 +66,23 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
   for (int i = 0; i < 4; ++i) {
     const int64_t gm = m0 + tm * 4 + i;
     if (gm >= M) continue;
+    if (swiglu) {
+      // columns n..n+3 = gate 2j, gate 2j+1, up 2j, up 2j+1 (rows of w interleaved in pairs);
+      // qwen_model_runner.py:215-216: silu(gate) * up
+      const int64_t gn = n0 + tn * 4;
+      if (gn >= N) continue;
+      const int64_t at = gm * (N / 2) + gn / 2;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float g = acc[i][j];
+        const float v = g / (1.0f + expf(-g)) * acc[i][j + 2];
+        if (out_is_f32)
+          static_cast<float*>(y)[at + j] = v;
+        else
+          static_cast<T*>(y)[at + j] = from_f32<T>(v);
+      }
+      continue;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t gn = n0 + tn * 4 + j;
@@ -85,21 +102,22 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 using namespace mlr;
 
 extern "C" int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                               int out_is_f32, int dtype, int m, int n, int k, hipStream_t stream) {
+                               int out_is_f32, int swiglu, int dtype, int m, int n, int k, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   MLR_REQUIRE(dtype == kBF16 || (out_is_f32 && (bias == nullptr || bias_is_f32)),
               "a float32 product has float32 bias and output");
+  MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
   dim3 grid((n + kTN - 1) / kTN, (m + kTM - 1) / kTM);
   MLR_REQUIRE(grid.y < 65536u, "too many rows for one launch");
   if (dtype == kF32)
     gemm_simple_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x),
                                                         static_cast<const float*>(w), bias, bias_is_f32, y,
-                                                        out_is_f32, m, n, k);
+                                                        out_is_f32, swiglu, m, n, k);
   else
     gemm_simple_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w),
-                                                       bias, bias_is_f32, y, out_is_f32, m, n, k);
+                                                       bias, bias_is_f32, y, out_is_f32, swiglu, m, n, k);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -2,39 +2,41 @@
 // src/mini_llm_runtime/engine.py:222) and temperature sampling by inverse CDF.
 // The reference samples greedily only; temperature is this engine's addition.
 //
-// One workgroup per row.  Every lane owns one contiguous chunk of the vocabulary,
-// so the cumulative sums are taken in index order and the result for a given
-// uniform number does not depend on what else is in the batch.
+// Two kernels.  sample_partial: one workgroup per (row, segment of 4,096 vocabulary
+// entries) reads its segment once, coalesced, and leaves (max, first index of the
+// max, sum of exp((x - max) / T)).  sample_final: one workgroup per row combines
+// the segments; for a sampled row it finds the segment in which the cumulative
+// sum passes uniform * total, then the 16-entry chunk, then the entry, always in
+// index order.  The draw for a given uniform number therefore depends on the row's
+// logits only, never on what else is in the batch.
 #include "api.h"
 #include "common.h"
 
 namespace mlr {
 
+constexpr int kSegment = 4096;
 constexpr int kSampleThreads = 256;
+constexpr int kChunk = kSegment / kSampleThreads;  // 16 consecutive entries per thread in the final scan
 
-__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits,
-                                                                const float* __restrict__ temperature,
-                                                                const float* __restrict__ uniform,
-                                                                int* __restrict__ tokens, int vocab) {
+__global__ __launch_bounds__(kSampleThreads) void sample_partial_kernel(const float* __restrict__ logits,
+                                                                        const float* __restrict__ temperature,
+                                                                        float* __restrict__ partial, int vocab,
+                                                                        int segments) {
   __shared__ float s_val[kSampleThreads];
   __shared__ int s_idx[kSampleThreads];
-  __shared__ float s_part[kSampleThreads];
-  __shared__ int s_pick;
-  __shared__ float s_before;
-  __shared__ float s_target;
-
+  __shared__ float scratch[16];
   const int row = blockIdx.x;
+  const int seg = blockIdx.y;
   const int tid = threadIdx.x;
   const float* z = logits + static_cast<int64_t>(row) * vocab;
-  const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
-  const int begin = min(vocab, tid * chunk);
-  const int end = min(vocab, begin + chunk);
+  const int begin = seg * kSegment;
+  const int end = min(vocab, begin + kSegment);
 
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = begin; i < end; ++i) {
+  for (int i = begin + tid; i < end; i += kSampleThreads) {
     const float v = z[i];
-    if (v > best || best_i == 0x7fffffff) {
+    if (best_i == 0x7fffffff || v > best) {  // i grows, so '>' keeps the first maximum
       best = v;
       best_i = i;
     }
@@ -46,8 +48,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
     if (tid < step) {
       const float ov = s_val[tid + step];
       const int oi = s_idx[tid + step];
-      // chunks are in index order, so on a tie the lower thread already holds the lower index
-      if (oi != 0x7fffffff && (s_idx[tid] == 0x7fffffff || ov > s_val[tid])) {
+      const float mv = s_val[tid];
+      const int mi = s_idx[tid];
+      if (oi != 0x7fffffff && (mi == 0x7fffffff || ov > mv || (ov == mv && oi < mi))) {
         s_val[tid] = ov;
         s_idx[tid] = oi;
       }
@@ -56,51 +59,123 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   }
   const float zmax = s_val[0];
   const int arg = s_idx[0];
+  float total = 0.f;
   const float temp = temperature != nullptr ? temperature[row] : 0.f;
-  if (!(temp > 0.f)) {
-    if (tid == 0) tokens[row] = arg;
-    return;
+  if (temp > 0.f) {
+    const float inv_t = 1.0f / temp;
+    float part = 0.f;
+    for (int i = begin + tid; i < end; i += kSampleThreads) part += expf((z[i] - zmax) * inv_t);
+    total = block_sum(part, scratch);
   }
+  if (tid == 0) {
+    float* dst = partial + (static_cast<int64_t>(row) * segments + seg) * 3;
+    dst[0] = zmax;
+    dst[1] = __int_as_float(arg);
+    dst[2] = total;
+  }
+}
 
-  const float inv_t = 1.0f / temp;
+__global__ __launch_bounds__(kSampleThreads) void sample_final_kernel(const float* __restrict__ logits,
+                                                                      const float* __restrict__ temperature,
+                                                                      const float* __restrict__ uniform,
+                                                                      const float* __restrict__ partial,
+                                                                      int* __restrict__ tokens, int vocab,
+                                                                      int segments) {
+  __shared__ float s_part[kSampleThreads];
+  __shared__ int s_seg;
+  __shared__ int s_pick;
+  __shared__ float s_before;
+  __shared__ float s_target;
+  __shared__ float s_max;
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* src = partial + static_cast<int64_t>(row) * segments * 3;
+  const float temp = temperature != nullptr ? temperature[row] : 0.f;
+  const float inv_t = temp > 0.f ? 1.0f / temp : 0.f;
+
+  if (tid == 0) {
+    float zmax = -INFINITY;
+    int arg = 0;
+    for (int s = 0; s < segments; ++s) {
+      const float m = src[3 * s];
+      if (s == 0 || m > zmax) {  // segments are in index order: '>' keeps the first maximum
+        zmax = m;
+        arg = __float_as_int(src[3 * s + 1]);
+      }
+    }
+    s_max = zmax;
+    s_seg = -1;
+    if (!(temp > 0.f)) {
+      tokens[row] = arg;
+    } else {
+      float total = 0.f;
+      for (int s = 0; s < segments; ++s) total += src[3 * s + 2] * expf((src[3 * s] - zmax) * inv_t);
+      const float target = uniform[row] * total;
+      float before = 0.f;
+      int pick = -1;
+      for (int s = 0; s < segments; ++s) {
+        const float w = src[3 * s + 2] * expf((src[3 * s] - zmax) * inv_t);
+        if (before + w > target && w > 0.f) {
+          pick = s;
+          break;
+        }
+        before += w;
+      }
+      if (pick < 0) {
+        tokens[row] = arg;  // uniform * total rounded up to the total: the mode stands in
+      } else {
+        s_seg = pick;
+        s_before = before;
+        s_target = target;
+      }
+    }
+  }
+  __syncthreads();
+  const int seg = s_seg;
+  if (seg < 0) return;
+  const float zmax = s_max;
+  const float* z = logits + static_cast<int64_t>(row) * vocab;
+  const int begin = min(vocab, seg * kSegment + tid * kChunk);
+  const int end = min(vocab, begin + kChunk);
   float part = 0.f;
   for (int i = begin; i < end; ++i) part += expf((z[i] - zmax) * inv_t);
   s_part[tid] = part;
   __syncthreads();
   if (tid == 0) {
-    float total = 0.f;
-    for (int i = 0; i < kSampleThreads; ++i) total += s_part[i];
-    const float target = uniform[row] * total;
-    float before = 0.f;
+    float before = s_before;
     int pick = -1;
+    int last_positive = -1;
     for (int i = 0; i < kSampleThreads; ++i) {
-      const float after = before + s_part[i];
-      if (after > target && s_part[i] > 0.f) {
+      if (s_part[i] > 0.f) last_positive = i;
+      if (before + s_part[i] > s_target && s_part[i] > 0.f) {
         pick = i;
         break;
       }
-      before = after;
+      before += s_part[i];
+    }
+    if (pick < 0) {  // rounding left the running sum a hair below the target
+      pick = last_positive;
+      before = INFINITY;
     }
     s_pick = pick;
     s_before = before;
-    s_target = target;
-    if (pick < 0) tokens[row] = arg;  // uniform rounded up to the total: fall back to the mode
   }
   __syncthreads();
   if (s_pick == tid) {
     float cum = s_before;
     int chosen = -1;
-    int last_positive = arg;
+    int last_positive = begin;
     for (int i = begin; i < end; ++i) {
       const float e = expf((z[i] - zmax) * inv_t);
-      cum += e;
       if (e > 0.f) last_positive = i;
-      if (cum > s_target) {
-        chosen = i;
-        break;
+      if (cum != INFINITY) {
+        cum += e;
+        if (cum > s_target) {
+          chosen = i;
+          break;
+        }
       }
     }
-    // rounding may leave the chunk's own running sum a hair below the target
     tokens[row] = chosen >= 0 ? chosen : last_positive;
   }
 }
@@ -109,12 +184,27 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
 
 using namespace mlr;
 
-extern "C" int mlr_sample(const float* logits, const float* temperature, const float* uniform, int* tokens,
-                          int rows, int vocab, hipStream_t stream) {
-  MLR_REQUIRE(logits && tokens, "null pointer");
+extern "C" {
+
+// Floats of scratch mlr_sample needs.
+int64_t mlr_sample_scratch(int rows, int vocab) {
+  return static_cast<int64_t>(rows) * ((vocab + kSegment - 1) / kSegment) * 3;
+}
+
+int mlr_sample(const float* logits, const float* temperature, const float* uniform, int* tokens, float* scratch,
+               int rows, int vocab, hipStream_t stream) {
+  MLR_REQUIRE(logits && tokens && scratch, "null pointer");
   MLR_REQUIRE(rows > 0 && vocab > 0, "sizes must be > 0");
   MLR_REQUIRE((temperature == nullptr) == (uniform == nullptr), "temperature and uniform come together");
-  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, tokens, vocab);
+  const int segments = (vocab + kSegment - 1) / kSegment;
+  MLR_REQUIRE(segments <= 65535, "vocabulary too large for one launch");
+  sample_partial_kernel<<<dim3(rows, segments), kSampleThreads, 0, stream>>>(logits, temperature, scratch, vocab,
+                                                                             segments);
+  MLR_LAUNCH_CHECK();
+  sample_final_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, scratch, tokens, vocab,
+                                                           segments);
   MLR_LAUNCH_CHECK();
   return 0;
 }
+
+}  // extern "C"

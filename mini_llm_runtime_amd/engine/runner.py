@@ -66,7 +66,15 @@ def _pack_int32(arrays: Sequence[np.ndarray]) -> tuple[np.ndarray, list[tuple[in
 
 
 class ModelRunner:
-    def __init__(self, model: DecoderModel, cache: CacheManager, ops: Any) -> None:
+    def __init__(
+        self,
+        model: DecoderModel,
+        cache: CacheManager,
+        ops: Any,
+        *,
+        use_graphs: bool = True,
+        max_graph_batch: int = 256,
+    ) -> None:
         if model.embed_weight is None:
             raise ValueError("the model's parameters are not loaded")
         self.model = model
@@ -81,6 +89,12 @@ class ModelRunner:
         if tuple(specs) != tuple(cache.site_specs):
             raise ValueError("the cache manager was built for another model's sites")
         self._pinned = torch.cuda.is_available() and self.device.type == "cuda"
+        # Steps that hold single tokens only are captured once per (padded batch, table
+        # width) as a HIP graph and replayed: a decode step of a small model is hundreds of
+        # short kernels, and launching them one by one from the host costs more than running them.
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
+        self.max_graph_batch = int(max_graph_batch)
+        self._graphs: dict[tuple[int, int], tuple] = {}
 
     # -------------------------------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -104,30 +118,46 @@ class ModelRunner:
                     f"max_position_embeddings={self.max_positions}"
                 )
 
-    def _upload(self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray) -> StepContext:
-        groups = len(self.cache.groups)
-        single = layout.q_lens == 1
-        tiles = [(r, q0) for r, n in enumerate(layout.q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
-        tile_array = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
-        arrays = [
-            token_ids,
-            layout.positions,
-            layout.token_entry,
-            layout.cu_q,
-            layout.q_starts,
-            layout.context_lens,
-            layout.state_read,
-            layout.state_write,
-            logit_rows,
-            tile_array,
-            *layout.slot_mappings,
-            *layout.block_tables,
+    # ---- metadata of a step ------------------------------------------------------------------
+    def _arrays(
+        self,
+        layout: StepLayout,
+        token_ids: np.ndarray,
+        logit_rows: np.ndarray,
+        tiles: np.ndarray,
+        pad_entries: Optional[int] = None,
+        table_width: Optional[int] = None,
+    ) -> list[np.ndarray]:
+        """The int32 arrays a step uploads, in a fixed order.  With `pad_entries` (a batch
+        of single tokens only) every array is padded to that many entries: padded entries
+        have no cached tokens, write nothing (slot -1) and own no page."""
+        if pad_entries is None:
+            return [
+                token_ids, layout.positions, layout.token_entry, layout.cu_q, layout.q_starts,
+                layout.context_lens, layout.state_read, layout.state_write, logit_rows, tiles,
+                *layout.slot_mappings, *layout.block_tables,
+            ]
+        count, padded = layout.num_entries, pad_entries
+
+        def pad(a: np.ndarray, fill: int) -> np.ndarray:
+            out = np.full(padded, fill, dtype=np.int32)
+            out[:count] = a
+            return out
+
+        tables = []
+        for t in layout.block_tables:
+            wide = np.full((padded, table_width), -1, dtype=np.int32)
+            wide[:count, : t.shape[1]] = t
+            tables.append(wide)
+        return [
+            pad(token_ids, 0), pad(layout.positions, 0), np.arange(padded, dtype=np.int32),
+            np.arange(padded + 1, dtype=np.int32), pad(layout.q_starts, 0), pad(layout.context_lens, 0),
+            pad(layout.state_read, 0), pad(layout.state_write, 0), np.arange(padded, dtype=np.int32), tiles,
+            *[pad(m, -1) for m in layout.slot_mappings], *tables,
         ]
-        buf, spans = _pack_int32(arrays)
-        host = torch.from_numpy(buf)
-        if self._pinned:
-            host = host.pin_memory()
-        dev = host.to(self.device, non_blocking=True)
+
+    def _context(self, dev: torch.Tensor, spans, layout: StepLayout, **plan) -> StepContext:
+        groups = len(self.cache.groups)
 
         def view(i: int) -> torch.Tensor:
             start, shape = spans[i]
@@ -138,21 +168,15 @@ class ModelRunner:
             ops=self.ops,
             dtype=self.dtype,
             device=self.device,
-            num_tokens=layout.num_tokens,
-            num_entries=layout.num_entries,
             token_ids=view(0),
             positions=view(1),
             token_entry=view(2),
             cu_q=view(3),
             q_starts=view(4),
             context_lens=view(5),
-            max_q_len=int(layout.q_lens.max()),
-            max_context_len=int(layout.context_lens.max()),
             host=layout,
-            query_tiles=view(9) if tiles else None,
-            num_query_tiles=len(tiles),
-            num_decode_entries=int(single.sum()),
-            max_decode_context=int(layout.context_lens[single].max()) if single.any() else 0,
+            query_tiles=view(9) if plan["num_query_tiles"] else None,
+            **plan,
         )
         state_read, state_write = view(6), view(7)
         ctx.memo["logit_rows"] = view(8)
@@ -176,6 +200,89 @@ class ModelRunner:
                 ctx.state_views[site] = StateView(self.cache.state_banks[source].tensor, state_read, state_write)
         return ctx
 
+    def _stage(self, arrays: list[np.ndarray]):
+        buf, spans = _pack_int32(arrays)
+        host = torch.from_numpy(buf)
+        if self._pinned:
+            host = host.pin_memory()
+        return host, spans
+
+    def _forward_eager(self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray) -> Optional[torch.Tensor]:
+        single = layout.q_lens == 1
+        tiles = [(r, q0) for r, n in enumerate(layout.q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
+        tile_array = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, tile_array))
+        dev = host.to(self.device, non_blocking=True)
+        ctx = self._context(
+            dev,
+            spans,
+            layout,
+            num_tokens=layout.num_tokens,
+            num_entries=layout.num_entries,
+            max_q_len=int(layout.q_lens.max()),
+            max_context_len=int(layout.context_lens.max()),
+            num_query_tiles=len(tiles),
+            num_decode_entries=int(single.sum()),
+            max_decode_context=int(layout.context_lens[single].max()) if single.any() else 0,
+        )
+        return self.model.forward(ctx, ctx.memo["logit_rows"] if logit_rows.size else None)
+
+    # ---- decode steps as HIP graphs ---------------------------------------------------------------
+    def _graph_key(self, layout: StepLayout) -> Optional[tuple[int, int]]:
+        """(padded batch, block table width) when the step can replay a captured graph."""
+        if not self.use_graphs or self.cache.state_banks or (layout.q_lens != 1).any():
+            return None
+        count = layout.num_entries
+        if count > self.max_graph_batch:
+            return None
+        padded = 1
+        while padded < count:
+            padded *= 2
+        bs = self.cache.block_size
+        pages = -(-int(layout.context_lens.max()) // bs)
+        quantum = max(1, 1024 // bs)  # table widths in steps of 1,024 tokens
+        return padded, -(-pages // quantum) * quantum
+
+    def _forward_graph(
+        self, key: tuple[int, int], layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray
+    ) -> torch.Tensor:
+        padded, width = key
+        empty = np.zeros((0, 2), dtype=np.int32)
+        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, empty, padded, width))
+        graph = self._graphs.get(key)
+        if graph is None:
+            static = torch.empty_like(host, device=self.device)
+            static.copy_(host, non_blocking=True)
+            ctx = self._context(
+                static,
+                spans,
+                layout,
+                num_tokens=padded,
+                num_entries=padded,
+                max_q_len=1,
+                max_context_len=width * self.cache.block_size,
+                num_query_tiles=0,
+                num_decode_entries=padded,
+                max_decode_context=width * self.cache.block_size,
+            )
+            # one eager run first: everything that is set up lazily must exist before capture
+            self.model.forward(ctx, ctx.memo["logit_rows"])
+            torch.cuda.synchronize(self.device)
+            ctx.memo = {"logit_rows": ctx.memo["logit_rows"]}
+            captured = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(captured):
+                out = self.model.forward(ctx, ctx.memo["logit_rows"])
+            graph = (captured, static, out)
+            self._graphs[key] = graph
+        captured, static, out = graph
+        static.copy_(host, non_blocking=True)
+        captured.replay()
+        if logit_rows.size == layout.num_entries and (logit_rows == np.arange(layout.num_entries)).all():
+            return out[: layout.num_entries]
+        if logit_rows.size == 0:
+            return None
+        return out[torch.from_numpy(logit_rows.astype(np.int64)).to(self.device)]
+
     # -------------------------------------------------------------------------------------------
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry]) -> StepOutput:
@@ -190,11 +297,14 @@ class ModelRunner:
                     rows.append((e.request_id, w))
                     flat.append(int(layout.cu_q[r]) + w)
             logit_rows = np.asarray(flat, dtype=np.int32)
-            ctx = self._upload(layout, token_ids, logit_rows)
             if self.fail_next_step is not None:
                 error, self.fail_next_step = self.fail_next_step, None
                 raise error
-            logits = self.model.forward(ctx, ctx.memo["logit_rows"] if flat else None)
+            key = self._graph_key(layout)
+            if key is not None:
+                logits = self._forward_graph(key, layout, token_ids, logit_rows)
+            else:
+                logits = self._forward_eager(layout, token_ids, logit_rows)
         except BaseException:
             self.cache.abort_step()
             raise

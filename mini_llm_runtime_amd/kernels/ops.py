@@ -19,6 +19,7 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from . import build
+from .deferred import DeferredNorm
 
 _VP = ctypes.c_void_p
 _I = ctypes.c_int
@@ -34,13 +35,15 @@ _SIGNATURES = {
     "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16_norm": ([_VP, _VP, _VP, _I, _F, _VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
         _I,
     ),
-    "mlr_sample": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
+    "mlr_sample": ([_VP, _VP, _VP, _VP, _VP, _I, _I, _VP], _I),
+    "mlr_sample_scratch": ([_I, _I], _I64),
     "mlr_attention_head_dim": ([], _I),
     "mlr_attention_key_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
@@ -210,40 +213,68 @@ class HipOps:
     # ---- matrix products ----------------------------------------------------------------------
     def linear(
         self,
-        x: torch.Tensor,
+        x: Union[torch.Tensor, DeferredNorm],
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
         out_dtype: Optional[torch.dtype] = None,
         kernel: str = "auto",
+        swiglu: bool = False,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
 
         bfloat16 products run on the matrix cores when k is a multiple of 8; float32
         products, and everything with kernel="fma", run as plain 32-bit FMA arithmetic.
+        swiglu: the rows of `weight` are groups (gate 2j, gate 2j+1, up 2j, up 2j+1) and
+        the result is silu(gate) * up, [M, N / 2].
+        x may be a DeferredNorm: for up to 64 tokens its addition and norm run inside
+        the matrix-core kernel; otherwise it is computed first.
         """
-        self._check(x, "linear input", self.dtype, (None, None))
-        m, k = x.shape
+        if kernel not in ("auto", "fma"):
+            raise KernelError("kernel must be 'auto' or 'fma'")
+        deferred = x if isinstance(x, DeferredNorm) else None
+        if deferred is not None:
+            stream_x, delta = deferred.inputs()
+            m, k = stream_x.shape
+        else:
+            self._check(x, "linear input", self.dtype, (None, None))
+            m, k = x.shape
         self._check(weight, "linear weight", self.dtype, (None, k))
         n = weight.shape[0]
         if bias is not None:
             self._check(bias, "linear bias", (torch.float32, self.dtype), (n,))
+        if swiglu and (n % 4 or bias is not None):
+            raise KernelError("a SwiGLU product needs a multiple of 4 rows and no bias")
         out_dtype = out_dtype or self.dtype
         if out_dtype not in (torch.float32, self.dtype):
             raise KernelError(f"linear output must be float32 or {self.dtype}")
-        y = self._empty((m, n), out_dtype)
-        if kernel not in ("auto", "fma"):
-            raise KernelError("kernel must be 'auto' or 'fma'")
-        if kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0:
+        y = self._empty((m, n // 2 if swiglu else n), out_dtype)
+        bias_f32 = int(bias is not None and bias.dtype == torch.float32)
+        out_f32 = int(out_dtype == torch.float32)
+        mfma = kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0
+        if deferred is not None:
+            if mfma and m <= 64 and not deferred.materialized:
+                self._check(stream_x, "residual stream", torch.float32, (m, k))
+                self._check(deferred.weight, "norm weight", (torch.float32, self.dtype), (k,))
+                if delta is not None:
+                    self._check(delta, "residual delta", self.dtype, (m, k))
+                x_out = self._empty((m, k), torch.float32) if delta is not None else None
+                self._call(
+                    "mlr_gemm_bf16_norm", self._ptr(stream_x), self._ptr(delta), self._ptr(deferred.weight),
+                    int(deferred.weight.dtype == torch.float32), deferred.eps, self._ptr(x_out), self._ptr(weight),
+                    self._ptr(bias), bias_f32, self._ptr(y), out_f32, int(swiglu), m, n, k, self._stream(),
+                )
+                deferred.fused(x_out)
+                return y
+            x = deferred.tensor()
+        if mfma:
             self._call(
-                "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias),
-                int(bias is not None and bias.dtype == torch.float32), self._ptr(y),
-                int(out_dtype == torch.float32), m, n, k, self._stream(),
+                "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
+                int(swiglu), m, n, k, self._stream(),
             )
             return y
         self._call(
-            "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias),
-            int(bias is not None and bias.dtype == torch.float32), self._ptr(y),
-            int(out_dtype == torch.float32), self.code, m, n, k, self._stream(),
+            "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
+            int(swiglu), self.code, m, n, k, self._stream(),
         )
         return y
 
@@ -425,8 +456,9 @@ class HipOps:
             self._check(temperature, "temperature", torch.float32, (rows,))
             self._check(uniform, "uniform numbers", torch.float32, (rows,))
         out = self._empty((rows,), torch.int32)
+        scratch = self._empty((self.lib.mlr_sample_scratch(rows, vocab),), torch.float32)
         self._call(
             "mlr_sample", self._ptr(logits), self._ptr(temperature), self._ptr(uniform), self._ptr(out),
-            rows, vocab, self._stream(),
+            self._ptr(scratch), rows, vocab, self._stream(),
         )
         return out

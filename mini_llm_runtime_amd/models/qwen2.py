@@ -52,8 +52,10 @@ def qwen2_spec(config: Qwen2Config) -> ModelSpec:
             WeightRule(src + "self_attn.v_proj.bias", dst + "mixer.qkv_bias_vec", q_rows + kv_rows, kv_rows),
             WeightRule(src + "self_attn.o_proj.weight", dst + "mixer.o_weight"),
             WeightRule(src + "post_attention_layernorm.weight", dst + "norm_post_mixer.weight"),
-            WeightRule(src + "mlp.gate_proj.weight", dst + "feed_forward.gate_up_weight", 0, inter),
-            WeightRule(src + "mlp.up_proj.weight", dst + "feed_forward.gate_up_weight", inter, inter),
+            # gate and up rows woven in pairs (g g u u g g u u ...): the product's epilogue
+            # then holds a gate sum beside its up sum and applies SwiGLU without another kernel
+            WeightRule(src + "mlp.gate_proj.weight", dst + "feed_forward.gate_up_weight", 0, inter, block=2, period=4),
+            WeightRule(src + "mlp.up_proj.weight", dst + "feed_forward.gate_up_weight", 2, inter, block=2, period=4),
             WeightRule(src + "mlp.down_proj.weight", dst + "feed_forward.down_weight"),
         ]
     rules.append(WeightRule("model.norm.weight", "final_norm.weight"))

@@ -33,6 +33,8 @@ class GQAAttention(Mixer):
     [Wq; Wk; Wv] (made by the weight rules at load time).
     """
 
+    accepts_deferred_norm = True
+
     def __init__(
         self,
         hidden_size: int,

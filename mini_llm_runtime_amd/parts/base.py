@@ -36,6 +36,11 @@ class Norm(Part):
         (in place, summed in 32-bit); returns norm(x) in the engine's dtype."""
         raise NotImplementedError
 
+    def defer(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None):
+        """Optional: a `DeferredNorm` that a part with `accepts_deferred_norm` may fuse
+        into its first matrix product.  None: this norm is always computed by `forward`."""
+        return None
+
 
 class PositionEncoding(Part):
     def rotation(self, ctx: StepContext) -> Optional[tuple[torch.Tensor, torch.Tensor, int]]:
@@ -50,6 +55,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True: `forward` may receive a DeferredNorm instead of a tensor and hands it to ops.linear
+    accepts_deferred_norm = False
+
     def cache_spec(self) -> Any:
         """PagedKVSpec, SlotStateSpec or None."""
         return None
@@ -60,6 +68,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_deferred_norm = False
+
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
@@ -69,8 +79,9 @@ class Block(Part):
 
     def forward(
         self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor], site: int
-    ) -> Optional[torch.Tensor]:
-        """x: float32 residual stream, updated in place.  `delta` is the previous
-        layer's output that has not been added yet (None at the first layer); the
-        return value is this layer's own not-yet-added output."""
+    ) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """x: float32 residual stream.  `delta` is the previous layer's output that has
+        not been added yet (None at the first layer).  Returns the residual stream (the
+        same tensor updated in place, or a new one) and this layer's own not-yet-added
+        output."""
         raise NotImplementedError

@@ -17,12 +17,16 @@ class SwiGLU(FeedForward):
     """Dense gated feed-forward: `down(silu(gate(x)) * up(x))`, no biases.
 
     Formula: src/mini_llm_runtime/qwen_model_runner.py:215-217.  Gate and up are one
-    matrix product over [Wgate; Wup] (concatenated by the weight rules).
+    matrix product over a matrix that holds the rows of Wgate and Wup woven in pairs
+    (gate 0, gate 1, up 0, up 1, gate 2, ...; made by the weight rules), and
+    silu(gate) * up is that product's epilogue.
     """
 
+    accepts_deferred_norm = True
+
     def __init__(self, hidden_size: int, intermediate_size: int) -> None:
-        if hidden_size <= 0 or intermediate_size <= 0:
-            raise ValueError("SwiGLU sizes must be > 0")
+        if hidden_size <= 0 or intermediate_size <= 0 or intermediate_size % 2:
+            raise ValueError("SwiGLU sizes must be > 0 and the intermediate size even")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.gate_up_weight: Optional[torch.Tensor] = None
@@ -36,6 +40,5 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
-        gate_up = ops.linear(h, self.gate_up_weight, None)
-        hidden = ops.silu_mul(gate_up)
+        hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
         return ops.linear(hidden, self.down_weight, None)

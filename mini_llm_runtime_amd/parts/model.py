@@ -120,12 +120,14 @@ class DecoderModel:
         x = ops.embedding(self.embed_weight, ctx.token_ids)
         delta: Optional[torch.Tensor] = None
         for site, entry in enumerate(self.spec.order):
-            delta = self.layers[entry.layer].forward(ctx, x, delta, site)
+            x, delta = self.layers[entry.layer].forward(ctx, x, delta, site)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         rows = ops.gather_rows(x, logit_rows)
         delta_rows = ops.gather_rows(delta, logit_rows) if delta is not None else None
-        h = self.final_norm.forward(ctx, rows, delta_rows)
+        h = self.final_norm.defer(ctx, rows, delta_rows)
+        if h is None:
+            h = self.final_norm.forward(ctx, rows, delta_rows)
         return ops.linear(h, self.head_weight, None, out_dtype=torch.float32)
 
 

@@ -56,9 +56,11 @@ class OrderEntry:
 @dataclass(frozen=True)
 class WeightRule:
     """Checkpoint tensor `name` fills rows [row_start, row_start + rows) of parameter
-    `dest` (all of it when `rows` is None).  `optional` tensors may be absent; when
-    `must_equal` names another parameter, a present tensor has to equal it (a tied
-    head stored a second time)."""
+    `dest` (all of it when `rows` is None).  With `block` and `period` the rows are
+    interleaved instead: source row i goes to row_start + (i // block) * period +
+    i % block (two matrices woven together in groups of `block` rows).  `optional`
+    tensors may be absent; when `must_equal` names another parameter, a present
+    tensor has to equal it (a tied head stored a second time)."""
 
     name: str
     dest: str
@@ -66,6 +68,14 @@ class WeightRule:
     rows: Optional[int] = None
     optional: bool = False
     must_equal: Optional[str] = None
+    block: int = 0
+    period: int = 0
+
+    def dest_rows(self, count: int) -> "list[int]":
+        """Destination row of each of `count` source rows."""
+        if not self.block:
+            return list(range(self.row_start, self.row_start + count))
+        return [self.row_start + (i // self.block) * self.period + i % self.block for i in range(count)]
 
 
 @dataclass(frozen=True)

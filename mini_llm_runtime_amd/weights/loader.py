@@ -106,16 +106,10 @@ def _check_coverage(model: DecoderModel) -> None:
             continue
         rows = specs[rule.dest].shape[0]
         n = rows if rule.rows is None else rule.rows
-        covered[rule.dest].append((rule.row_start, rule.row_start + n))
-    for name, spans in covered.items():
-        spans.sort()
-        at = 0
-        for a, b in spans:
-            if a != at:
-                raise ValueError(f"weight rules leave rows {at}..{a} of {name} unfilled or fill them twice")
-            at = b
-        if at != specs[name].shape[0]:
-            raise ValueError(f"weight rules fill {at} of {specs[name].shape[0]} rows of {name}")
+        covered[rule.dest].extend(rule.dest_rows(n))
+    for name, rows in covered.items():
+        if sorted(rows) != list(range(specs[name].shape[0])):
+            raise ValueError(f"the weight rules do not fill every row of {name} exactly once")
 
 
 def load_weights(
@@ -176,7 +170,11 @@ def load_weights(
                 continue
             dest = params[rule.dest]
             rows = dest.shape[0] if rule.rows is None else rule.rows
-            dest[rule.row_start : rule.row_start + rows].copy_(tensor.to(dest.dtype))
+            if rule.block:
+                index = torch.tensor(rule.dest_rows(rows), dtype=torch.long, device=dest.device)
+                dest.index_copy_(0, index, tensor.to(dest.dtype).to(dest.device))
+            else:
+                dest[rule.row_start : rule.row_start + rows].copy_(tensor.to(dest.dtype))
         for n, other, tensor in checks:
             ref = params[other]
             if not torch.equal(tensor.to(ref.dtype).to(ref.device), ref):

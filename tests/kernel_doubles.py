@@ -16,6 +16,8 @@ from typing import Optional
 
 import torch
 
+from mini_llm_runtime_amd.kernels.deferred import DeferredNorm
+
 
 class TorchOps:
     def __init__(self, dtype: torch.dtype = torch.float32, device: str = "cpu") -> None:
@@ -46,11 +48,17 @@ class TorchOps:
         return x[rows.long()].contiguous()
 
     # matrix products ---------------------------------------------------------------------
-    def linear(self, x, weight, bias=None, out_dtype=None):
+    def linear(self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False):
         self._count("linear")
+        if isinstance(x, DeferredNorm):
+            x = x.tensor()
         y = x.float() @ weight.float().t()
         if bias is not None:
             y = y + bias.float()
+        if swiglu:  # rows of weight: gate 2j, gate 2j+1, up 2j, up 2j+1
+            quads = y.view(y.shape[0], -1, 4)
+            gate, up = quads[..., :2], quads[..., 2:]
+            y = (gate * torch.sigmoid(gate) * up).reshape(y.shape[0], -1)
         return y.to(out_dtype or self.dtype)
 
     def silu_mul(self, gate_up):

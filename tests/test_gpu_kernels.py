@@ -150,6 +150,58 @@ def test_linear_bf16_matrix_cores(ops_for, m, n, k):
     torch.testing.assert_close(got16, ref - b.double(), **_tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,inter,k", [(1, 352, 96), (8, 4864, 896), (40, 130, 64), (200, 352, 136), (300, 64, 1000)])
+def test_linear_swiglu_epilogue(ops_for, dtype, m, inter, k):
+    """silu(gate) * up as the product's epilogue over rows woven in pairs (g g u u ...), on every
+    kernel: matrix cores (skinny and tiled) and plain FMA."""
+    ops = ops_for(dtype)
+    x = _rand((m, k), dtype, 43)
+    gate = _rand((inter, k), dtype, 44, 0.1)
+    up = _rand((inter, k), dtype, 45, 0.1)
+    woven = torch.empty(2 * inter, k, dtype=dtype)
+    idx = torch.arange(inter)
+    woven[(idx // 2) * 4 + idx % 2] = gate
+    woven[(idx // 2) * 4 + 2 + idx % 2] = up
+    g = x.double() @ gate.double().t()
+    ref = g * torch.sigmoid(g) * (x.double() @ up.double().t())
+    for kernel in ("auto", "fma"):
+        got = ops.linear(x.cuda(), woven.cuda(), None, swiglu=True, kernel=kernel).cpu()
+        assert got.shape == (m, inter)
+        tol = dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else _tol(dtype)
+        torch.testing.assert_close(got.double(), ref, **tol)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1152, 896), (8, 9728, 896), (16, 130, 64), (33, 517, 2056), (64, 96, 4864)])
+@pytest.mark.parametrize("weight_f32", [False, True])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_linear_with_fused_norm(ops_for, m, n, k, weight_f32, with_delta):
+    """x += delta, RMSNorm and the product in one kernel against the three separate steps in float64."""
+    from mini_llm_runtime_amd.kernels.deferred import DeferredNorm
+
+    ops = ops_for(torch.bfloat16)
+    x = _rand((m, k), torch.float32, 46, 2.0)
+    delta = _rand((m, k), torch.bfloat16, 47) if with_delta else None
+    nw = (1 + _rand((k,), torch.float32, 48, 0.1)).to(torch.float32 if weight_f32 else torch.bfloat16)
+    w = _rand((n, k), torch.bfloat16, 49, 0.05)
+    b = _rand((n,), torch.float32, 50)
+    eps = 1e-6
+    summed = x.double() + (delta.double() if with_delta else 0)
+    ref = plain.rms_norm(summed, nw.double(), eps) @ w.double().t() + b.double()
+    xd = x.cuda()
+    deferred = DeferredNorm(ops, xd, delta.cuda() if with_delta else None, nw.cuda(), eps)
+    got = ops.linear(deferred, w.cuda(), b.cuda(), out_dtype=torch.float32).cpu()
+    # the kernel rounds (x * norm weight) to bfloat16 before the product: one rounding per input element
+    torch.testing.assert_close(got.double(), ref, atol=3e-2 * float(ref.abs().max()) / 4, rtol=1.6e-2)
+    assert float((got.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()) < 4e-3
+    torch.testing.assert_close(deferred.residual.cpu().double(), summed, atol=1e-6, rtol=1e-6)
+    if with_delta:
+        assert torch.equal(xd.cpu(), x), "the fused kernel must not write into its input stream"
+    # a second consumer of the same deferred norm gets the separately computed activations
+    again = ops.linear(deferred, w.cuda(), b.cuda(), out_dtype=torch.float32).cpu()
+    assert float((again.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()) < 4e-3
+
+
 # ---- rotary encoding and cache write ----------------------------------------------------------------
 def test_rope_table(ops_for):
     ops = ops_for(torch.float32)

@@ -12,7 +12,7 @@ import torch
 import mini_llm_runtime_amd.models  # noqa: F401
 import plain_qwen2 as plain
 import schedules
-from helpers import BLOCK_SIZE, TINY, make_model_dir, make_runner, random_tokens, read_weights
+from helpers import BLOCK_SIZE, TINY, StepEntry, make_model_dir, make_runner, random_tokens, read_weights
 from kernel_doubles import TorchOps
 
 LENGTHS = {"A": (5, 17, 33, 70, 41, 52), "B": (1, 9, 24, 40, 63, 37)}
@@ -144,3 +144,56 @@ def test_schedules_agree_with_each_other(tmp_path, backend, dtype):
     for other in results[1:]:
         for key, row in results[0].items():
             assert torch.allclose(row, other[key], atol=2e-5, rtol=0), key
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_long_decoding_graph_replays_match_eager(tmp_path, dtype):
+    """Decode steps replay a captured HIP graph.  Every replay, with eager steps (portions of a
+    further prompt) and synchronisations between the replays, must give exactly what the same
+    step gives when its kernels are launched one by one; both follow the plain implementation
+    over 100 decoded tokens, across page edges and a change of the graph's batch size."""
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    which = "B"
+    model_dir = make_model_dir(tmp_path, which, seed=12)
+    cfg, weights = read_weights(model_dir)
+    vocab = cfg["vocab_size"]
+    requests = {f"d{i}": random_tokens(n, vocab, 500 + i) for i, n in enumerate((130, 117, 141))}
+    extra = random_tokens(90, vocab, 600)
+    ops = HipOps(dtype, "cuda")
+    results = []
+    for use_graphs in (True, False):
+        config, model, cache, runner = make_runner(model_dir, ops, block_size=8, num_blocks=80, max_requests=4)
+        runner.use_graphs = use_graphs
+        cache.poison()
+        got = {}
+        for rid, toks in requests.items():
+            cache.create_request(rid)
+            out = runner.step([StepEntry.of(rid, toks[:30], range(30))])
+            for i in range(30):
+                got[(rid, i)] = out.logits[i].float().cpu()
+        cache.create_request("x")
+        fed_x = 0
+        for step in range(30, 141):
+            live = [rid for rid, toks in requests.items() if step < len(toks)]
+            out = runner.step([StepEntry.of(rid, [requests[rid][step]], (0,)) for rid in live])
+            rows = out.logits.float().cpu()
+            for i, rid in enumerate(live):
+                got[(rid, step)] = rows[i].clone()
+            if step % 7 == 0 and fed_x < len(extra):  # eager work between the replays
+                n = min(5, len(extra) - fed_x)
+                out = runner.step([StepEntry.of("x", extra[fed_x : fed_x + n], range(n))])
+                for i in range(n):
+                    got[("x", fed_x + i)] = out.logits[i].float().cpu()
+                fed_x += n
+        if use_graphs:
+            assert len(runner._graphs) >= 2, "the decode steps did not go through captured graphs"
+        results.append(got)
+    graph, eager = results
+    assert graph.keys() == eager.keys()
+    for key in graph:
+        assert torch.equal(graph[key], eager[key]), f"graph replay differs from eager launch at {key}"
+    everything = dict(requests)
+    everything["x"] = extra[: max(p for r, p in graph if r == "x") + 1]
+    _compare(graph, everything, weights, cfg, dtype)
