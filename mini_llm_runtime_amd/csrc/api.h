@@ -21,18 +21,21 @@ int mlr_version();
 int mlr_embedding(const void* table, int dtype, const int* ids, float* out, int tokens, int hidden,
                   int vocab, hipStream_t stream);
 
-// x (float32 [rows, hidden]) += delta (dtype, may be null), then
-// out = weight * x * rsqrt(mean(x^2) + eps) in `dtype`; weight is float32 when
-// weight_is_f32, else `dtype`.
-int mlr_rmsnorm(float* x, const void* delta, const void* weight, int weight_is_f32, void* out,
-                int dtype, int rows, int hidden, float eps, hipStream_t stream);
+// x (float32 [rows, hidden]) += delta, then out = weight * x * rsqrt(mean(x^2) + eps)
+// in `dtype`; weight is float32 when weight_is_f32, else `dtype`.  The delta is
+// `delta` ([rows, hidden] in `dtype`), or `slices` float32 partial sums `partial`
+// [slices, rows, hidden] added in slice order, or nothing (both null).
+int mlr_rmsnorm(float* x, const void* delta, const float* partial, int slices, const void* weight,
+                int weight_is_f32, void* out, int dtype, int rows, int hidden, float eps,
+                hipStream_t stream);
 
 // x (float32) += delta (dtype), count elements.
 int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t stream);
 
-// out[k, :] = src[rows[k], :]; rows are `row_bytes` wide (a multiple of 4).
+// out[p, k, :] = src[p, rows[k], :] for every plane p of src [planes, src_rows, width];
+// rows are `row_bytes` wide (a multiple of 4).
 int mlr_gather_rows(const void* src, const int* rows, void* out, int count, int64_t row_bytes,
-                    int src_rows, hipStream_t stream);
+                    int src_rows, int planes, hipStream_t stream);
 
 // out[m, i] = silu(gate_up[m, i]) * gate_up[m, inter + i].
 int mlr_silu_mul(const void* gate_up, void* out, int dtype, int rows, int inter, hipStream_t stream);
@@ -60,18 +63,12 @@ int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_
                     int out_is_f32, int swiglu, int dtype, int m, int n, int k, hipStream_t stream);
 
 // The same product in bfloat16 on the matrix cores (float32 accumulation).  Needs
-// k % 8 == 0 and 16-byte aligned x and w; any m and n.
+// k % 8 == 0 and 16-byte aligned x and w; any m and n.  With slices > 1 (a value
+// mlr_gemm_bf16_slices returned for this shape) y is float32 [slices, m, n]: partial
+// sums over slices of k, the bias in slice 0, for the consumer to add up in order.
+int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                  int out_is_f32, int swiglu, int m, int n, int k, hipStream_t stream);
-
-// mlr_gemm_bf16 with the RMSNorm of its input fused in, for up to 64 tokens: the
-// input is norm(x + delta) with x float32 [m, k], delta bfloat16 (may be null) and
-// norm weight [k] (float32 when norm_weight_is_f32, else bfloat16); x + delta is
-// written to x_out (float32 [m, k]; may be null; must not alias x).
-int mlr_gemm_bf16_norm(const float* x, const void* delta, const void* norm_weight,
-                       int norm_weight_is_f32, float eps, float* x_out, const void* w,
-                       const void* bias, int bias_is_f32, void* y, int out_is_f32, int swiglu, int m,
-                       int n, int k, hipStream_t stream);
+                  int out_is_f32, int swiglu, int slices, int m, int n, int k, hipStream_t stream);
 
 // Attention of every token over its request's pages: token t (entry
 // token_entry[t], absolute position positions[t]) sees the keys

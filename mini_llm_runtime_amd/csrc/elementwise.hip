@@ -8,6 +8,8 @@
 
 namespace mlr {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 // ---- embedding -------------------------------------------------------------------
 // qwen_model_runner.py:263 (F.embedding): a row gather, no scaling.
 template <typename T>
@@ -27,26 +29,73 @@ __global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ ta
 
 // ---- RMSNorm (+ residual addition) ---------------------------------------------------
 // qwen_model_runner.py:22-26: weight * x * rsqrt(mean(x^2) + eps), statistics in float32.
-template <typename T, typename TW>
+// The not-yet-added delta is either one tensor in the engine's dtype or `slices`
+// float32 partial sums [slice, rows, hidden] of a product that was cut along k;
+// they are added in slice order, so the sum does not depend on timing.
+// One workgroup per row; a row of up to 256 * 4 * VPT elements stays in registers
+// between the statistics and the scaling (hidden must be a multiple of 4).
+template <typename T, typename TW, int VPT>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                                      const float* __restrict__ partial, int slices, int rows,
                                                       const TW* __restrict__ weight, T* __restrict__ out,
                                                       int hidden, float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
+  const int quads = hidden / 4;
+  f32x4 v[VPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * 256;
+    v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (i >= quads) continue;
+    const int64_t at = row * hidden + 4 * i;
+    f32x4 a = *reinterpret_cast<const f32x4*>(x + at);
+    bool changed = false;
+    if (delta != nullptr) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] += to_f32(delta[at + e]);
+      changed = true;
+    }
+    for (int s = 0; s < slices; ++s) {
+      const f32x4 p = *reinterpret_cast<const f32x4*>(partial + (static_cast<int64_t>(s) * rows + row) * hidden + 4 * i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] += p[e];
+      changed = true;
+    }
+    if (changed) *reinterpret_cast<f32x4*>(x + at) = a;
+    v[j] = a;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += a[e] * a[e];
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i >= quads) continue;
+    const int64_t at = row * hidden + 4 * i;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[at + e] = from_f32<T>(to_f32(weight[4 * i + e]) * (v[j][e] * inv));
+  }
+}
+
+// Any width: the row is read again for the scaling.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void rmsnorm_any_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                                          const float* __restrict__ partial, int slices, int rows,
+                                                          const TW* __restrict__ weight, T* __restrict__ out,
+                                                          int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
   float* xr = x + row * hidden;
   float ss = 0.f;
-  if (delta != nullptr) {
-    const T* dr = delta + row * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      const float v = xr[i] + to_f32(dr[i]);
-      xr[i] = v;
-      ss += v * v;
-    }
-  } else {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      const float v = xr[i];
-      ss += v * v;
-    }
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = xr[i];
+    if (delta != nullptr) v += to_f32(delta[row * hidden + i]);
+    for (int s = 0; s < slices; ++s) v += partial[(static_cast<int64_t>(s) * rows + row) * hidden + i];
+    if (delta != nullptr || slices > 0) xr[i] = v;
+    ss += v * v;
   }
   const float total = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
@@ -54,6 +103,25 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
   // each thread re-reads the elements it wrote itself
   for (int i = threadIdx.x; i < hidden; i += blockDim.x)
     orow[i] = from_f32<T>(to_f32(weight[i]) * (xr[i] * inv));
+}
+
+template <typename T, typename TW>
+static void launch_rmsnorm(float* x, const void* delta, const float* partial, int slices, const void* weight,
+                           void* out, int rows, int hidden, float eps, hipStream_t stream) {
+  const T* d = static_cast<const T*>(delta);
+  const TW* w = static_cast<const TW*>(weight);
+  T* o = static_cast<T*>(out);
+  const int quads = hidden / 4;
+  if (hidden % 4 != 0 || quads > 256 * 8)
+    rmsnorm_any_kernel<T, TW><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
+  else if (quads <= 256)
+    rmsnorm_kernel<T, TW, 1><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
+  else if (quads <= 512)
+    rmsnorm_kernel<T, TW, 2><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
+  else if (quads <= 1024)
+    rmsnorm_kernel<T, TW, 4><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
+  else
+    rmsnorm_kernel<T, TW, 8><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
 }
 
 template <typename T>
@@ -69,7 +137,8 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint32_t* __rest
                                                           int src_rows) {
   const int k = blockIdx.x;
   const int r = rows[k];
-  uint32_t* dst = out + static_cast<int64_t>(k) * row_words;
+  src += static_cast<int64_t>(blockIdx.y) * src_rows * row_words;  // plane of a [planes, rows, width] source
+  uint32_t* dst = out + (static_cast<int64_t>(blockIdx.y) * gridDim.x + k) * row_words;
   if (r < 0 || r >= src_rows) {
     for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) dst[i] = 0xffffffffu;  // NaN in both types
     return;
@@ -204,25 +273,21 @@ int mlr_embedding(const void* table, int dtype, const int* ids, float* out, int 
   return 0;
 }
 
-int mlr_rmsnorm(float* x, const void* delta, const void* weight, int weight_is_f32, void* out, int dtype,
-                int rows, int hidden, float eps, hipStream_t stream) {
+int mlr_rmsnorm(float* x, const void* delta, const float* partial, int slices, const void* weight,
+                int weight_is_f32, void* out, int dtype, int rows, int hidden, float eps, hipStream_t stream) {
   MLR_REQUIRE(x && weight && out, "null pointer");
   MLR_REQUIRE(rows > 0 && hidden > 0, "sizes must be > 0");
   MLR_REQUIRE(eps >= 0.f, "eps must be >= 0");
+  MLR_REQUIRE(slices >= 0 && slices <= 64 && (slices == 0) == (partial == nullptr), "partial sums and their count come together");
+  MLR_REQUIRE(delta == nullptr || partial == nullptr, "one kind of delta at a time");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   if (dtype == kF32) {
     MLR_REQUIRE(weight_is_f32, "a float32 engine needs float32 norm weights");
-    rmsnorm_kernel<float, float><<<rows, 256, 0, stream>>>(x, static_cast<const float*>(delta),
-                                                          static_cast<const float*>(weight),
-                                                          static_cast<float*>(out), hidden, eps);
+    launch_rmsnorm<float, float>(x, delta, partial, slices, weight, out, rows, hidden, eps, stream);
   } else if (weight_is_f32) {
-    rmsnorm_kernel<bf16, float><<<rows, 256, 0, stream>>>(x, static_cast<const bf16*>(delta),
-                                                         static_cast<const float*>(weight),
-                                                         static_cast<bf16*>(out), hidden, eps);
+    launch_rmsnorm<bf16, float>(x, delta, partial, slices, weight, out, rows, hidden, eps, stream);
   } else {
-    rmsnorm_kernel<bf16, bf16><<<rows, 256, 0, stream>>>(x, static_cast<const bf16*>(delta),
-                                                        static_cast<const bf16*>(weight),
-                                                        static_cast<bf16*>(out), hidden, eps);
+    launch_rmsnorm<bf16, bf16>(x, delta, partial, slices, weight, out, rows, hidden, eps, stream);
   }
   MLR_LAUNCH_CHECK();
   return 0;
@@ -243,11 +308,11 @@ int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t s
 }
 
 int mlr_gather_rows(const void* src, const int* rows, void* out, int count, int64_t row_bytes, int src_rows,
-                    hipStream_t stream) {
+                    int planes, hipStream_t stream) {
   MLR_REQUIRE(src && rows && out, "null pointer");
-  MLR_REQUIRE(count > 0 && src_rows > 0, "sizes must be > 0");
+  MLR_REQUIRE(count > 0 && src_rows > 0 && planes > 0 && planes < 65536, "sizes must be > 0");
   MLR_REQUIRE(row_bytes > 0 && row_bytes % 4 == 0, "rows must be a multiple of 4 bytes wide");
-  gather_rows_kernel<<<count, 256, 0, stream>>>(static_cast<const uint32_t*>(src), rows,
+  gather_rows_kernel<<<dim3(count, planes), 256, 0, stream>>>(static_cast<const uint32_t*>(src), rows,
                                                 static_cast<uint32_t*>(out), row_bytes / 4, src_rows);
   MLR_LAUNCH_CHECK();
   return 0;

@@ -6,28 +6,29 @@
 // accumulator then holds four consecutive output features of one token per lane,
 // which gives 8-byte stores and lets an epilogue see neighbouring features.
 //
-// Two kernels:
-//  * gemm_skinny: up to 64 tokens (decode).  Bound by streaming w once.  A
-//    workgroup owns 16 output features; its wavefronts split K between them
-//    (interleaved, so the workgroup reads contiguous spans of every weight row),
-//    keep several 16-byte loads in flight per lane, and add their partial sums
-//    through LDS.  Activations come straight from L2.
+// Kernels:
+//  * gemm_skinny_split: up to 16 tokens (decode at small batch).  Bound by streaming
+//    w once, and a single compute unit can only keep a few dozen cache lines in
+//    flight, so the stream has to be spread over all of them: a workgroup owns 16
+//    output features and one slice of K (grid.y slices); its wavefronts split the
+//    slice between them (interleaved, so the workgroup reads contiguous spans of
+//    every weight row), keep eight 16-byte loads in flight per lane, and add their
+//    partial sums through LDS.  Activations come straight from L2.
+//  * gemm_skinny_rows: 17..64 tokens.  A workgroup owns 64 output features, one
+//    16-row slab per wavefront, and one slice of K; the wavefronts read the same
+//    activation chunks at the same time, so those come from the L1 cache.
+//    With more than one K slice both kernels write float32 partial sums
+//    [slice, M, N]; the consumer (the residual-adding norm kernel) sums them in a
+//    fixed order, so results do not depend on which slice finishes first.
 //  * gemm_tiled: many tokens (prompts).  128 x 128 output tile per workgroup,
 //    K in slices of 64 staged through double-buffered LDS, four wavefronts of
 //    64 x 64 each, 32x32x16 MFMA.
 // K must be a multiple of 8 (16-byte rows); other shapes take the FMA kernel.
 //
-// Fusions (they save whole kernels in a decode step, which is a chain of very
-// short ones):
-//  * norm prologue (skinny only): the input is the float32 residual stream plus
-//    a not-yet-added delta; the kernel adds them, writes the sum out once,
-//    multiplies by the norm weight while building its operand, collects the sum
-//    of squares on the way and scales the finished sums by rsqrt(mean + eps).
-//    RMSNorm commutes with the product because its statistic is one scalar per
-//    token (formula: src/mini_llm_runtime/qwen_model_runner.py:22-26).
-//  * SwiGLU epilogue: with gate and up rows interleaved in pairs
-//    (g0 g1 u0 u1 g2 g3 u2 u3 ...) a lane holds two gate sums and their two up
-//    sums and stores silu(gate) * up (qwen_model_runner.py:215-216) directly.
+// SwiGLU epilogue: with gate and up rows interleaved in pairs
+// (g0 g1 u0 u1 g2 g3 u2 u3 ...) a lane holds two gate sums and their two up sums
+// and stores silu(gate) * up (src/mini_llm_runtime/qwen_model_runner.py:215-216)
+// directly, which saves a kernel and a round trip of the widest activation.
 #include "api.h"
 #include "common.h"
 #include "mfma.h"
@@ -40,15 +41,6 @@ struct GemmEpilogue {
   void* y;
   int out_is_f32;
   int swiglu;  // store silu(v0) * v2, silu(v1) * v3 into a row of N / 2
-};
-
-struct NormPrologue {
-  const float* x;      // residual stream [M, K]
-  const bf16* delta;   // not-yet-added delta [M, K], may be null
-  const void* weight;  // norm weight [K]
-  int weight_is_f32;
-  float* x_out;        // x + delta [M, K], may be null
-  float eps;
 };
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
@@ -102,134 +94,131 @@ __device__ __forceinline__ void store4(const GemmEpilogue& ep, int64_t m, int n,
   }
 }
 
-// Eight consecutive elements of the normed-but-not-yet-scaled input of token row
-// `m` at chunk c: (x + delta) * weight, rounded to bfloat16; adds their squares
-// to `ssq` and, when asked, writes x + delta out.
-__device__ __forceinline__ bf16x8_t norm_chunk(const NormPrologue& np, int64_t row_offset, int c, bool write_out,
-                                               float& ssq) {
-  const f32x4_t* xp = reinterpret_cast<const f32x4_t*>(np.x + row_offset) + 2 * c;
-  f32x4_t lo = xp[0];
-  f32x4_t hi = xp[1];
-  float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  if (np.delta != nullptr) {
-    const u16x8_t d = *(reinterpret_cast<const u16x8_t*>(np.delta + row_offset) + c);
+// Store one accumulator tile (4 consecutive features of one token per lane): the
+// final result, or this K slice's partial sums.
+__device__ __forceinline__ void finish4(const GemmEpilogue& ep, int slice, int slices, int m, int n, int M, int N,
+                                        const float (&v)[4]) {
+  if (m >= M || n >= N) return;
+  if (slices == 1) {
+    store4(ep, m, n, N, v[0], v[1], v[2], v[3]);
+    return;
+  }
+  float* dst = static_cast<float*>(ep.y) + (static_cast<int64_t>(slice) * M + m) * N + n;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] += to_f32(bf16{d[i]});
+  for (int i = 0; i < 4; ++i) {
+    if (n + i >= N) continue;
+    float out = v[i];
+    if (slice == 0 && ep.bias != nullptr) out += load_as_f32(ep.bias, n + i, ep.bias_is_f32);
+    dst[i] = out;
   }
-  if (write_out) {
-    f32x4_t* op = reinterpret_cast<f32x4_t*>(np.x_out + row_offset) + 2 * c;
-    op[0] = f32x4_t{v[0], v[1], v[2], v[3]};
-    op[1] = f32x4_t{v[4], v[5], v[6], v[7]};
-  }
-  float w[8];
-  if (np.weight_is_f32) {
-    const f32x4_t* wp = reinterpret_cast<const f32x4_t*>(np.weight) + 2 * c;
-    const f32x4_t a = wp[0], b = wp[1];
-    w[0] = a[0]; w[1] = a[1]; w[2] = a[2]; w[3] = a[3];
-    w[4] = b[0]; w[5] = b[1]; w[6] = b[2]; w[7] = b[3];
-  } else {
-    const u16x8_t ww = *(reinterpret_cast<const u16x8_t*>(np.weight) + c);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) w[i] = to_f32(bf16{ww[i]});
-  }
-  u16x8_t out;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    ssq += v[i] * v[i];
-    out[i] = f32_to_bf16(v[i] * w[i]).bits;
-  }
-  return __builtin_bit_cast(bf16x8_t, out);
 }
 
-// ---- skinny: M <= 16 * MT ---------------------------------------------------------------
-template <int MT, int WAVES, bool NORM>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ x,
-                                                                 const bf16* __restrict__ w, NormPrologue np,
-                                                                 GemmEpilogue ep, int M, int N, int K) {
-  constexpr int U = NORM ? 4 : 8;  // k-steps in flight per wavefront
-  __shared__ float red[WAVES][MT][kWave][4];
-  __shared__ float red_ssq[NORM ? WAVES : 1][MT][16];
+// ---- skinny, up to 16 tokens: wavefronts split K ------------------------------------------
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf16* __restrict__ x,
+                                                                       const bf16* __restrict__ w,
+                                                                       GemmEpilogue ep, int M, int N, int K) {
+  constexpr int U = 8;  // k-steps in flight per wavefront
+  __shared__ float red[WAVES][kWave][4];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int r = lane % 16;
   const int q = lane / 16;
   const int n0 = blockIdx.x * 16;
-  const int wrow = min(n0 + r, N - 1);
+  const int slices = gridDim.y;
   const int chunks = K / 8;             // 16-byte chunks per row
   const int ksteps = (chunks + 3) / 4;  // one MFMA consumes 4 chunks (32 elements of k)
-  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(wrow) * K);
+  const int per = (ksteps + slices - 1) / slices;
+  const int sb = blockIdx.y * per;
+  const int se = min(ksteps, sb + per);
+  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(n0 + r, N - 1)) * K);
+  const bf16x8_t* xp = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(r, M - 1)) * K);
+  const bool xok = r < M;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+  for (int s0 = sb + wave; s0 < se; s0 += WAVES * U) {
+    bf16x8_t a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * WAVES;
+      const int c = s * 4 + q;
+      a[u] = (s < se && c < chunks) ? __builtin_nontemporal_load(wp + c) : zero_bf16x8();
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * WAVES;
+      const int c = s * 4 + q;
+      b[u] = (xok && s < se && c < chunks) ? xp[c] : zero_bf16x8();
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc = mfma_16x16x32(a[u], b[u], acc);
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+  __syncthreads();
+  if (wave == 0) {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int ww = 0; ww < WAVES; ++ww)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] += red[ww][lane][i];
+    finish4(ep, blockIdx.y, slices, r, n0 + q * 4, M, N, v);
+  }
+}
+
+// ---- skinny, 17..64 tokens: one 16-row slab per wavefront ----------------------------------
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_skinny_rows_kernel(const bf16* __restrict__ x,
+                                                               const bf16* __restrict__ w, GemmEpilogue ep,
+                                                               int M, int N, int K) {
+  constexpr int U = 4;
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int r = lane % 16;
+  const int q = lane / 16;
+  const int n0 = (blockIdx.x * 4 + wave) * 16;
+  if (n0 >= N) return;
+  const int slices = gridDim.y;
+  const int chunks = K / 8;
+  const int ksteps = (chunks + 3) / 4;
+  const int per = (ksteps + slices - 1) / slices;
+  const int sb = blockIdx.y * per;
+  const int se = min(ksteps, sb + per);
+  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(n0 + r, N - 1)) * K);
   const bf16x8_t* xp[MT];
-  int64_t xoff[MT];
   bool xok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
     xok[mt] = m < M;
-    xoff[mt] = static_cast<int64_t>(min(m, M - 1)) * K;
-    xp[mt] = NORM ? nullptr : reinterpret_cast<const bf16x8_t*>(x + xoff[mt]);
+    xp[mt] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(m, M - 1)) * K);
   }
-  const bool write_out = NORM && np.x_out != nullptr && blockIdx.x == 0;
   f32x4_t acc[MT];
-  float ssq[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    ssq[mt] = 0.f;
-  }
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (int s0 = wave; s0 < ksteps; s0 += WAVES * U) {
+  for (int s0 = sb; s0 < se; s0 += U) {
     bf16x8_t a[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = (s0 + u * WAVES) * 4 + q;
-      a[u] = c < chunks ? __builtin_nontemporal_load(wp + c) : zero_bf16x8();
+      const int c = (s0 + u) * 4 + q;
+      a[u] = (s0 + u < se && c < chunks) ? __builtin_nontemporal_load(wp + c) : zero_bf16x8();
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = (s0 + u * WAVES) * 4 + q;
+      const int c = (s0 + u) * 4 + q;
+      const bool in = s0 + u < se && c < chunks;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        bf16x8_t b = zero_bf16x8();
-        if (xok[mt] && c < chunks) {
-          if (NORM)
-            b = norm_chunk(np, xoff[mt], c, write_out, ssq[mt]);
-          else
-            b = xp[mt][c];
-        }
+        const bf16x8_t b = (in && xok[mt]) ? xp[mt][c] : zero_bf16x8();
         acc[mt] = mfma_16x16x32(a[u], b, acc[mt]);
       }
     }
   }
-
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][mt][lane][i] = acc[mt][i];
-    if (NORM) {
-      float s = ssq[mt];
-      s += __shfl_xor(s, 16, kWave);
-      s += __shfl_xor(s, 32, kWave);
-      if (q == 0) red_ssq[wave][mt][r] = s;
-    }
-  }
-  __syncthreads();
-  // wavefront w < MT finishes token tile w (MT <= WAVES)
-  if (wave < MT) {
-    const int mt = wave;
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int ww = 0; ww < WAVES; ++ww)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] += red[ww][mt][lane][i];
-    if (NORM) {
-      float total = 0.f;
-      for (int ww = 0; ww < WAVES; ++ww) total += red_ssq[ww][mt][r];
-      const float inv = 1.0f / sqrtf(total / static_cast<float>(K) + np.eps);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] *= inv;
-    }
-    const int m = mt * 16 + r;
-    const int n = n0 + q * 4;
-    if (m < M && n < N) store4(ep, m, n, N, v[0], v[1], v[2], v[3]);
+    const float v[4] = {acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]};
+    finish4(ep, blockIdx.y, slices, mt * 16 + r, n0 + q * 4, M, N, v);
   }
 }
 
@@ -343,30 +332,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     }
 }
 
-template <int MT, int WAVES>
-static void launch_skinny(const bf16* x, const bf16* w, const NormPrologue* np, const GemmEpilogue& ep, int m,
-                          int n, int k, hipStream_t stream) {
-  const unsigned grid = (n + 15) / 16;
-  if (np != nullptr)
-    gemm_skinny_kernel<MT, WAVES, true><<<grid, WAVES * 64, 0, stream>>>(x, w, *np, ep, m, n, k);
-  else
-    gemm_skinny_kernel<MT, WAVES, false><<<grid, WAVES * 64, 0, stream>>>(x, w, NormPrologue{}, ep, m, n, k);
+// K slices for a skinny product: enough workgroups to keep every compute unit
+// streaming, as long as a slice keeps a few MFMA steps.  1 unless `allowed`.
+static int choose_slices(int groups, int ksteps, int allowed) {
+  if (allowed <= 1) return 1;
+  int slices = 1;
+  while (slices < allowed && groups * slices < 256 && ksteps / (slices * 2) >= 8) slices *= 2;
+  return slices;
 }
 
-static int gemm_bf16(const bf16* xb, const bf16* wb, const NormPrologue* np, const GemmEpilogue& ep, int m, int n,
-                     int k, hipStream_t stream) {
-  if (m <= 64) {
-    const bool deep = k >= 2048;
-    if (m <= 16) {
-      if (deep) launch_skinny<1, 16>(xb, wb, np, ep, m, n, k, stream);
-      else launch_skinny<1, 4>(xb, wb, np, ep, m, n, k, stream);
-    } else if (m <= 32) {
-      if (deep) launch_skinny<2, 8>(xb, wb, np, ep, m, n, k, stream);
-      else launch_skinny<2, 4>(xb, wb, np, ep, m, n, k, stream);
-    } else {
-      if (deep) launch_skinny<4, 8>(xb, wb, np, ep, m, n, k, stream);
-      else launch_skinny<4, 4>(xb, wb, np, ep, m, n, k, stream);
-    }
+static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
+                     hipStream_t stream) {
+  if (m <= 16) {
+    dim3 grid((n + 15) / 16, slices);
+    gemm_skinny_split_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
+  } else if (m <= 64) {
+    dim3 grid((n + 63) / 64, slices);
+    if (m <= 32)
+      gemm_skinny_rows_kernel<2><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
+    else
+      gemm_skinny_rows_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
   } else {
     static bool configured = false;
     if (!configured) {
@@ -394,45 +379,34 @@ using namespace mlr;
 
 extern "C" {
 
+// How many K slices mlr_gemm_bf16 would use for this shape when the caller can take
+// partial sums (at most `max_slices`); 1 means it writes the finished product.
+int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
+  if (m > 64 || k % 8 != 0) return 1;
+  const int groups = m <= 16 ? (n + 15) / 16 : (n + 63) / 64;
+  return choose_slices(groups, (k / 8 + 3) / 4, max_slices);
+}
+
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
 // argument meanings.  Requires k % 8 == 0 and 16-byte aligned x and w.  With
 // `swiglu` the rows of w are (gate, gate, up, up) groups, there is no bias, n is
-// a multiple of 4 and y is [m, n / 2].
+// a multiple of 4 and y is [m, n / 2].  With slices > 1 (the value of
+// mlr_gemm_bf16_slices; not with swiglu) y is float32 [slices, m, n]: partial sums
+// over slices of k, the bias in slice 0, for the consumer to add up.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
-                  int swiglu, int m, int n, int k, hipStream_t stream) {
+                  int swiglu, int slices, int m, int n, int k, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
   MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
+  MLR_REQUIRE(slices >= 1 && slices <= 64, "slices must be within 1..64");
+  MLR_REQUIRE(slices == 1 || (m <= 64 && !swiglu && out_is_f32),
+              "partial sums are float32, for up to 64 tokens, without SwiGLU");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
               "x and w must be 16-byte aligned");
   GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
-  if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), nullptr, ep, m, n, k, stream) != 0)
+  if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, stream) != 0)
     return -1;
-  MLR_LAUNCH_CHECK();
-  return 0;
-}
-
-// The same product with the RMSNorm of its input fused in, for up to 64 tokens:
-// input = norm(x + delta) with x float32 [m, k], delta bfloat16 (may be null),
-// norm weight [k] (float32 when norm_weight_is_f32, else bfloat16); x + delta is
-// written to x_out (float32 [m, k], may be null; must not alias x).
-int mlr_gemm_bf16_norm(const float* x, const void* delta, const void* norm_weight, int norm_weight_is_f32,
-                       float eps, float* x_out, const void* w, const void* bias, int bias_is_f32, void* y,
-                       int out_is_f32, int swiglu, int m, int n, int k, hipStream_t stream) {
-  MLR_REQUIRE(x && norm_weight && w && y, "null pointer");
-  MLR_REQUIRE(m > 0 && m <= 64 && n > 0 && k > 0, "sizes must be > 0 and m <= 64");
-  MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
-  MLR_REQUIRE(eps >= 0.f, "eps must be >= 0");
-  MLR_REQUIRE(x_out != x, "x_out must not alias x");
-  MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
-  MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
-                  reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(norm_weight) % 16 == 0 &&
-                  reinterpret_cast<uintptr_t>(x_out) % 16 == 0,
-              "operands must be 16-byte aligned");
-  NormPrologue np{x, static_cast<const bf16*>(delta), norm_weight, norm_weight_is_f32, x_out, eps};
-  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
-  if (gemm_bf16(nullptr, static_cast<const bf16*>(w), &np, ep, m, n, k, stream) != 0) return -1;
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -19,7 +19,6 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from . import build
-from .deferred import DeferredNorm
 
 _VP = ctypes.c_void_p
 _I = ctypes.c_int
@@ -29,15 +28,15 @@ _F = ctypes.c_float
 _SIGNATURES = {
     "mlr_version": ([], _I),
     "mlr_embedding": ([_VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
-    "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
+    "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
-    "mlr_gather_rows": ([_VP, _VP, _VP, _I, _I64, _I, _VP], _I),
+    "mlr_gather_rows": ([_VP, _VP, _VP, _I, _I64, _I, _I, _VP], _I),
     "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_bf16_norm": ([_VP, _VP, _VP, _I, _F, _VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
         _I,
@@ -115,6 +114,7 @@ class HipOps:
             raise KernelError("the built kernel library is of another version than this package")
         self._attention_libs: dict[int, ctypes.CDLL] = {}
         self.decode_partition = int(os.environ.get("MLR_DECODE_PARTITION", "256"))
+        self.max_k_slices = int(os.environ.get("MLR_MAX_K_SLICES", "16"))
 
     def attention_library(self, head_dim: int) -> ctypes.CDLL:
         """The MFMA attention kernels of one head size, compiled on first use."""
@@ -180,14 +180,22 @@ class HipOps:
     def rmsnorm(
         self, x: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor] = None
     ) -> torch.Tensor:
+        """x (float32 residual stream [rows, hidden]) += delta in place, then the RMSNorm of x
+        in the engine's dtype.  delta: [rows, hidden] in the engine's dtype, or a float32 stack
+        [S, rows, hidden] of partial sums (see `linear`), or None."""
         self._check(x, "residual stream", torch.float32, (None, None))
         rows, hidden = x.shape
         self._check(weight, "norm weight", (torch.float32, self.dtype), (hidden,))
-        if delta is not None:
-            self._check(delta, "residual delta", self.dtype, (rows, hidden))
+        plain = partial = None
+        slices = 0
+        if delta is not None and delta.dim() == 3:
+            partial = self._check(delta, "partial sums", torch.float32, (None, rows, hidden))
+            slices = delta.shape[0]
+        elif delta is not None:
+            plain = self._check(delta, "residual delta", self.dtype, (rows, hidden))
         out = self._empty((rows, hidden), self.dtype)
         self._call(
-            "mlr_rmsnorm", self._ptr(x), self._ptr(delta), self._ptr(weight),
+            "mlr_rmsnorm", self._ptr(x), self._ptr(plain), self._ptr(partial), slices, self._ptr(weight),
             int(weight.dtype == torch.float32), self._ptr(out), self.code, rows, hidden, float(eps), self._stream(),
         )
         return out
@@ -198,27 +206,34 @@ class HipOps:
         self._call("mlr_add", self._ptr(x), self._ptr(delta), self.code, x.numel(), self._stream())
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
-        self._check(x, "rows source", (torch.float32, torch.bfloat16), (None, None))
+        """x[rows] for x [T, H], or x[:, rows] for a stack [S, T, H]."""
+        self._check(x, "rows source", (torch.float32, torch.bfloat16))
+        if x.dim() not in (2, 3):
+            raise KernelError("gather_rows takes [T, H] or [S, T, H]")
         self._check(rows, "row indices", torch.int32, (None,))
-        row_bytes = x.shape[1] * x.element_size()
+        planes = x.shape[0] if x.dim() == 3 else 1
+        src_rows, width = x.shape[-2], x.shape[-1]
+        row_bytes = width * x.element_size()
         if row_bytes % 4:
             raise KernelError("gather_rows needs rows that are a multiple of 4 bytes wide")
-        out = self._empty((rows.shape[0], x.shape[1]), x.dtype)
+        shape = (planes, rows.shape[0], width) if x.dim() == 3 else (rows.shape[0], width)
+        out = self._empty(shape, x.dtype)
         self._call(
             "mlr_gather_rows", self._ptr(x), self._ptr(rows), self._ptr(out), rows.shape[0], row_bytes,
-            x.shape[0], self._stream(),
+            src_rows, planes, self._stream(),
         )
         return out
 
     # ---- matrix products ----------------------------------------------------------------------
     def linear(
         self,
-        x: Union[torch.Tensor, DeferredNorm],
+        x: torch.Tensor,
         weight: torch.Tensor,
         bias: Optional[torch.Tensor] = None,
         out_dtype: Optional[torch.dtype] = None,
         kernel: str = "auto",
         swiglu: bool = False,
+        partial_sums: bool = False,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
 
@@ -226,18 +241,15 @@ class HipOps:
         products, and everything with kernel="fma", run as plain 32-bit FMA arithmetic.
         swiglu: the rows of `weight` are groups (gate 2j, gate 2j+1, up 2j, up 2j+1) and
         the result is silu(gate) * up, [M, N / 2].
-        x may be a DeferredNorm: for up to 64 tokens its addition and norm run inside
-        the matrix-core kernel; otherwise it is computed first.
+        partial_sums: the caller hands the result to a norm as a not-yet-added delta and
+        accepts, instead of [M, N], a float32 stack [S, M, N] of partial sums over slices
+        of k (bias in slice 0).  Narrow products of a few tokens are cut that way so that
+        all compute units stream the weight; the norm kernel adds the slices in order.
         """
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
-        deferred = x if isinstance(x, DeferredNorm) else None
-        if deferred is not None:
-            stream_x, delta = deferred.inputs()
-            m, k = stream_x.shape
-        else:
-            self._check(x, "linear input", self.dtype, (None, None))
-            m, k = x.shape
+        self._check(x, "linear input", self.dtype, (None, None))
+        m, k = x.shape
         self._check(weight, "linear weight", self.dtype, (None, k))
         n = weight.shape[0]
         if bias is not None:
@@ -247,34 +259,26 @@ class HipOps:
         out_dtype = out_dtype or self.dtype
         if out_dtype not in (torch.float32, self.dtype):
             raise KernelError(f"linear output must be float32 or {self.dtype}")
-        y = self._empty((m, n // 2 if swiglu else n), out_dtype)
         bias_f32 = int(bias is not None and bias.dtype == torch.float32)
-        out_f32 = int(out_dtype == torch.float32)
-        mfma = kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0
-        if deferred is not None:
-            if mfma and m <= 64 and not deferred.materialized:
-                self._check(stream_x, "residual stream", torch.float32, (m, k))
-                self._check(deferred.weight, "norm weight", (torch.float32, self.dtype), (k,))
-                if delta is not None:
-                    self._check(delta, "residual delta", self.dtype, (m, k))
-                x_out = self._empty((m, k), torch.float32) if delta is not None else None
-                self._call(
-                    "mlr_gemm_bf16_norm", self._ptr(stream_x), self._ptr(delta), self._ptr(deferred.weight),
-                    int(deferred.weight.dtype == torch.float32), deferred.eps, self._ptr(x_out), self._ptr(weight),
-                    self._ptr(bias), bias_f32, self._ptr(y), out_f32, int(swiglu), m, n, k, self._stream(),
-                )
-                deferred.fused(x_out)
-                return y
-            x = deferred.tensor()
-        if mfma:
+        if kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0:
+            slices = 1
+            if partial_sums and not swiglu:
+                slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices)
+            if slices > 1:
+                y = self._empty((slices, m, n), torch.float32)
+                out_f32 = 1
+            else:
+                y = self._empty((m, n // 2 if swiglu else n), out_dtype)
+                out_f32 = int(out_dtype == torch.float32)
             self._call(
                 "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-                int(swiglu), m, n, k, self._stream(),
+                int(swiglu), slices, m, n, k, self._stream(),
             )
             return y
+        y = self._empty((m, n // 2 if swiglu else n), out_dtype)
         self._call(
-            "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-            int(swiglu), self.code, m, n, k, self._stream(),
+            "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
+            int(out_dtype == torch.float32), int(swiglu), self.code, m, n, k, self._stream(),
         )
         return y
 

@@ -33,8 +33,6 @@ class GQAAttention(Mixer):
     [Wq; Wk; Wv] (made by the weight rules at load time).
     """
 
-    accepts_deferred_norm = True
-
     def __init__(
         self,
         hidden_size: int,
@@ -128,4 +126,4 @@ class GQAAttention(Mixer):
             scale=self.scale,
             window=self.window,
         )
-        return ops.linear(attended, self.o_weight, self.o_bias_vec)
+        return ops.linear(attended, self.o_weight, self.o_bias_vec, partial_sums=True)

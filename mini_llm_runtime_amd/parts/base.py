@@ -33,13 +33,10 @@ class Part:
 class Norm(Part):
     def forward(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x: float32 residual stream [T, H].  When `delta` is given, first x += delta
-        (in place, summed in 32-bit); returns norm(x) in the engine's dtype."""
+        (in place, summed in 32-bit); returns norm(x) in the engine's dtype.  `delta` is a
+        part's output: [T, H] in the engine's dtype, or, from a part that ends in
+        `ops.linear(..., partial_sums=True)`, a float32 stack [S, T, H] whose sum over S it is."""
         raise NotImplementedError
-
-    def defer(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None):
-        """Optional: a `DeferredNorm` that a part with `accepts_deferred_norm` may fuse
-        into its first matrix product.  None: this norm is always computed by `forward`."""
-        return None
 
 
 class PositionEncoding(Part):
@@ -55,9 +52,6 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    # True: `forward` may receive a DeferredNorm instead of a tensor and hands it to ops.linear
-    accepts_deferred_norm = False
-
     def cache_spec(self) -> Any:
         """PagedKVSpec, SlotStateSpec or None."""
         return None
@@ -68,8 +62,6 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    accepts_deferred_norm = False
-
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

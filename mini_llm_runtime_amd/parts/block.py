@@ -39,20 +39,10 @@ class PreNormBlock(Block):
             "norm_post_mixer": self.norm_post_mixer,
         }
 
-    @staticmethod
-    def _normed(ctx: StepContext, norm: Norm, part: Part, x: torch.Tensor, delta: Optional[torch.Tensor]):
-        """(what the part receives, a function that gives the residual stream afterwards)."""
-        deferred = norm.defer(ctx, x, delta) if getattr(part, "accepts_deferred_norm", False) else None
-        if deferred is not None:
-            return deferred, lambda: deferred.residual
-        return norm.forward(ctx, x, delta), lambda: x
-
     def forward(
         self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor], site: int
     ) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
-        h, residual = self._normed(ctx, self.norm_input, self.mixer, x, delta)
+        h = self.norm_input.forward(ctx, x, delta)
         mixed = self.mixer.forward(ctx, h, site)
-        x = residual()
-        h, residual = self._normed(ctx, self.norm_post_mixer, self.feed_forward, x, mixed)
-        out = self.feed_forward.forward(ctx, h)
-        return residual(), out
+        h = self.norm_post_mixer.forward(ctx, x, mixed)
+        return x, self.feed_forward.forward(ctx, h)

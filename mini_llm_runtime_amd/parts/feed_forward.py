@@ -22,8 +22,6 @@ class SwiGLU(FeedForward):
     silu(gate) * up is that product's epilogue.
     """
 
-    accepts_deferred_norm = True
-
     def __init__(self, hidden_size: int, intermediate_size: int) -> None:
         if hidden_size <= 0 or intermediate_size <= 0 or intermediate_size % 2:
             raise ValueError("SwiGLU sizes must be > 0 and the intermediate size even")
@@ -41,4 +39,4 @@ class SwiGLU(FeedForward):
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
         hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
-        return ops.linear(hidden, self.down_weight, None)
+        return ops.linear(hidden, self.down_weight, None, partial_sums=True)

@@ -125,9 +125,7 @@ class DecoderModel:
             return None
         rows = ops.gather_rows(x, logit_rows)
         delta_rows = ops.gather_rows(delta, logit_rows) if delta is not None else None
-        h = self.final_norm.defer(ctx, rows, delta_rows)
-        if h is None:
-            h = self.final_norm.forward(ctx, rows, delta_rows)
+        h = self.final_norm.forward(ctx, rows, delta_rows)
         return ops.linear(h, self.head_weight, None, out_dtype=torch.float32)
 
 

@@ -6,7 +6,6 @@ from typing import Optional
 
 import torch
 
-from ..kernels.deferred import DeferredNorm
 from .base import Norm
 from .context import StepContext
 from .registry import register_part
@@ -35,5 +34,3 @@ class RMSNorm(Norm):
     def forward(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ctx.ops.rmsnorm(x, self.weight, self.eps, delta=delta)
 
-    def defer(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> DeferredNorm:
-        return DeferredNorm(ctx.ops, x, delta, self.weight, self.eps)

@@ -16,8 +16,6 @@ from typing import Optional
 
 import torch
 
-from mini_llm_runtime_amd.kernels.deferred import DeferredNorm
-
 
 class TorchOps:
     def __init__(self, dtype: torch.dtype = torch.float32, device: str = "cpu") -> None:
@@ -37,7 +35,7 @@ class TorchOps:
         self._count("rmsnorm")
         assert x.dtype == torch.float32
         if delta is not None:
-            x += delta.float()
+            x += delta.float().sum(0) if delta.dim() == 3 else delta.float()
         variance = x.pow(2).mean(-1, keepdim=True)
         return (weight.float() * (x * torch.rsqrt(variance + eps))).to(self.dtype)
 
@@ -45,13 +43,11 @@ class TorchOps:
         x += delta.float()
 
     def gather_rows(self, x, rows):
-        return x[rows.long()].contiguous()
+        return (x[:, rows.long()] if x.dim() == 3 else x[rows.long()]).contiguous()
 
     # matrix products ---------------------------------------------------------------------
-    def linear(self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False):
+    def linear(self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False):
         self._count("linear")
-        if isinstance(x, DeferredNorm):
-            x = x.tensor()
         y = x.float() @ weight.float().t()
         if bias is not None:
             y = y + bias.float()

@@ -172,34 +172,37 @@ def test_linear_swiglu_epilogue(ops_for, dtype, m, inter, k):
         torch.testing.assert_close(got.double(), ref, **tol)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 1152, 896), (8, 9728, 896), (16, 130, 64), (33, 517, 2056), (64, 96, 4864)])
-@pytest.mark.parametrize("weight_f32", [False, True])
-@pytest.mark.parametrize("with_delta", [False, True])
-def test_linear_with_fused_norm(ops_for, m, n, k, weight_f32, with_delta):
-    """x += delta, RMSNorm and the product in one kernel against the three separate steps in float64."""
-    from mini_llm_runtime_amd.kernels.deferred import DeferredNorm
-
+@pytest.mark.parametrize("m,n,k", [(1, 896, 4864), (8, 896, 896), (16, 130, 2056), (33, 517, 2056), (64, 896, 4864), (8, 151936, 96)])
+def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
+    """A narrow product of a few tokens may come back as float32 partial sums over slices of k;
+    the norm kernel adds them, in order, to the residual stream."""
     ops = ops_for(torch.bfloat16)
-    x = _rand((m, k), torch.float32, 46, 2.0)
-    delta = _rand((m, k), torch.bfloat16, 47) if with_delta else None
-    nw = (1 + _rand((k,), torch.float32, 48, 0.1)).to(torch.float32 if weight_f32 else torch.bfloat16)
-    w = _rand((n, k), torch.bfloat16, 49, 0.05)
-    b = _rand((n,), torch.float32, 50)
-    eps = 1e-6
-    summed = x.double() + (delta.double() if with_delta else 0)
-    ref = plain.rms_norm(summed, nw.double(), eps) @ w.double().t() + b.double()
-    xd = x.cuda()
-    deferred = DeferredNorm(ops, xd, delta.cuda() if with_delta else None, nw.cuda(), eps)
-    got = ops.linear(deferred, w.cuda(), b.cuda(), out_dtype=torch.float32).cpu()
-    # the kernel rounds (x * norm weight) to bfloat16 before the product: one rounding per input element
-    torch.testing.assert_close(got.double(), ref, atol=3e-2 * float(ref.abs().max()) / 4, rtol=1.6e-2)
-    assert float((got.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()) < 4e-3
-    torch.testing.assert_close(deferred.residual.cpu().double(), summed, atol=1e-6, rtol=1e-6)
-    if with_delta:
-        assert torch.equal(xd.cpu(), x), "the fused kernel must not write into its input stream"
-    # a second consumer of the same deferred norm gets the separately computed activations
-    again = ops.linear(deferred, w.cuda(), b.cuda(), out_dtype=torch.float32).cpu()
-    assert float((again.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()) < 4e-3
+    x = _rand((m, k), torch.bfloat16, 46)
+    w = _rand((n, k), torch.bfloat16, 47, 0.05)
+    b = _rand((n,), torch.float32, 48)
+    ref = x.double() @ w.double().t() + b.double()
+    got = ops.linear(x.cuda(), w.cuda(), b.cuda(), partial_sums=True)
+    if got.dim() == 3:
+        assert got.dtype == torch.float32 and got.shape[1:] == (m, n) and got.shape[0] > 1
+        total = got.cpu().double().sum(0)
+    else:
+        assert got.shape == (m, n)  # wide enough: not cut
+        total = got.cpu().double()
+    torch.testing.assert_close(total, ref, **(_tol(torch.bfloat16) if got.dim() == 2 else dict(atol=2e-3, rtol=1e-4)))
+    if k == 4864:
+        assert got.dim() == 3, "a long, narrow product should be cut along k"
+    stream = _rand((m, n), torch.float32, 49, 2.0)
+    nw = (1 + _rand((n,), torch.float32, 50, 0.1)).to(torch.bfloat16)
+    sd = stream.cuda().clone()
+    h = ops.rmsnorm(sd, nw.cuda(), 1e-6, delta=got).cpu()
+    summed = stream.double() + (total if got.dim() == 3 else got.cpu().double())
+    torch.testing.assert_close(sd.cpu().double(), summed, atol=1e-5, rtol=1e-6)
+    torch.testing.assert_close(h.double(), plain.rms_norm(summed, nw.double(), 1e-6), **_tol(torch.bfloat16))
+    again = ops.linear(x.cuda(), w.cuda(), b.cuda(), partial_sums=True)
+    assert torch.equal(again, got), "partial sums must not depend on timing"
+    rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
+    picked = ops.gather_rows(got, rows).cpu()
+    assert torch.equal(picked, got.cpu()[..., [m - 1, 0], :])
 
 
 # ---- rotary encoding and cache write ----------------------------------------------------------------
