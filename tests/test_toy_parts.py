@@ -1,0 +1,345 @@
+"""Generality of the parts: toy parts that exist only in this file are registered,
+built into a model by config.json, given random weights, loaded and stepped,
+without a change to the framework's files.
+
+* a mixer with state of its own (a causal running mean kept in a per-request
+  state slot), in layers that alternate with attention layers;
+* an execution order that names a layer twice (two sites, two caches) and lets a
+  site read another site's cache;
+* attention layers with a window beside layers without (two page pools);
+* another position encoding (a learned-free additive ramp applied to q and k).
+
+None of them is a model of anybody's; they only show that the interfaces hold.
+Each is compared with a plain computation written out in this file, whole and in
+portions.
+"""
+
+from __future__ import annotations
+
+import json
+import math
+from dataclasses import dataclass, fields
+from typing import Any, ClassVar, Mapping
+
+import pytest
+import torch
+
+import mini_llm_runtime_amd as mlr
+import plain_qwen2 as plain
+from helpers import random_tokens
+from kernel_doubles import TorchOps
+from mini_llm_runtime_amd.cache import PagedKVSpec, SlotStateSpec
+from mini_llm_runtime_amd.config.model_config import ModelConfig
+from mini_llm_runtime_amd.engine import ModelRunner, StepEntry
+from mini_llm_runtime_amd.models import register_architecture, unregister_architecture
+from mini_llm_runtime_amd.parts import (
+    LayerSpec,
+    Mixer,
+    ModelSpec,
+    OrderEntry,
+    ParamSpec,
+    PartSpec,
+    PositionEncoding,
+    WeightRule,
+    register_part,
+    unregister_part,
+)
+from mini_llm_runtime_amd.weights import SafetensorsFile
+
+CASES = [
+    pytest.param("double", torch.float32, id="double-f32"),
+    pytest.param("hip", torch.float32, id="hip-f32", marks=pytest.mark.gpu),
+    pytest.param("hip", torch.bfloat16, id="hip-bf16", marks=pytest.mark.gpu),
+]
+
+
+def _ops(backend, dtype):
+    if backend == "double":
+        return TorchOps(dtype, "cpu")
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    return HipOps(dtype, "cuda")
+
+
+# ---- toy parts -------------------------------------------------------------------------------------
+class RunningMeanMixer(Mixer):
+    """out_t = W_out * mean_{i <= t}(W_in h_i): state = the running sum, one vector per request."""
+
+    def __init__(self, hidden_size: int) -> None:
+        self.hidden_size = hidden_size
+        self.in_weight = None
+        self.out_weight = None
+
+    def param_specs(self):
+        h = self.hidden_size
+        return {"in_weight": ParamSpec((h, h)), "out_weight": ParamSpec((h, h))}
+
+    def cache_spec(self):
+        return SlotStateSpec((self.hidden_size,), "float32")
+
+    def forward(self, ctx, h, site):
+        ops = ctx.ops
+        u = ops.linear(h, self.in_weight, None).float()
+        state = ctx.state(site)
+        out = torch.empty_like(u)
+        lay = ctx.host
+        for r in range(lay.num_entries):
+            a, b = int(lay.cu_q[r]), int(lay.cu_q[r + 1])
+            start = int(lay.q_starts[r])
+            running = torch.cumsum(u[a:b], dim=0)
+            if start > 0:
+                running = running + state.tensor[int(lay.state_read[r])]
+            counts = torch.arange(start + 1, start + 1 + (b - a), device=u.device, dtype=torch.float32)
+            out[a:b] = running / counts[:, None]
+            state.tensor[int(lay.state_write[r])] = running[-1]
+        return ops.linear(out.to(ctx.dtype), self.out_weight, None)
+
+
+class RampPosition(PositionEncoding):
+    """q and k get `slope * position` added to their first dim: not a rotation, so the
+    attention part has to call `apply` and store k without the fused rotation."""
+
+    def __init__(self, head_dim: int, slope: float) -> None:
+        self.head_dim = head_dim
+        self.slope = slope
+
+    def apply(self, ctx, q, k):
+        ramp = (ctx.positions.float() * self.slope)[:, None]
+        q[:, :, 0] = (q[:, :, 0].float() + ramp).to(q.dtype)
+        k[:, :, 0] = (k[:, :, 0].float() + ramp).to(k.dtype)
+
+
+@dataclass(frozen=True)
+class ToyConfig(ModelConfig):
+    architecture: ClassVar[str] = "ToyForCausalLM"
+    model_type: ClassVar[str] = "toy"
+    vocab_size: int = 0
+    hidden_size: int = 0
+    intermediate_size: int = 0
+    num_attention_heads: int = 0
+    num_key_value_heads: int = 0
+    head_dim: int = 0
+    max_position_embeddings: int = 0
+    rms_norm_eps: float = 1e-6
+    layer_kinds: tuple = ()  # per layer: "mean", "attention", "window", "ramp"
+    order: tuple = ()  # execution sites: (layer, reads_cache_of or -1)
+    window: int = 0
+    rope_theta: float = 10000.0
+    ramp_slope: float = 0.01
+
+    @classmethod
+    def from_dict(cls, data: Mapping[str, Any]) -> "ToyConfig":
+        names = [f.name for f in fields(cls)]
+        kw = {n: data[n] for n in names if n in data}
+        kw["layer_kinds"] = tuple(kw["layer_kinds"])
+        kw["order"] = tuple(tuple(o) for o in kw["order"])
+        return cls(**kw)
+
+    def to_dict(self):
+        d = super().to_dict()
+        d["layer_kinds"] = list(self.layer_kinds)
+        d["order"] = [list(o) for o in self.order]
+        return d
+
+
+def toy_spec(c: ToyConfig) -> ModelSpec:
+    norm = PartSpec("rms_norm", {"size": c.hidden_size, "eps": c.rms_norm_eps})
+    ffn = PartSpec("swiglu", {"hidden_size": c.hidden_size, "intermediate_size": c.intermediate_size})
+    q_rows, kv_rows = c.num_attention_heads * c.head_dim, c.num_key_value_heads * c.head_dim
+    layers, rules = [], [WeightRule("embed.weight", "embed.weight"), WeightRule("norm.weight", "final_norm.weight")]
+    for i, kind in enumerate(c.layer_kinds):
+        p = f"layers.{i}."
+        if kind == "mean":
+            mixer = PartSpec("toy_running_mean", {"hidden_size": c.hidden_size})
+            rules += [WeightRule(p + "mean.in", p + "mixer.in_weight"), WeightRule(p + "mean.out", p + "mixer.out_weight")]
+        else:
+            position = (
+                PartSpec("toy_ramp", {"head_dim": c.head_dim, "slope": c.ramp_slope})
+                if kind == "ramp"
+                else PartSpec("rotary", {"head_dim": c.head_dim, "theta": c.rope_theta})
+            )
+            mixer = PartSpec(
+                "gqa_attention",
+                {
+                    "hidden_size": c.hidden_size,
+                    "num_heads": c.num_attention_heads,
+                    "num_kv_heads": c.num_key_value_heads,
+                    "head_dim": c.head_dim,
+                    "qkv_bias": False,
+                    "position": position,
+                    "window": c.window if kind == "window" else None,
+                },
+            )
+            rules += [
+                WeightRule(p + "attn.q", p + "mixer.qkv_weight", 0, q_rows),
+                WeightRule(p + "attn.k", p + "mixer.qkv_weight", q_rows, kv_rows),
+                WeightRule(p + "attn.v", p + "mixer.qkv_weight", q_rows + kv_rows, kv_rows),
+                WeightRule(p + "attn.o", p + "mixer.o_weight"),
+            ]
+        rules += [
+            WeightRule(p + "norm1", p + "norm_input.weight"),
+            WeightRule(p + "norm2", p + "norm_post_mixer.weight"),
+            WeightRule(p + "ffn.gate", p + "feed_forward.gate_up_weight", 0, c.intermediate_size, block=2, period=4),
+            WeightRule(p + "ffn.up", p + "feed_forward.gate_up_weight", 2, c.intermediate_size, block=2, period=4),
+            WeightRule(p + "ffn.down", p + "feed_forward.down_weight"),
+        ]
+        layers.append(LayerSpec("pre_norm", mixer, ffn, {"input": norm, "post_mixer": norm}))
+    return ModelSpec(
+        architecture=c.architecture,
+        vocab_size=c.vocab_size,
+        hidden_size=c.hidden_size,
+        max_position_embeddings=c.max_position_embeddings,
+        layers=tuple(layers),
+        order=tuple(OrderEntry(l, None if src < 0 else src) for l, src in c.order),
+        final_norm=norm,
+        tie_word_embeddings=True,
+        weight_rules=tuple(rules),
+        init_std=0.05,
+    )
+
+
+@pytest.fixture()
+def toy_registered():
+    register_part("mixer", "toy_running_mean", RunningMeanMixer, replace=True)
+    register_part("position", "toy_ramp", RampPosition, replace=True)
+    register_architecture("ToyForCausalLM", ToyConfig, toy_spec, replace=True)
+    yield
+    unregister_architecture("ToyForCausalLM")
+    unregister_part("mixer", "toy_running_mean")
+    unregister_part("position", "toy_ramp")
+
+
+# ---- the plain computation of the same toy model ------------------------------------------------------
+def toy_plain(tokens, w, c: ToyConfig):
+    x = w["embed.weight"].double()[torch.tensor(tokens)]
+    n = len(tokens)
+    pos = torch.arange(n)
+    cached_kv = {}
+    for site, (layer, src) in enumerate(c.order):
+        p = f"layers.{layer}."
+        kind = c.layer_kinds[layer]
+        h = plain.rms_norm(x, w[p + "norm1"].double(), c.rms_norm_eps)
+        if kind == "mean":
+            u = h @ w[p + "mean.in"].double().t()
+            mean = torch.cumsum(u, 0) / torch.arange(1, n + 1)[:, None]
+            mixed = mean @ w[p + "mean.out"].double().t()
+        else:
+            hq, hkv, d = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+            q = (h @ w[p + "attn.q"].double().t()).view(n, hq, d).transpose(0, 1)
+            if src < 0:
+                k = (h @ w[p + "attn.k"].double().t()).view(n, hkv, d).transpose(0, 1)
+                v = (h @ w[p + "attn.v"].double().t()).view(n, hkv, d).transpose(0, 1)
+            if kind == "ramp":
+                q = q.clone()
+                q[:, :, 0] += pos * c.ramp_slope
+                if src < 0:
+                    k = k.clone()
+                    k[:, :, 0] += pos * c.ramp_slope
+            else:
+                q = plain.apply_rope(q, pos, c.rope_theta)
+                if src < 0:
+                    k = plain.apply_rope(k, pos, c.rope_theta)
+            if src < 0:
+                cached_kv[site] = (k, v)
+            else:
+                k, v = cached_kv[src]  # this site reads the other site's keys and values
+            att = plain.causal_attention(q, k, v, window=c.window if kind == "window" else None)
+            mixed = att.transpose(0, 1).reshape(n, hq * d) @ w[p + "attn.o"].double().t()
+        x = x + mixed
+        h = plain.rms_norm(x, w[p + "norm2"].double(), c.rms_norm_eps)
+        g = h @ w[p + "ffn.gate"].double().t()
+        x = x + (g * torch.sigmoid(g) * (h @ w[p + "ffn.up"].double().t())) @ w[p + "ffn.down"].double().t()
+    x = plain.rms_norm(x, w["norm.weight"].double(), c.rms_norm_eps)
+    return x @ w["embed.weight"].double().t()
+
+
+TOYS = {
+    # a mixer with state of its own between attention layers; layer 1 runs twice
+    "state": dict(layer_kinds=["attention", "mean", "attention"], order=[[0, -1], [1, -1], [2, -1], [1, -1]], window=0),
+    # window layers beside full layers (two page pools), a site that reads another site's cache, another position encoding
+    "window": dict(layer_kinds=["window", "attention", "ramp"], order=[[0, -1], [1, -1], [2, -1], [1, 1], [0, -1]], window=11),
+}
+
+
+def _toy_config(name):
+    base = dict(
+        architectures=["ToyForCausalLM"], model_type="toy", vocab_size=97, hidden_size=48, intermediate_size=80,
+        num_attention_heads=3, num_key_value_heads=1, head_dim=16, max_position_embeddings=256, rms_norm_eps=1e-5,
+    )
+    base.update(TOYS[name])
+    return base
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("name", list(TOYS))
+def test_toy_model_whole_and_in_portions(tmp_path, toy_registered, name, backend, dtype):
+    config = mlr.models.config_from_dict(_toy_config(name))
+    assert isinstance(config, ToyConfig)
+    folder = mlr.write_random_model(config, tmp_path / name, seed=7)
+    assert json.loads((folder / "config.json").read_text())["architectures"] == ["ToyForCausalLM"]
+    with SafetensorsFile(folder / "model.safetensors") as f:
+        weights = {n: f.tensor(n) for n in f.entries}
+    ops = _ops(backend, dtype)
+    cfg, model = mlr.load_model(folder, dtype=dtype, device=ops.device)
+    specs = model.site_cache_specs()
+    if name == "state":
+        assert [type(s).__name__ for s in specs] == ["PagedKVSpec", "SlotStateSpec", "PagedKVSpec", "SlotStateSpec"]
+    else:
+        assert specs[3] is None and specs[0] == PagedKVSpec(1, 16, 11) and specs[1] == PagedKVSpec(1, 16, None)
+    cache = mlr.make_cache(model, block_size=4, num_blocks=24, max_requests=3)
+    if name == "window":
+        assert len(cache.groups) == 2 and cache.groups[0].sites == (0, 4) and cache.groups[1].sites == (1, 2)
+    cache.poison()
+    runner = ModelRunner(model, cache, ops)
+    requests = {"a": random_tokens(45, 97, 1), "b": random_tokens(23, 97, 2)}
+    refs = {rid: toy_plain(toks, weights, config) for rid, toks in requests.items()}
+
+    def check(got, rid, base):
+        ref = refs[rid][base : base + got.shape[0]]
+        err = (got.double().cpu() - ref).abs().max() / ref.abs().max()
+        assert err < (1e-4 if dtype == torch.float32 else 4e-2), (rid, base, float(err))
+
+    # whole
+    for rid, toks in requests.items():
+        cache.create_request(rid)
+        out = runner.step([StepEntry.of(rid, toks, range(len(toks)))])
+        check(out.logits, rid, 0)
+        cache.release_request(rid)
+    # portions, both requests in one batch, single tokens at the end, one aborted step in between
+    fed = {rid: 0 for rid in requests}
+    for rid in requests:
+        cache.create_request(rid)
+    sizes = [5, 2, 9, 3, 1, 1, 7, 1, 4, 6, 1, 1, 1, 8, 2]
+    i = 0
+    while any(fed[r] < len(requests[r]) for r in requests):
+        entries = []
+        for rid, toks in requests.items():
+            n = min(sizes[(i + (rid == "b")) % len(sizes)], len(toks) - fed[rid])
+            if n > 0:
+                entries.append(StepEntry.of(rid, toks[fed[rid] : fed[rid] + n], range(n)))
+        if i == 3:  # a failed step must leave pages and state as they were
+            runner.fail_next_step = RuntimeError("injected")
+            with pytest.raises(RuntimeError, match="injected"):
+                runner.step(entries)
+        out = runner.step(entries)
+        at = 0
+        for e in entries:
+            check(out.logits[at : at + len(e.tokens)], e.request_id, fed[e.request_id])
+            at += len(e.tokens)
+            fed[e.request_id] += len(e.tokens)
+        i += 1
+        cache.check_invariants()
+    if name == "window":  # the window pool gave pages back while the full pool kept them
+        a = cache.get_request("a")
+        assert a.tables[0][0] == -1 and len(a.live_blocks(0)) < len(a.live_blocks(1))
+    for rid in requests:
+        cache.release_request(rid)
+    assert all(g.allocator.free_count == g.num_blocks for g in cache.groups)
+
+
+def test_unknown_part_kind_is_named(toy_registered):
+    bad = _toy_config("state")
+    config = mlr.models.config_from_dict(bad)
+    unregister_part("mixer", "toy_running_mean")
+    with pytest.raises(KeyError, match="toy_running_mean.*gqa_attention"):
+        mlr.build_model(config)
