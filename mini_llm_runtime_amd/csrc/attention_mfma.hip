@@ -83,7 +83,8 @@ __device__ __forceinline__ f32x4_t score_tile(const RowOperand& k, const RowOper
   return s;
 }
 
-// Running softmax state of one column (row of the attention problem) in a lane.
+// Running softmax state of one column (row of the attention problem) in a lane, in base 2:
+// m is the running maximum of score * scale * log2(e).
 struct Softmax {
   float m;
   float l;  // this lane's share of the sum (its own 4 keys of every tile)
@@ -91,29 +92,31 @@ struct Softmax {
 
 // Fold a tile of 4 scores into the state; returns the probabilities as the B
 // operand of the value product and the factor the accumulator must be scaled by.
-__device__ __forceinline__ s16x4_t softmax_tile(Softmax& st, f32x4_t s, const bool (&ok)[4], float scale,
+__device__ __forceinline__ s16x4_t softmax_tile(Softmax& st, f32x4_t s, const bool (&ok)[4], float scale2,
                                                 float& alpha) {
-  float v[4];
   float tmax = -INFINITY;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    v[i] = ok[i] ? s[i] * scale : -INFINITY;
-    tmax = fmaxf(tmax, v[i]);
+    if (!ok[i]) s[i] = -INFINITY;
+    tmax = fmaxf(tmax, s[i]);
   }
   tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
   tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-  const float m_new = fmaxf(st.m, tmax);
-  alpha = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_new);
+  const float m_new = fmaxf(st.m, tmax * scale2);
+  const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+  alpha = fast_exp2(st.m - m_use);
   float p[4];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    p[i] = (v[i] == -INFINITY) ? 0.f : __expf(v[i] - m_new);
+    p[i] = fast_exp2(fmaf(s[i], scale2, -m_use));
     sum += p[i];
   }
   st.l = st.l * alpha + sum;
   st.m = m_new;
-  return pack_bf16x4(p[0], p[1], p[2], p[3]);
+  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+  const u32x2_t packed = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3])};
+  return __builtin_bit_cast(s16x4_t, packed);
 }
 
 // ---- decode ---------------------------------------------------------------------------------
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
       }
     }
     float alpha;
-    const s16x4_t pb = softmax_tile(sm, s, ok, scale, alpha);
+    const s16x4_t pb = softmax_tile(sm, s, ok, scale * 1.44269504088896340736f, alpha);
 #pragma unroll
     for (int dt = 0; dt < kDimTiles; ++dt) {
 #pragma unroll
@@ -282,7 +285,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     float num = 0.f, den = 0.f;
 #pragma unroll
     for (int w = 0; w < kDecodeWaves; ++w) {
-      const float wgt = (sm_m[w][c] == -INFINITY) ? 0.f : __expf(sm_m[w][c] - mstar);
+      const float wgt = (sm_m[w][c] == -INFINITY) ? 0.f : fast_exp2(sm_m[w][c] - mstar);
       num += wgt * sm_acc[w][c][d];
       den += wgt * sm_l[w][c];
     }
@@ -324,8 +327,8 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
     const float ls = sp < splits ? src[sp * kPartialStride + D + 1] : 0.f;
     const float round_max = wave_max(ms);
     const float m_new = fmaxf(mstar, round_max);
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m_new);
-    const float rescale = (mstar == -INFINITY) ? 0.f : __expf(mstar - m_new);
+    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - m_new);
+    const float rescale = (mstar == -INFINITY) ? 0.f : fast_exp2(mstar - m_new);
     den = den * rescale + wave_sum(w * ls);
     mstar = m_new;
   }
@@ -334,7 +337,7 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
   for (int j = 0; j < (D + kWave - 1) / kWave; ++j) num[j] = 0.f;
   for (int sp = 0; sp < splits; ++sp) {
     const float ms = src[sp * kPartialStride + D];
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - mstar);
+    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - mstar);
 #pragma unroll
     for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
       const int d = lane + j * kWave;
@@ -349,20 +352,31 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 }
 
 // ---- prefill ----------------------------------------------------------------------------------
-constexpr int kTileQ = 64;   // queries per workgroup (16 per wavefront)
+constexpr int kTileQ = 64;                 // queries per workgroup (16 per wavefront)
 constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounded by LDS)
-constexpr int kKLd = D + 8;  // padded key row in LDS (elements)
+constexpr int kSubTiles = kTileK / 16;
+constexpr int kPairs = kSubTiles / 2;      // the value product takes 32 key positions per MFMA
+constexpr int kKLd = D + 8;                // padded key row in LDS (elements)
 constexpr int kVLd = kTileK + 8;
+constexpr int kKChunks = (kTileK * (D / 8) + 255) / 256;  // 16-byte pieces of a key tile per thread
+constexpr int kVChunks = (kTileK * D / 4 + 255) / 256;    // 8-byte pieces of a value tile per thread
+
+// One key/value tile on its way from the pages to LDS.
+struct TileInFlight {
+  bf16x8_t k[kKChunks];
+  s16x4_t v[kVChunks];
+};
 
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
-    bf16* __restrict__ out, int heads, int kv_heads, int block_size, int num_pages, float scale, int window) {
+    bf16* __restrict__ out, int heads, int kv_heads, int bs_shift, int num_pages, float scale, int window) {
   __shared__ __attribute__((aligned(16))) bf16 ks[kTileK * kKLd];
   __shared__ __attribute__((aligned(16))) bf16 vs[D * kVLd];
   __shared__ int sm_bad;
 
+  const int block_size = 1 << bs_shift;
   const int entry = tiles[2 * blockIdx.x];
   const int q0 = tiles[2 * blockIdx.x + 1];
   const int head = blockIdx.y;
@@ -379,7 +393,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int pos0 = ctx - q_len;  // position of the entry's first new token
   const int* table = block_table + static_cast<int64_t>(entry) * table_width;
   if (tid == 0) sm_bad = 0;
-  __syncthreads();
 
   // this lane's query (a column of S^T)
   const int qi = q0 + wave * 16 + col;
@@ -398,92 +411,180 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int w_last = pos0 + min(q0 + wave * 16 + 15, q_len - 1);
   const int w_first = window > 0 ? max(0, pos0 + q0 + wave * 16 - window + 1) : 0;
   const bool wave_has_queries = q0 + wave * 16 < q_len;
+  // a tile is fully visible to the wavefront when it ends at or before its first query's position
+  // and starts at or after its last query's window start (queries beyond q_len are never stored)
+  const int w_min_pos = pos0 + q0 + wave * 16;
+  const int w_max_first = window > 0 ? max(0, pos0 + q0 + wave * 16 + 15 - window + 1) : 0;
+  // softmax in base 2: exp(x) = exp2(x * log2(e))
+  const float scale2 = scale * 1.44269504088896340736f;
 
-  Softmax sm{-INFINITY, 0.f};
+  float m_run = -INFINITY;
+  float l_run = 0.f;  // this lane's share of the sum
   f32x4_t acc[kDimTiles];
 #pragma unroll
   for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   bool bad = false;
 
+  // Which piece of a tile each thread moves does not change from tile to tile: work it out
+  // once (block_size is a power of two here, so positions split into page and offset by shifts).
+  const int bs_mask = block_size - 1;
+  const int per_row_shift = bs_shift - 2;  // 8-byte pieces per dim row of a value page, as a shift
+  int k_row[kKChunks], k_lds[kKChunks];
+  int64_t k_off[kKChunks];
+#pragma unroll
+  for (int i = 0; i < kKChunks; ++i) {
+    const int c = tid + i * 256;
+    const int row = c / (D / 8);
+    const int ch = c - row * (D / 8);
+    k_row[i] = c < kTileK * (D / 8) ? row : -1;
+    k_lds[i] = row * kKLd + ch * 8;
+    k_off[i] = static_cast<int64_t>(kvh) * block_size * D + ch * 8;  // within a key page
+  }
+  int v_key[kVChunks], v_lds[kVChunks];
+  int64_t v_off[kVChunks];
+#pragma unroll
+  for (int i = 0; i < kVChunks; ++i) {
+    const int c = tid + i * 256;
+    const int piece = c >> per_row_shift;        // (page in tile) * D + dim
+    const int kg = c - (piece << per_row_shift);  // group of 4 positions inside the page
+    const int pg = piece / D;
+    const int d = piece - pg * D;
+    v_key[i] = c < kTileK * D / 4 ? pg * block_size + kg * 4 : -1;  // first position, relative to the tile
+    v_lds[i] = d * kVLd + pg * block_size + kg * 4;
+    v_off[i] = (static_cast<int64_t>(kvh) * D + d) * block_size + kg * 4;  // within a value page
+  }
+  const int64_t page_elems = static_cast<int64_t>(kv_heads) * block_size * D;
+
+  auto fetch = [&](int kt0, TileInFlight& t) {
+    const bool last = kt0 + kTileK > k_end;  // only the last tile has positions beyond k_end
+#pragma unroll
+    for (int i = 0; i < kKChunks; ++i) {
+      const int key = kt0 + k_row[i];
+      const bool want = k_row[i] >= 0 && key < k_end;
+      const int page = want ? table[key >> bs_shift] : 0;
+      const bool ok = want && page >= 0 && page < num_pages;
+      bad = bad || (want && !ok && key >= k_begin_raw);
+      const bf16* src = key_pages + (ok ? page * page_elems + static_cast<int64_t>(key & bs_mask) * D + k_off[i] : 0);
+      const bf16x8_t val = load_bf16x8(src);
+      t.k[i] = ok ? val : zero_bf16x8();
+    }
+    // values: per page a contiguous [D][block_size] block; pieces of 4 key positions
+#pragma unroll
+    for (int i = 0; i < kVChunks; ++i) {
+      const int key = kt0 + v_key[i];
+      const bool want = v_key[i] >= 0 && key < k_end;
+      const int page = want ? table[key >> bs_shift] : 0;
+      const bool ok = want && page >= 0 && page < num_pages;
+      const bf16* src = value_pages + (ok ? page * page_elems + v_off[i] : 0);
+      s16x4_t val = *reinterpret_cast<const s16x4_t*>(src);
+      if (!ok) val = s16x4_t{0, 0, 0, 0};
+      if (last) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (key + e >= k_end) val[e] = 0;  // beyond the last visible key: may be unwritten
+      }
+      t.v[i] = val;
+    }
+  };
+  auto stash = [&](const TileInFlight& t) {
+#pragma unroll
+    for (int i = 0; i < kKChunks; ++i)
+      if (k_row[i] >= 0) *reinterpret_cast<bf16x8_t*>(ks + k_lds[i]) = t.k[i];
+#pragma unroll
+    for (int i = 0; i < kVChunks; ++i)
+      if (v_key[i] >= 0) *reinterpret_cast<s16x4_t*>(vs + v_lds[i]) = t.v[i];
+  };
+
+  TileInFlight flight;
+  fetch(k_begin, flight);
+  stash(flight);
+  __syncthreads();
   for (int kt0 = k_begin; kt0 < k_end; kt0 += kTileK) {
-    __syncthreads();  // the previous tile has been consumed
-    // keys: kTileK rows of D dims, 16-byte chunks
-    for (int c = tid; c < kTileK * (D / 8); c += 256) {
-      const int row = c / (D / 8);
-      const int ch = c - row * (D / 8);
-      const int key = kt0 + row;
-      bf16x8_t val = zero_bf16x8();
-      if (key < k_end) {
-        const int logical = key / block_size;
-        const int page = table[logical];
-        if (page < 0 || page >= num_pages) {
-          bad = bad || key >= k_begin_raw;
-        } else {
-          val = load_bf16x8(key_pages +
-                            ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size +
-                             (key - logical * block_size)) * D + ch * 8);
-        }
-      }
-      *reinterpret_cast<bf16x8_t*>(ks + row * kKLd + ch * 8) = val;
-    }
-    // values: per page a contiguous [D][block_size] block; 8-byte chunks of 4 key positions
-    {
-      const int per_row = block_size / 4;      // chunks per dim row of a page
-      const int per_page = D * per_row;        // chunks per page
-      const int pages_in_tile = kTileK / block_size;
-      for (int c = tid; c < pages_in_tile * per_page; c += 256) {
-        const int pg = c / per_page;
-        const int rem = c - pg * per_page;
-        const int d = rem / per_row;
-        const int kg = rem - d * per_row;
-        const int key = kt0 + pg * block_size + kg * 4;
-        s16x4_t val = {0, 0, 0, 0};
-        if (key < k_end) {
-          const int page = table[key / block_size];
-          if (page >= 0 && page < num_pages) {
-            val = *reinterpret_cast<const s16x4_t*>(
-                value_pages + ((static_cast<int64_t>(page) * kv_heads + kvh) * D + d) * block_size + kg * 4);
+    const bool more = kt0 + kTileK < k_end;
+    if (more) fetch(kt0 + kTileK, flight);  // in flight while this tile is computed
+
+    if (wave_has_queries && kt0 <= w_last && kt0 + kTileK - 1 >= w_first) {
+      // Scores of the whole tile, then ONE softmax update for its kTileK positions.  The
+      // vector ALU, not the matrix core, bounds this loop (a wavefront instruction takes four
+      // cycles, an exponential sixteen), so every per-score operation counts: the scale is
+      // folded into the exponent's multiply-add, hidden scores are -inf and become 0 in the
+      // exponential by themselves, and only tiles that cross a query's limits build masks.
+      f32x4_t s[kSubTiles];
+      const bool full = kt0 + kTileK - 1 <= w_min_pos && kt0 >= w_max_first;  // uniform in the wavefront
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (key + i >= k_end) val[i] = 0;  // beyond the last visible key: may be unwritten
+      for (int sub = 0; sub < kSubTiles; ++sub)
+        s[sub] = score_tile(load_row(ks + (sub * 16 + col) * kKLd, true, quarter), qo);
+      if (!full) {
+#pragma unroll
+        for (int sub = 0; sub < kSubTiles; ++sub)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kt0 + sub * 16 + quarter * 4 + i;
+            if (!(q_ok && key <= pq && key >= pq_first)) s[sub][i] = -INFINITY;
           }
+      }
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int sub = 0; sub < kSubTiles; ++sub)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[sub][i]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(m_run, tmax * scale2);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
+      const float alpha = fast_exp2(m_run - m_use);            // 2^-inf = 0 for the first tile
+      float sum = 0.f;
+      uint32_t pw[kSubTiles][2];
+#pragma unroll
+      for (int sub = 0; sub < kSubTiles; ++sub) {
+        float p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          p[i] = fast_exp2(fmaf(s[sub][i], scale2, -m_use));
+          sum += p[i];
         }
-        *reinterpret_cast<s16x4_t*>(vs + d * kVLd + pg * block_size + kg * 4) = val;
+        pw[sub][0] = pack_bf16x2(p[0], p[1]);
+        pw[sub][1] = pack_bf16x2(p[2], p[3]);
+      }
+      l_run = l_run * alpha + sum;
+      m_run = m_new;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+      }
+      // O^T += V^T P^T, 32 key positions per MFMA: k-slots 0..3 of a lane are its 4 keys of the
+      // pair's first sub-tile, slots 4..7 those of the second; the value operand follows the same map
+      typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int pr = 0; pr < kPairs; ++pr) {
+        const u32x4_t pb = {pw[2 * pr][0], pw[2 * pr][1], pw[2 * pr + 1][0], pw[2 * pr + 1][1]};
+        const bf16x8_t pop = __builtin_bit_cast(bf16x8_t, pb);
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt) {
+          const bf16* vrow = vs + (dt * 16 + col) * kVLd + pr * 32 + quarter * 4;
+          const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vrow);
+          const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vrow + 16);
+          const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
+          acc[dt] = mfma_16x16x32(__builtin_bit_cast(bf16x8_t, va), pop, acc[dt]);
+        }
       }
     }
+
+    __syncthreads();  // every wavefront has consumed the tile
+    if (more) stash(flight);
     __syncthreads();
-    if (!wave_has_queries) continue;
-#pragma unroll
-    for (int sub = 0; sub < kTileK / 16; ++sub) {
-      const int ts = kt0 + sub * 16;
-      if (ts > w_last || ts + 15 < w_first) continue;  // nothing visible to this wavefront
-      const f32x4_t s = score_tile(load_row(ks + (sub * 16 + col) * kKLd, true, quarter), qo);
-      bool ok[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = ts + quarter * 4 + i;
-        ok[i] = q_ok && key <= pq && key >= pq_first;
-      }
-      float alpha;
-      const s16x4_t pb = softmax_tile(sm, s, ok, scale, alpha);
-#pragma unroll
-      for (int dt = 0; dt < kDimTiles; ++dt) {
-        const s16x4_t va =
-            *reinterpret_cast<const s16x4_t*>(vs + (dt * 16 + col) * kVLd + sub * 16 + quarter * 4);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
-        acc[dt] = mfma_16x16x16(va, pb, acc[dt]);
-      }
-    }
   }
 
   if (bad) atomicOr(&sm_bad, 1);
   __syncthreads();
   const bool poisoned = sm_bad != 0;
-  sm.l += __shfl_xor(sm.l, 16, kWave);
-  sm.l += __shfl_xor(sm.l, 32, kWave);
+  l_run += __shfl_xor(l_run, 16, kWave);
+  l_run += __shfl_xor(l_run, 32, kWave);
   if (q_ok) {
-    const float inv = 1.0f / sm.l;
+    const float inv = 1.0f / l_run;
     bf16* orow = out + (static_cast<int64_t>(t_first + qi) * heads + head) * D;
 #pragma unroll
     for (int dt = 0; dt < kDimTiles; ++dt) {
@@ -558,8 +659,10 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
                           int block_size, int num_pages, float scale, int window, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(num_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad sizes");
-  MLR_REQUIRE(block_size >= 4 && block_size % 4 == 0 && kTileK % block_size == 0,
-              "block_size must be a multiple of 4 that divides the key tile");
+  MLR_REQUIRE(block_size >= 4 && (block_size & (block_size - 1)) == 0 && block_size <= kTileK,
+              "block_size must be a power of two within 4 and the key tile");
+  int bs_shift = 0;
+  while ((1 << bs_shift) < block_size) ++bs_shift;
   MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
   MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * D && q_stride % 8 == 0, "q_stride must cover a row and keep 16-byte alignment");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
@@ -570,7 +673,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   attn_prefill_kernel<<<dim3(num_tiles, heads), 256, 0, stream>>>(
       static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
       static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,
-      static_cast<bf16*>(out), heads, kv_heads, block_size, num_pages, scale, window);
+      static_cast<bf16*>(out), heads, kv_heads, bs_shift, num_pages, scale, window);
   MLR_LAUNCH_CHECK();
   return 0;
 }

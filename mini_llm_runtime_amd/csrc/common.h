@@ -30,8 +30,13 @@ __host__ __device__ inline float to_f32(bf16 v) {
   return c.f;
 }
 
-// Round to nearest even; NaN stays NaN.
+// Round to nearest even; NaN stays NaN.  On the device this is the hardware conversion.
 __host__ __device__ inline bf16 f32_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  bf16 hw;
+  hw.bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+  return hw;
+#endif
   union {
     uint32_t u;
     float f;

@@ -30,6 +30,19 @@ __device__ __forceinline__ bf16x8_t zero_bf16x8() {
   return __builtin_bit_cast(bf16x8_t, z);
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// Two floats to two bfloat16 in one 32-bit word (v_cvt_pk_bf16_f32, round to nearest even).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// 2^x by the hardware instruction (no denormal fix-up: results below 2^-126 become 0,
+// 2^-inf is 0), for softmax weights.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ f32x4_t mfma_16x16x32(bf16x8_t a, bf16x8_t b, f32x4_t c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }

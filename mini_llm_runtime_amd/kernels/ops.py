@@ -403,8 +403,8 @@ class HipOps:
         lib = None
         if use_mfma:
             lib = self.attention_library(head_dim)
-            if num_tiles and lib.mlr_attention_key_tile() % block_size:
-                use_mfma = False
+            if num_tiles and (block_size & (block_size - 1) or block_size > lib.mlr_attention_key_tile()):
+                use_mfma = False  # the tiled prefill kernel takes power-of-two pages up to its key tile
         if not use_mfma:
             self._call(
                 "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
