@@ -14,15 +14,16 @@
 //    slice between them (interleaved, so the workgroup reads contiguous spans of
 //    every weight row), keep eight 16-byte loads in flight per lane, and add their
 //    partial sums through LDS.  Activations come straight from L2.
-//  * gemm_skinny_rows: 17..64 tokens.  A workgroup owns 64 output features, one
-//    16-row slab per wavefront, and one slice of K; the wavefronts read the same
-//    activation chunks at the same time, so those come from the L1 cache.
+//  * gemm_tiled: everything else.  An output tile per workgroup (64 x 64 up to 64
+//    tokens, else 128 tokens x 64 or 128 features, whichever fills the compute
+//    units), K in slices of 64 staged through double-buffered LDS by range-checked
+//    buffer loads (edge tiles and the tail of K read zeros, no branches), four
+//    wavefronts, 32x32x16 MFMA.  Workgroups are placed so that those resident on
+//    one XCD share operands in its L2.  Up to 16 tokens take this kernel too once
+//    its tiles fill the compute units (it streams a wide weight fastest).
 //    With more than one K slice both kernels write float32 partial sums
 //    [slice, M, N]; the consumer (the residual-adding norm kernel) sums them in a
 //    fixed order, so results do not depend on which slice finishes first.
-//  * gemm_tiled: many tokens (prompts).  128 x 128 output tile per workgroup,
-//    K in slices of 64 staged through double-buffered LDS, four wavefronts of
-//    64 x 64 each, 32x32x16 MFMA.
 // K must be a multiple of 8 (16-byte rows); other shapes take the FMA kernel.
 //
 // SwiGLU epilogue: with gate and up rows interleaved in pairs
@@ -166,78 +167,58 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   }
 }
 
-// ---- skinny, 17..64 tokens: one 16-row slab per wavefront ----------------------------------
-template <int MT>
-__global__ __launch_bounds__(256) void gemm_skinny_rows_kernel(const bf16* __restrict__ x,
-                                                               const bf16* __restrict__ w, GemmEpilogue ep,
-                                                               int M, int N, int K) {
-  constexpr int U = 4;
-  const int lane = threadIdx.x % kWave;
-  const int wave = threadIdx.x / kWave;
-  const int r = lane % 16;
-  const int q = lane / 16;
-  const int n0 = (blockIdx.x * 4 + wave) * 16;
-  if (n0 >= N) return;
-  const int slices = gridDim.y;
-  const int chunks = K / 8;
-  const int ksteps = (chunks + 3) / 4;
-  const int per = (ksteps + slices - 1) / slices;
-  const int sb = blockIdx.y * per;
-  const int se = min(ksteps, sb + per);
-  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(n0 + r, N - 1)) * K);
-  const bf16x8_t* xp[MT];
-  bool xok[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r;
-    xok[mt] = m < M;
-    xp[mt] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(m, M - 1)) * K);
-  }
-  f32x4_t acc[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+// ---- tiled: more than 16 tokens, and wide products of fewer ---------------------------------
+// Four wavefronts in a 2 x 2 arrangement; each owns WM x WN blocks of 32 x 32 (tokens x
+// features), so the workgroup tile is (64 WM) tokens x (64 WN) features.  K in slices of 64
+// through double-buffered LDS (one barrier per slice).  grid.z cuts K into slices whose
+// float32 partial sums go to [slice, M, N].
+constexpr int kBK = 64;       // k per LDS slice
+constexpr int kLd = kBK + 8;  // padded LDS row, in elements (144 bytes)
 
-  for (int s0 = sb; s0 < se; s0 += U) {
-    bf16x8_t a[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int c = (s0 + u) * 4 + q;
-      a[u] = (s0 + u < se && c < chunks) ? __builtin_nontemporal_load(wp + c) : zero_bf16x8();
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int c = (s0 + u) * 4 + q;
-      const bool in = s0 + u < se && c < chunks;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8_t b = (in && xok[mt]) ? xp[mt][c] : zero_bf16x8();
-        acc[mt] = mfma_16x16x32(a[u], b, acc[mt]);
-      }
-    }
-  }
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const float v[4] = {acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]};
-    finish4(ep, blockIdx.y, slices, mt * 16 + r, n0 + q * 4, M, N, v);
-  }
+template <int WM, int WN>
+struct TiledShape {
+  static constexpr int BM = 64 * WM;
+  static constexpr int BN = 64 * WN;
+  static constexpr int kPieces = (BM + BN) * (kBK / 8) / 256;  // 16-byte pieces per thread and slice
+  static constexpr int kLds = 2 * (BM + BN) * kLd * 2;         // bytes, two buffers
+};
+
+// Workgroup -> (slice, token tile, feature tile).  Consecutive workgroups go to the eight
+// XCDs in turn, each with an L2 of its own: the ones that land on one XCD take a contiguous
+// run of the tile order, and that order walks groups of eight token tiles feature tile by
+// feature tile, so that the workgroups resident on an XCD at one time form a compact block
+// of the output and share their operands in its L2.
+struct TileOrder {
+  int m_tiles, n_tiles, slices;
+};
+__device__ __forceinline__ void place_workgroup(const TileOrder& order, int id, int& slice, int& mt, int& nt) {
+  constexpr int kXcds = 8, kGroup = 8;
+  const int tiles = order.m_tiles * order.n_tiles;
+  const int total = tiles * order.slices;
+  const int q = total / kXcds, r = total % kXcds;
+  const int xcd = id % kXcds, local = id / kXcds;
+  int pos = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
+  slice = pos / tiles;
+  pos -= slice * tiles;
+  const int per_group = kGroup * order.n_tiles;
+  const int group = pos / per_group;
+  const int first = group * kGroup;
+  const int size = min(order.m_tiles - first, kGroup);
+  const int in_group = pos - group * per_group;
+  mt = first + in_group % size;
+  nt = in_group / size;
 }
 
-// ---- tiled: many tokens -----------------------------------------------------------------
-constexpr int kBM = 128;  // tokens per workgroup tile
-constexpr int kBN = 128;  // output features per workgroup tile
-constexpr int kBK = 64;   // k per LDS slice
-constexpr int kLd = kBK + 8;  // padded LDS row, in elements (144 bytes)
-constexpr int kTiledLds = 2 * (kBM + kBN) * kLd * 2;  // bytes, two buffers
-
+template <int WM, int WN>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
-                                                         GemmEpilogue ep, int M, int N, int K) {
+                                                         GemmEpilogue ep, TileOrder order, int M, int N, int K) {
+  using Shape = TiledShape<WM, WN>;
+  constexpr int BM = Shape::BM, BN = Shape::BN, PIECES = Shape::kPieces;
+  // Two LDS buffers, each BN rows of w and then BM rows of x.  Addressed as offsets from
+  // the one shared array so that every access stays an LDS instruction.
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bf16* ws[2];
-  bf16* xs[2];
-  ws[0] = reinterpret_cast<bf16*>(smem);
-  xs[0] = ws[0] + kBN * kLd;
-  ws[1] = xs[0] + kBM * kLd;
-  xs[1] = ws[1] + kBN * kLd;
+  bf16* const lds = reinterpret_cast<bf16*>(smem);
+  constexpr int kBuffer = (BM + BN) * kLd;
 
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
@@ -246,90 +227,119 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
   const int wm = wave / 2;
   const int r32 = lane % 32;
   const int h = lane / 32;
-  const int n0 = blockIdx.x * kBN;
-  const int m0 = blockIdx.y * kBM;
+  int slice, mt, nt;
+  place_workgroup(order, blockIdx.x, slice, mt, nt);
+  const int n0 = nt * BN;
+  const int m0 = mt * BM;
   const int chunks = K / 8;
+  const int slices = order.slices;
+  const int k_slices = (K + kBK - 1) / kBK;
+  const int per = (k_slices + slices - 1) / slices;
+  const int s_begin = slice * per;
+  const int s_end = min(k_slices, s_begin + per);
 
-  // global -> register staging: 4 chunks of w and 4 of x per thread and slice
-  const bf16x8_t* wsrc[4];
-  const bf16x8_t* xsrc[4];
-  int lds_off[4];
-  int chunk_in_slice[4];
+  // global -> register staging through two buffer resources that cover exactly this tile's
+  // rows: rows past the end of the matrix, and the tail of K, read as zeros.
+  const int w_rows = min(BN, N - n0), x_rows = min(BM, M - m0);
+  const __amdgpu_buffer_rsrc_t w_buf = make_buffer(w + static_cast<int64_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2u);
+  const __amdgpu_buffer_rsrc_t x_buf = make_buffer(x + static_cast<int64_t>(m0) * K, static_cast<unsigned>(x_rows) * K * 2u);
+  unsigned piece_off[PIECES];  // byte offset of the piece in slice 0
+  int lds_off[PIECES];
+  int piece_chunk[PIECES];
 #pragma unroll
-  for (int it = 0; it < 4; ++it) {
+  for (int it = 0; it < PIECES; ++it) {
     const int idx = tid + it * 256;
     const int row = idx / 8;
     const int ch = idx % 8;
-    wsrc[it] = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(n0 + row, N - 1)) * K);
-    xsrc[it] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(m0 + row, M - 1)) * K);
+    piece_off[it] = static_cast<unsigned>(row < BN ? row : row - BN) * K * 2u + ch * 16u;
     lds_off[it] = row * kLd + ch * 8;
-    chunk_in_slice[it] = ch;
+    piece_chunk[it] = ch;
   }
 
-  f32x16_t acc[2][2];
+  f32x16_t acc[WN][WM];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WN; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WM; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int slices = (K + kBK - 1) / kBK;
-  bf16x8_t wreg[4], xreg[4];
+  bf16x8_t reg[PIECES];
   auto fetch = [&](int slice) {
+    const int left = chunks - slice * (kBK / 8);  // chunks of K from this slice on
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int c = slice * (kBK / 8) + chunk_in_slice[it];
-      wreg[it] = c < chunks ? wsrc[it][c] : zero_bf16x8();
-      xreg[it] = c < chunks ? xsrc[it][c] : zero_bf16x8();
+    for (int it = 0; it < PIECES; ++it) {
+      const unsigned off = piece_chunk[it] < left ? piece_off[it] + slice * (kBK * 2u) : kOutOfBuffer;
+      reg[it] = buffer_load_bf16x8(it * 256 / 8 < BN ? w_buf : x_buf, off);
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      *reinterpret_cast<bf16x8_t*>(ws[buf] + lds_off[it]) = wreg[it];
-      *reinterpret_cast<bf16x8_t*>(xs[buf] + lds_off[it]) = xreg[it];
-    }
+    for (int it = 0; it < PIECES; ++it) *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + lds_off[it]) = reg[it];
   };
 
-  fetch(0);
-  stash(0);
+  if (s_begin < s_end) {
+    fetch(s_begin);
+    stash(0);
+  }
   __syncthreads();
-  for (int s = 0; s < slices; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < slices) fetch(s + 1);
-    const bf16* wt = ws[buf] + (wn * 64 + r32) * kLd + h * 8;
-    const bf16* xt = xs[buf] + (wm * 64 + r32) * kLd + h * 8;
+  for (int s = s_begin; s < s_end; ++s) {
+    const int buf = (s - s_begin) & 1;
+    if (s + 1 < s_end) fetch(s + 1);
+    const bf16* wt = lds + buf * kBuffer + (wn * 32 * WN + r32) * kLd + h * 8;
+    const bf16* xt = lds + buf * kBuffer + (BN + wm * 32 * WM + r32) * kLd + h * 8;
 #pragma unroll
     for (int kk = 0; kk < kBK / 16; ++kk) {
-      bf16x8_t a[2], b[2];
+      bf16x8_t a[WN], b[WM];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = load_bf16x8(wt + i * 32 * kLd + kk * 16);
+      for (int i = 0; i < WN; ++i) a[i] = load_bf16x8(wt + i * 32 * kLd + kk * 16);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = load_bf16x8(xt + j * 32 * kLd + kk * 16);
+      for (int j = 0; j < WM; ++j) b[j] = load_bf16x8(xt + j * 32 * kLd + kk * 16);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WN; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < WM; ++j) acc[i][j] = mfma_32x32x16(a[i], b[j], acc[i][j]);
     }
-    if (s + 1 < slices) stash(buf ^ 1);
+    if (s + 1 < s_end) stash(buf ^ 1);
     __syncthreads();
   }
 
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WN; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int64_t m = m0 + wm * 64 + j * 32 + r32;
-      if (m >= M) continue;
+    for (int j = 0; j < WM; ++j) {
+      const int m = m0 + (wm * WM + j) * 32 + r32;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * 64 + i * 32 + g * 8 + h * 4;
-        if (n < N)
-          store4(ep, m, n, N, acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
-                 acc[i][j][g * 4 + 3]);
+        const int n = n0 + (wn * WN + i) * 32 + g * 8 + h * 4;
+        const float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+        finish4(ep, slice, slices, m, n, M, N, v);
       }
     }
+}
+
+template <int WM, int WN>
+static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
+                        hipStream_t stream) {
+  using Shape = TiledShape<WM, WN>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLds);
+    if (e != hipSuccess) {
+      set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
+      return -1;
+    }
+    configured = true;
+  }
+  TileOrder order{(m + Shape::BM - 1) / Shape::BM, (n + Shape::BN - 1) / Shape::BN, slices};
+  const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles * slices;
+  if (groups >= (1ll << 31)) {
+    set_error("mlr_gemm_bf16: too many tiles for one launch");
+    return -1;
+  }
+  gemm_tiled_kernel<WM, WN><<<dim3(static_cast<unsigned>(groups)), 256, Shape::kLds, stream>>>(xb, wb, ep, order, m, n, k);
+  return 0;
 }
 
 // K slices for a skinny product: enough workgroups to keep every compute unit
@@ -341,36 +351,24 @@ static int choose_slices(int groups, int ksteps, int allowed) {
   return slices;
 }
 
+// Workgroups of the 128 x 128 tiling for this shape.
+static int tiled_groups(int m, int n, int bn) { return ((n + bn - 1) / bn) * ((m + 127) / 128); }
+
+// Up to 16 tokens: the LDS-tiled kernel once its 64-feature tiles (times slices) fill the
+// compute units, the 16-feature streaming kernel below that.
+static bool few_tokens_tiled(int n, int slices) { return ((n + 63) / 64) * slices >= 256; }
+
 static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
                      hipStream_t stream) {
-  if (m <= 16) {
+  if (m <= 16 && !few_tokens_tiled(n, slices)) {
     dim3 grid((n + 15) / 16, slices);
     gemm_skinny_split_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
-  } else if (m <= 64) {
-    dim3 grid((n + 63) / 64, slices);
-    if (m <= 32)
-      gemm_skinny_rows_kernel<2><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
-    else
-      gemm_skinny_rows_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
-  } else {
-    static bool configured = false;
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, kTiledLds);
-      if (e != hipSuccess) {
-        set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
-        return -1;
-      }
-      configured = true;
-    }
-    dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
-    if (grid.y >= 65536u) {
-      set_error("mlr_gemm_bf16: too many rows for one launch");
-      return -1;
-    }
-    gemm_tiled_kernel<<<grid, 256, kTiledLds, stream>>>(xb, wb, ep, m, n, k);
+    return 0;
   }
-  return 0;
+  if (m <= 64) return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
+  // too few 128 x 128 tiles to fill the compute units: halve the tile along the features
+  if (tiled_groups(m, n, 128) * slices < 256) return launch_tiled<2, 1>(xb, wb, ep, m, n, k, slices, stream);
+  return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
 }
 
 }  // namespace mlr
@@ -382,7 +380,14 @@ extern "C" {
 // How many K slices mlr_gemm_bf16 would use for this shape when the caller can take
 // partial sums (at most `max_slices`); 1 means it writes the finished product.
 int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
-  if (m > 64 || k % 8 != 0) return 1;
+  if (k % 8 != 0) return 1;
+  if (m > 64) {
+    // tiled kernel: cut K while the grid is small and a slice keeps at least 8 LDS slices of 64
+    int slices = 1;
+    while (slices < max_slices && slices < 4 && tiled_groups(m, n, 128) * slices < 256 && k / (slices * 2) >= 8 * kBK)
+      slices *= 2;
+    return slices;
+  }
   const int groups = m <= 16 ? (n + 15) / 16 : (n + 63) / 64;
   return choose_slices(groups, (k / 8 + 3) / 4, max_slices);
 }
@@ -398,10 +403,10 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
+  MLR_REQUIRE(k <= (1 << 20), "k must not exceed 2^20 (32-bit byte offsets inside a tile)");
   MLR_REQUIRE(!swiglu || (n % 4 == 0 && bias == nullptr), "swiglu needs n % 4 == 0 and no bias");
   MLR_REQUIRE(slices >= 1 && slices <= 64, "slices must be within 1..64");
-  MLR_REQUIRE(slices == 1 || (m <= 64 && !swiglu && out_is_f32),
-              "partial sums are float32, for up to 64 tokens, without SwiGLU");
+  MLR_REQUIRE(slices == 1 || (!swiglu && out_is_f32), "partial sums are float32, without SwiGLU");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
               "x and w must be 16-byte aligned");
   GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};

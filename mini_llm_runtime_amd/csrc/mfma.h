@@ -30,6 +30,17 @@ __device__ __forceinline__ bf16x8_t zero_bf16x8() {
   return __builtin_bit_cast(bf16x8_t, z);
 }
 
+// Buffer resource over `bytes` bytes at p: loads through it return zero beyond the end, so
+// tiles at the edge of a matrix need no branches.  Offsets are unsigned 32-bit byte counts.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+constexpr unsigned kOutOfBuffer = 0x80000000u;  // larger than any resource made here
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
+}
+__device__ __forceinline__ bf16x8_t buffer_load_bf16x8(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_offset) {
+  return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0));
+}
+
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 

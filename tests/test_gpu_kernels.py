@@ -172,7 +172,11 @@ def test_linear_swiglu_epilogue(ops_for, dtype, m, inter, k):
         torch.testing.assert_close(got.double(), ref, **tol)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 896, 4864), (8, 896, 896), (16, 130, 2056), (33, 517, 2056), (64, 896, 4864), (8, 151936, 96)])
+@pytest.mark.parametrize(
+    "m,n,k",
+    [(1, 896, 4864), (8, 896, 896), (16, 130, 2056), (33, 517, 2056), (64, 896, 4864), (8, 151936, 96),
+     (300, 517, 4104), (2048, 896, 4864), (130, 130, 1032)],
+)
 def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     """A narrow product of a few tokens may come back as float32 partial sums over slices of k;
     the norm kernel adds them, in order, to the residual stream."""
