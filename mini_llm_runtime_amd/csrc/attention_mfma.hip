@@ -358,13 +358,14 @@ constexpr int kSubTiles = kTileK / 16;
 constexpr int kPairs = kSubTiles / 2;      // the value product takes 32 key positions per MFMA
 constexpr int kKLd = D + 8;                // padded key row in LDS (elements)
 constexpr int kVLd = kTileK + 8;
-constexpr int kKChunks = (kTileK * (D / 8) + 255) / 256;  // 16-byte pieces of a key tile per thread
-constexpr int kVChunks = (kTileK * D / 4 + 255) / 256;    // 8-byte pieces of a value tile per thread
+constexpr int kPieces = (kTileK * (D / 8) + 255) / 256;  // 16-byte pieces per thread, of the key and of the value tile
+constexpr int kNoPiece = 0x3fffffff;                      // position of a piece that a thread does not have
+constexpr int kPrefillLds = 2 * (kTileK * kKLd + D * kVLd) * 2 + 16;  // bytes: two buffers and a flag
 
 // One key/value tile on its way from the pages to LDS.
 struct TileInFlight {
-  bf16x8_t k[kKChunks];
-  s16x4_t v[kVChunks];
+  bf16x8_t k[kPieces];
+  bf16x8_t v[kPieces];
 };
 
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
@@ -372,9 +373,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int heads, int kv_heads, int bs_shift, int num_pages, float scale, int window) {
-  __shared__ __attribute__((aligned(16))) bf16 ks[kTileK * kKLd];
-  __shared__ __attribute__((aligned(16))) bf16 vs[D * kVLd];
-  __shared__ int sm_bad;
+  // two buffers of (key tile, value tile), then a flag; offsets from one array keep LDS addressing
+  extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
+  bf16* const lds = reinterpret_cast<bf16*>(prefill_lds);
+  constexpr int kBuffer = kTileK * kKLd + D * kVLd;  // elements
+  int& sm_bad = *reinterpret_cast<int*>(prefill_lds + 2 * kBuffer * 2);
 
   const int block_size = 1 << bs_shift;
   const int entry = tiles[2 * blockIdx.x];
@@ -425,83 +428,87 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   bool bad = false;
 
-  // Which piece of a tile each thread moves does not change from tile to tile: work it out
-  // once (block_size is a power of two here, so positions split into page and offset by shifts).
+  // Which pieces of a tile each thread moves does not change from tile to tile: work out once
+  // the page of the tile a piece lies in, its place inside that page and its place in LDS.
+  // A tile is kTileK / block_size pages; a key page holds [offset][dim], a value page [dim][offset].
   const int bs_mask = block_size - 1;
-  const int per_row_shift = bs_shift - 2;  // 8-byte pieces per dim row of a value page, as a shift
-  int k_row[kKChunks], k_lds[kKChunks];
-  int64_t k_off[kKChunks];
+  int k_row[kPieces], k_page[kPieces], k_in_page[kPieces], k_lds[kPieces];
 #pragma unroll
-  for (int i = 0; i < kKChunks; ++i) {
+  for (int i = 0; i < kPieces; ++i) {
     const int c = tid + i * 256;
     const int row = c / (D / 8);
     const int ch = c - row * (D / 8);
-    k_row[i] = c < kTileK * (D / 8) ? row : -1;
+    k_row[i] = c < kTileK * (D / 8) ? row : kNoPiece;
+    k_page[i] = row >> bs_shift;
+    k_in_page[i] = (kvh * block_size + (row & bs_mask)) * D + ch * 8;
     k_lds[i] = row * kKLd + ch * 8;
-    k_off[i] = static_cast<int64_t>(kvh) * block_size * D + ch * 8;  // within a key page
   }
-  int v_key[kVChunks], v_lds[kVChunks];
-  int64_t v_off[kVChunks];
+  int v_pos[kPieces], v_page[kPieces], v_in_page[kPieces], v_lds[kPieces];
+  const int per_page = D * (block_size / 8);  // 16-byte pieces of a value page (one kv head)
 #pragma unroll
-  for (int i = 0; i < kVChunks; ++i) {
+  for (int i = 0; i < kPieces; ++i) {
     const int c = tid + i * 256;
-    const int piece = c >> per_row_shift;        // (page in tile) * D + dim
-    const int kg = c - (piece << per_row_shift);  // group of 4 positions inside the page
-    const int pg = piece / D;
-    const int d = piece - pg * D;
-    v_key[i] = c < kTileK * D / 4 ? pg * block_size + kg * 4 : -1;  // first position, relative to the tile
-    v_lds[i] = d * kVLd + pg * block_size + kg * 4;
-    v_off[i] = (static_cast<int64_t>(kvh) * D + d) * block_size + kg * 4;  // within a value page
+    const int pg = c / per_page;
+    const int within = c - pg * per_page;
+    const int d = within >> (bs_shift - 3);
+    const int part = within & ((block_size >> 3) - 1);
+    v_pos[i] = c < kTileK * (D / 8) ? pg * block_size + part * 8 : kNoPiece;  // first position, relative to the tile
+    v_page[i] = pg;
+    v_in_page[i] = (kvh * D + d) * block_size + part * 8;
+    v_lds[i] = kTileK * kKLd + d * kVLd + pg * block_size + part * 8;
   }
   const int64_t page_elems = static_cast<int64_t>(kv_heads) * block_size * D;
+  const int last_page = (k_end - 1) >> bs_shift;  // the last table entry that any query here may use
 
+  // Loads are unconditional (a page that is absent or past the end reads page 0 instead) so
+  // that the tile loop stays free of branches.  Keys read that way need no clearing: their
+  // scores are masked by position.  Values are cleared, since 0 * NaN would reach the output;
+  // that can only happen in the last tile and under a window, whose early pages may be gone.
   auto fetch = [&](int kt0, TileInFlight& t) {
-    const bool last = kt0 + kTileK > k_end;  // only the last tile has positions beyond k_end
+    const int lim = k_end - kt0;  // positions of this tile that exist
+    const int page0 = kt0 >> bs_shift;
 #pragma unroll
-    for (int i = 0; i < kKChunks; ++i) {
-      const int key = kt0 + k_row[i];
-      const bool want = k_row[i] >= 0 && key < k_end;
-      const int page = want ? table[key >> bs_shift] : 0;
-      const bool ok = want && page >= 0 && page < num_pages;
-      bad = bad || (want && !ok && key >= k_begin_raw);
-      const bf16* src = key_pages + (ok ? page * page_elems + static_cast<int64_t>(key & bs_mask) * D + k_off[i] : 0);
-      const bf16x8_t val = load_bf16x8(src);
-      t.k[i] = ok ? val : zero_bf16x8();
+    for (int i = 0; i < kPieces; ++i) {
+      const int page = table[min(page0 + k_page[i], last_page)];
+      const bool in = static_cast<unsigned>(page) < static_cast<unsigned>(num_pages);
+      bad = bad || (!in && k_row[i] < lim && kt0 + k_row[i] >= k_begin_raw);
+      t.k[i] = load_bf16x8(key_pages + ((in ? page : 0) * page_elems + k_in_page[i]));
     }
-    // values: per page a contiguous [D][block_size] block; pieces of 4 key positions
+    const bool guard = lim < kTileK || window > 0;  // uniform
 #pragma unroll
-    for (int i = 0; i < kVChunks; ++i) {
-      const int key = kt0 + v_key[i];
-      const bool want = v_key[i] >= 0 && key < k_end;
-      const int page = want ? table[key >> bs_shift] : 0;
-      const bool ok = want && page >= 0 && page < num_pages;
-      const bf16* src = value_pages + (ok ? page * page_elems + v_off[i] : 0);
-      s16x4_t val = *reinterpret_cast<const s16x4_t*>(src);
-      if (!ok) val = s16x4_t{0, 0, 0, 0};
-      if (last) {
+    for (int i = 0; i < kPieces; ++i) {
+      const int page = table[min(page0 + v_page[i], last_page)];
+      const bool in = static_cast<unsigned>(page) < static_cast<unsigned>(num_pages);
+      bf16x8_t val = load_bf16x8(value_pages + ((in ? page : 0) * page_elems + v_in_page[i]));
+      if (guard) {
+        u16x8_t bits = __builtin_bit_cast(u16x8_t, val);
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (key + e >= k_end) val[e] = 0;  // beyond the last visible key: may be unwritten
+        for (int e = 0; e < 8; ++e)
+          if (!in || v_pos[i] + e >= lim) bits[e] = 0;
+        val = __builtin_bit_cast(bf16x8_t, bits);
       }
       t.v[i] = val;
     }
   };
-  auto stash = [&](const TileInFlight& t) {
+  auto stash = [&](const TileInFlight& t, int buf) {
 #pragma unroll
-    for (int i = 0; i < kKChunks; ++i)
-      if (k_row[i] >= 0) *reinterpret_cast<bf16x8_t*>(ks + k_lds[i]) = t.k[i];
-#pragma unroll
-    for (int i = 0; i < kVChunks; ++i)
-      if (v_key[i] >= 0) *reinterpret_cast<s16x4_t*>(vs + v_lds[i]) = t.v[i];
+    for (int i = 0; i < kPieces; ++i)
+      if (k_row[i] != kNoPiece) {
+        *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + k_lds[i]) = t.k[i];
+        *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + v_lds[i]) = t.v[i];
+      }
   };
 
   TileInFlight flight;
   fetch(k_begin, flight);
-  stash(flight);
+  stash(flight, 0);
   __syncthreads();
-  for (int kt0 = k_begin; kt0 < k_end; kt0 += kTileK) {
+  int buf = 0;
+  for (int kt0 = k_begin; kt0 < k_end; kt0 += kTileK, buf ^= 1) {
     const bool more = kt0 + kTileK < k_end;
     if (more) fetch(kt0 + kTileK, flight);  // in flight while this tile is computed
+    const bf16* ks = lds + buf * kBuffer;
+    const bf16* vs = ks + kTileK * kKLd;
 
     if (wave_has_queries && kt0 <= w_last && kt0 + kTileK - 1 >= w_first) {
       // Scores of the whole tile, then ONE softmax update for its kTileK positions.  The
@@ -573,8 +580,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       }
     }
 
-    __syncthreads();  // every wavefront has consumed the tile
-    if (more) stash(flight);
+    // the other buffer was last read one iteration ago, before that iteration's barrier
+    if (more) stash(flight, buf ^ 1);
     __syncthreads();
   }
 
@@ -630,7 +637,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   MLR_REQUIRE(splits == 1 || partial != nullptr, "several partitions need scratch memory");
   MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * D && q_stride % 8 == 0, "q_stride must cover a row and keep 16-byte alignment");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
-                  reinterpret_cast<uintptr_t>(value_pages) % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
+                  reinterpret_cast<uintptr_t>(value_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
               "operands must be 16-byte aligned");
   MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
   const int group = heads / kv_heads;
@@ -659,18 +666,28 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
                           int block_size, int num_pages, float scale, int window, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(num_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad sizes");
-  MLR_REQUIRE(block_size >= 4 && (block_size & (block_size - 1)) == 0 && block_size <= kTileK,
-              "block_size must be a power of two within 4 and the key tile");
+  MLR_REQUIRE(block_size >= 8 && (block_size & (block_size - 1)) == 0 && block_size <= kTileK,
+              "block_size must be a power of two within 8 and the key tile");
   int bs_shift = 0;
   while ((1 << bs_shift) < block_size) ++bs_shift;
   MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
   MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * D && q_stride % 8 == 0, "q_stride must cover a row and keep 16-byte alignment");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
-                  reinterpret_cast<uintptr_t>(value_pages) % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
+                  reinterpret_cast<uintptr_t>(value_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
               "operands must be 16-byte aligned");
   MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
   MLR_REQUIRE(heads <= 65535, "too many heads for one launch");
-  attn_prefill_kernel<<<dim3(num_tiles, heads), 256, 0, stream>>>(
+  static bool configured = false;
+  if (!configured) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
+    if (e != hipSuccess) {
+      set_error(std::string("mlr_attention_prefill: cannot raise the LDS limit: ") + hipGetErrorString(e));
+      return -1;
+    }
+    configured = true;
+  }
+  attn_prefill_kernel<<<dim3(num_tiles, heads), 256, kPrefillLds, stream>>>(
       static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
       static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,
       static_cast<bf16*>(out), heads, kv_heads, bs_shift, num_pages, scale, window);

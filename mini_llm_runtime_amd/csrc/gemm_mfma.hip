@@ -14,9 +14,9 @@
 //    slice between them (interleaved, so the workgroup reads contiguous spans of
 //    every weight row), keep eight 16-byte loads in flight per lane, and add their
 //    partial sums through LDS.  Activations come straight from L2.
-//  * gemm_tiled: everything else.  An output tile per workgroup (64 x 64 up to 64
-//    tokens, else 128 tokens x 64 or 128 features, whichever fills the compute
-//    units), K in slices of 64 staged through double-buffered LDS by range-checked
+//  * gemm_tiled: everything else.  An output tile per workgroup (128 x 128 when
+//    there are enough of those to fill the compute units, else 64 x 64), K in
+//    slices of 64 staged through double-buffered LDS by range-checked
 //    buffer loads (edge tiles and the tail of K read zeros, no branches), four
 //    wavefronts, 32x32x16 MFMA.  Workgroups are placed so that those resident on
 //    one XCD share operands in its L2.  Up to 16 tokens take this kernel too once
@@ -181,6 +181,7 @@ struct TiledShape {
   static constexpr int BN = 64 * WN;
   static constexpr int kPieces = (BM + BN) * (kBK / 8) / 256;  // 16-byte pieces per thread and slice
   static constexpr int kLds = 2 * (BM + BN) * kLd * 2;         // bytes, two buffers
+  static constexpr bool kDeep = WM * WN < 4;                   // loads two slices ahead for the small tiles
 };
 
 // Workgroup -> (slice, token tile, feature tile).  Consecutive workgroups go to the eight
@@ -209,7 +210,7 @@ __device__ __forceinline__ void place_workgroup(const TileOrder& order, int id, 
   nt = in_group / size;
 }
 
-template <int WM, int WN>
+template <int WM, int WN, bool DEEP>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                          GemmEpilogue ep, TileOrder order, int M, int N, int K) {
   using Shape = TiledShape<WM, WN>;
@@ -264,28 +265,27 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  bf16x8_t reg[PIECES];
-  auto fetch = [&](int slice) {
-    const int left = chunks - slice * (kBK / 8);  // chunks of K from this slice on
+  // The LDS buffers run one slice ahead of the matrix cores.  DEEP: two register sets, so
+  // that loads run two slices ahead (with a small tile one slice of work is shorter than a
+  // trip to memory); otherwise one.  A slice past the end reads zeros through the range
+  // check, so the loop bodies need no conditions on it.
+  bf16x8_t reg_a[PIECES], reg_b[DEEP ? PIECES : 1];
+  auto fetch = [&](int slice, auto& reg) {
+    const int left = slice < s_end ? chunks - slice * (kBK / 8) : 0;  // chunks of K from this slice on
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) {
       const unsigned off = piece_chunk[it] < left ? piece_off[it] + slice * (kBK * 2u) : kOutOfBuffer;
       reg[it] = buffer_load_bf16x8(it * 256 / 8 < BN ? w_buf : x_buf, off);
     }
+    // the loads are issued here, ahead of the products: the instruction scheduler would
+    // otherwise move them down next to the LDS stores that consume them
+    __builtin_amdgcn_sched_barrier(0);
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, const auto& reg) {
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + lds_off[it]) = reg[it];
   };
-
-  if (s_begin < s_end) {
-    fetch(s_begin);
-    stash(0);
-  }
-  __syncthreads();
-  for (int s = s_begin; s < s_end; ++s) {
-    const int buf = (s - s_begin) & 1;
-    if (s + 1 < s_end) fetch(s + 1);
+  auto multiply = [&](int buf) {
     const bf16* wt = lds + buf * kBuffer + (wn * 32 * WN + r32) * kLd + h * 8;
     const bf16* xt = lds + buf * kBuffer + (BN + wm * 32 * WM + r32) * kLd + h * 8;
 #pragma unroll
@@ -300,8 +300,32 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
         for (int j = 0; j < WM; ++j) acc[i][j] = mfma_32x32x16(a[i], b[j], acc[i][j]);
     }
-    if (s + 1 < s_end) stash(buf ^ 1);
-    __syncthreads();
+  };
+
+  fetch(s_begin, reg_a);
+  if constexpr (DEEP) fetch(s_begin + 1, reg_b);
+  stash(0, reg_a);
+  __syncthreads();
+  if constexpr (DEEP) {
+    for (int s = s_begin; s < s_end; s += 2) {
+      fetch(s + 2, reg_a);
+      multiply(0);
+      stash(1, reg_b);  // slice s + 1
+      __syncthreads();
+      if (s + 1 >= s_end) break;
+      fetch(s + 3, reg_b);
+      multiply(1);
+      stash(0, reg_a);  // slice s + 2
+      __syncthreads();
+    }
+  } else {
+    for (int s = s_begin; s < s_end; ++s) {
+      const int buf = (s - s_begin) & 1;
+      fetch(s + 1, reg_a);
+      multiply(buf);
+      stash(buf ^ 1, reg_a);
+      __syncthreads();
+    }
   }
 
 #pragma unroll
@@ -324,7 +348,7 @@ static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, 
   using Shape = TiledShape<WM, WN>;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, Shape::kDeep>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLds);
     if (e != hipSuccess) {
       set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
@@ -338,7 +362,7 @@ static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, 
     set_error("mlr_gemm_bf16: too many tiles for one launch");
     return -1;
   }
-  gemm_tiled_kernel<WM, WN><<<dim3(static_cast<unsigned>(groups)), 256, Shape::kLds, stream>>>(xb, wb, ep, order, m, n, k);
+  gemm_tiled_kernel<WM, WN, Shape::kDeep><<<dim3(static_cast<unsigned>(groups)), 256, Shape::kLds, stream>>>(xb, wb, ep, order, m, n, k);
   return 0;
 }
 
@@ -351,24 +375,38 @@ static int choose_slices(int groups, int ksteps, int allowed) {
   return slices;
 }
 
-// Workgroups of the 128 x 128 tiling for this shape.
-static int tiled_groups(int m, int n, int bn) { return ((n + bn - 1) / bn) * ((m + 127) / 128); }
+// Tiles of a shape under the 64 x 64 and the 128 x 128 tiling.
+static int tiles_64(int m, int n) { return ((n + 63) / 64) * ((m + 63) / 64); }
+static int tiles_128(int m, int n) { return ((n + 127) / 128) * ((m + 127) / 128); }
 
 // Up to 16 tokens: the LDS-tiled kernel once its 64-feature tiles (times slices) fill the
 // compute units, the 16-feature streaming kernel below that.
 static bool few_tokens_tiled(int n, int slices) { return ((n + 63) / 64) * slices >= 256; }
 
+// The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 = gemm_tiled with 64 x 64 and
+// 128 x 128 tiles.  The large tile needs less L2 traffic per flop and wins whenever there are
+// enough of them to fill the compute units.
+static int choose_kernel(int m, int n, int slices) {
+  if (m <= 16 && !few_tokens_tiled(n, slices)) return 16;
+  return (m > 64 && slices == 1 && tiles_128(m, n) >= 256) ? 22 : 11;
+}
+
 static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
-                     hipStream_t stream) {
-  if (m <= 16 && !few_tokens_tiled(n, slices)) {
-    dim3 grid((n + 15) / 16, slices);
-    gemm_skinny_split_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
-    return 0;
+                     int kernel, hipStream_t stream) {
+  switch (kernel) {
+    case 16: {
+      if (m > 16) {
+        set_error("mlr_gemm_bf16: the streaming kernel takes up to 16 tokens");
+        return -1;
+      }
+      dim3 grid((n + 15) / 16, slices);
+      gemm_skinny_split_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
+      return 0;
+    }
+    case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
+    case 22: return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 11 or 22"); return -1;
   }
-  if (m <= 64) return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
-  // too few 128 x 128 tiles to fill the compute units: halve the tile along the features
-  if (tiled_groups(m, n, 128) * slices < 256) return launch_tiled<2, 1>(xb, wb, ep, m, n, k, slices, stream);
-  return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
 }
 
 }  // namespace mlr
@@ -381,15 +419,9 @@ extern "C" {
 // partial sums (at most `max_slices`); 1 means it writes the finished product.
 int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
   if (k % 8 != 0) return 1;
-  if (m > 64) {
-    // tiled kernel: cut K while the grid is small and a slice keeps at least 8 LDS slices of 64
-    int slices = 1;
-    while (slices < max_slices && slices < 4 && tiled_groups(m, n, 128) * slices < 256 && k / (slices * 2) >= 8 * kBK)
-      slices *= 2;
-    return slices;
-  }
-  const int groups = m <= 16 ? (n + 15) / 16 : (n + 63) / 64;
-  return choose_slices(groups, (k / 8 + 3) / 4, max_slices);
+  if (m > 64 && tiles_128(m, n) >= 256) return 1;
+  const int groups = m <= 16 ? (n + 15) / 16 : tiles_64(m, n);
+  return choose_slices(groups, (k / 8 + 3) / 4, m > 64 ? min(max_slices, 4) : max_slices);
 }
 
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
@@ -399,7 +431,7 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
 // mlr_gemm_bf16_slices; not with swiglu) y is float32 [slices, m, n]: partial sums
 // over slices of k, the bias in slice 0, for the consumer to add up.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
-                  int swiglu, int slices, int m, int n, int k, hipStream_t stream) {
+                  int swiglu, int slices, int kernel, int m, int n, int k, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
@@ -410,7 +442,8 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
               "x and w must be 16-byte aligned");
   GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
-  if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, stream) != 0)
+  if (kernel == 0) kernel = choose_kernel(m, n, slices);
+  if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, kernel, stream) != 0)
     return -1;
   MLR_LAUNCH_CHECK();
   return 0;

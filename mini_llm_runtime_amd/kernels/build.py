@@ -40,6 +40,11 @@ FLAGS = [
     "-Xclang",
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # matrix-core accumulators in ordinary vector registers: every kernel here fits in 256 of
+    # them, and the separate accumulator file costs a copy per element whenever the vector
+    # ALU touches an accumulator (softmax rescaling, epilogues)
+    "-mllvm",
+    "-amdgpu-mfma-vgpr-form",
 ]
 HEADERS = ["api.h", "common.h", "mfma.h"]
 

@@ -35,7 +35,7 @@ _SIGNATURES = {
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
@@ -234,6 +234,8 @@ class HipOps:
         kernel: str = "auto",
         swiglu: bool = False,
         partial_sums: bool = False,
+        mfma_kernel: int = 0,
+        slices: Optional[int] = None,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
 
@@ -245,6 +247,8 @@ class HipOps:
         accepts, instead of [M, N], a float32 stack [S, M, N] of partial sums over slices
         of k (bias in slice 0).  Narrow products of a few tokens are cut that way so that
         all compute units stream the weight; the norm kernel adds the slices in order.
+        mfma_kernel, slices: force one of the matrix-core kernels (16, 11, 22) and a number
+        of k slices instead of letting the shape choose; for tests and tuning.
         """
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
@@ -261,9 +265,12 @@ class HipOps:
             raise KernelError(f"linear output must be float32 or {self.dtype}")
         bias_f32 = int(bias is not None and bias.dtype == torch.float32)
         if kernel == "auto" and self.dtype == torch.bfloat16 and k % 8 == 0:
-            slices = 1
-            if partial_sums and not swiglu:
-                slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices)
+            if slices is None:
+                slices = 1
+                if partial_sums and not swiglu:
+                    slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices)
+            elif slices < 1 or (slices > 1 and not (partial_sums and not swiglu)):
+                raise KernelError("k slices need partial_sums and no SwiGLU")
             if slices > 1:
                 y = self._empty((slices, m, n), torch.float32)
                 out_f32 = 1
@@ -272,7 +279,7 @@ class HipOps:
                 out_f32 = int(out_dtype == torch.float32)
             self._call(
                 "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-                int(swiglu), slices, m, n, k, self._stream(),
+                int(swiglu), slices, int(mfma_kernel), m, n, k, self._stream(),
             )
             return y
         y = self._empty((m, n // 2 if swiglu else n), out_dtype)
@@ -403,8 +410,8 @@ class HipOps:
         lib = None
         if use_mfma:
             lib = self.attention_library(head_dim)
-            if num_tiles and (block_size & (block_size - 1) or block_size > lib.mlr_attention_key_tile()):
-                use_mfma = False  # the tiled prefill kernel takes power-of-two pages up to its key tile
+            if num_tiles and (block_size & (block_size - 1) or not 8 <= block_size <= lib.mlr_attention_key_tile()):
+                use_mfma = False  # the tiled prefill kernel takes power-of-two pages from 8 up to its key tile
         if not use_mfma:
             self._call(
                 "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),

@@ -193,8 +193,8 @@ def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
         assert got.shape == (m, n)  # wide enough: not cut
         total = got.cpu().double()
     torch.testing.assert_close(total, ref, **(_tol(torch.bfloat16) if got.dim() == 2 else dict(atol=2e-3, rtol=1e-4)))
-    if k == 4864:
-        assert got.dim() == 3, "a long, narrow product should be cut along k"
+    if k >= 4104 and m <= 300:
+        assert got.dim() == 3, "a long, narrow product of few tokens should be cut along k"
     stream = _rand((m, n), torch.float32, 49, 2.0)
     nw = (1 + _rand((n,), torch.float32, 50, 0.1)).to(torch.bfloat16)
     sd = stream.cuda().clone()
@@ -207,6 +207,26 @@ def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
     picked = ops.gather_rows(got, rows).cpu()
     assert torch.equal(picked, got.cpu()[..., [m - 1, 0], :])
+
+
+@pytest.mark.parametrize("kernel", [16, 11, 22])
+@pytest.mark.parametrize("slices", [1, 3])
+def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
+    """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
+    shorter than an LDS slice, whole and cut along k."""
+    ops = ops_for(torch.bfloat16)
+    m, n, k = (13 if kernel == 16 else 150), 203, 1208
+    x = _rand((m, k), torch.bfloat16, 61)
+    w = _rand((n, k), torch.bfloat16, 62, 0.05)
+    b = _rand((n,), torch.float32, 63)
+    ref = x.double() @ w.double().t() + b.double()
+    got = ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, partial_sums=True, mfma_kernel=kernel, slices=slices)
+    assert got.shape == ((slices, m, n) if slices > 1 else (m, n))
+    total = got.cpu().double().sum(0) if slices > 1 else got.cpu().double()
+    torch.testing.assert_close(total, ref, atol=2e-3, rtol=1e-4)
+    if kernel != 16:
+        with pytest.raises(Exception, match="16 tokens"):
+            ops.linear(x.cuda(), w.cuda(), mfma_kernel=16)
 
 
 # ---- rotary encoding and cache write ----------------------------------------------------------------
