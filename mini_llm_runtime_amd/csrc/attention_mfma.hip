@@ -122,6 +122,7 @@ __device__ __forceinline__ s16x4_t softmax_tile(Softmax& st, f32x4_t s, const bo
 // ---- decode ---------------------------------------------------------------------------------
 constexpr int kDecodeWaves = D > 128 ? 2 : 4;  // bounded by the LDS the merge needs
 constexpr int kPartialStride = D + 2;  // numerator[D], max, denominator
+constexpr int kDecodeDepth = D > 128 ? 2 : 4;  // tiles of a wavefront in flight at once (registers)
 
 // Operands of one 16-key tile, loaded ahead of their use.
 struct DecodeTile {
@@ -223,40 +224,44 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   bool bad = false;
 
+  // The wavefronts take the partition's 16-key tiles in turn.  A tile's work is far shorter
+  // than a trip to memory, so a wavefront first issues the loads of up to kDecodeDepth of
+  // its tiles (a 256-key partition: all of them) and only then starts on the first.
   constexpr int kStride = kDecodeWaves * 16;
-  int ts = kb + wave * 16;
-  DecodeTile cur;
-  if (ts < ke)
-    cur = load_decode_tile(key_pages, value_pages, table, ts, ke, first, kvh, kv_heads, block_size, num_pages, col,
-                           quarter);
-  while (ts < ke) {
-    DecodeTile nxt;
-    const bool more = ts + kStride < ke;
-    if (more)  // the next tile's loads are in flight while this one is computed
-      nxt = load_decode_tile(key_pages, value_pages, table, ts + kStride, ke, first, kvh, kv_heads, block_size,
-                             num_pages, col, quarter);
-    bad = bad || cur.bad;
-    const f32x4_t s = score_tile(cur.k, qo);
-    bool ok[4];
+  const float scale2 = scale * 1.44269504088896340736f;
+  for (int ts0 = kb + wave * 16; ts0 < ke; ts0 += kDecodeDepth * kStride) {
+    DecodeTile tile[kDecodeDepth];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = ts + quarter * 4 + i;
-      ok[i] = key >= first && key < ke;
-      if (!ok[i]) {
+    for (int j = 0; j < kDecodeDepth; ++j)
+      if (ts0 + j * kStride < ke)
+        tile[j] = load_decode_tile(key_pages, value_pages, table, ts0 + j * kStride, ke, first, kvh, kv_heads,
+                                   block_size, num_pages, col, quarter);
 #pragma unroll
-        for (int dt = 0; dt < kDimTiles; ++dt) cur.v[dt][i] = 0;  // unwritten slots may hold NaN
+    for (int j = 0; j < kDecodeDepth; ++j) {
+      const int ts = ts0 + j * kStride;
+      if (ts >= ke) break;
+      DecodeTile& cur = tile[j];
+      bad = bad || cur.bad;
+      const f32x4_t s = score_tile(cur.k, qo);
+      bool ok[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = ts + quarter * 4 + i;
+        ok[i] = key >= first && key < ke;
+        if (!ok[i]) {
+#pragma unroll
+          for (int dt = 0; dt < kDimTiles; ++dt) cur.v[dt][i] = 0;  // unwritten slots may hold NaN
+        }
+      }
+      float alpha;
+      const s16x4_t pb = softmax_tile(sm, s, ok, scale2, alpha);
+#pragma unroll
+      for (int dt = 0; dt < kDimTiles; ++dt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+        acc[dt] = mfma_16x16x16(cur.v[dt], pb, acc[dt]);
       }
     }
-    float alpha;
-    const s16x4_t pb = softmax_tile(sm, s, ok, scale * 1.44269504088896340736f, alpha);
-#pragma unroll
-    for (int dt = 0; dt < kDimTiles; ++dt) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
-      acc[dt] = mfma_16x16x16(cur.v[dt], pb, acc[dt]);
-    }
-    if (more) cur = nxt;
-    ts += kStride;
   }
 
   // the column's sum is spread over the four lanes that share it

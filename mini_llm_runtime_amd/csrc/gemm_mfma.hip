@@ -115,10 +115,28 @@ __device__ __forceinline__ void finish4(const GemmEpilogue& ep, int slice, int s
 }
 
 // ---- skinny, up to 16 tokens: wavefronts split K ------------------------------------------
-template <int WAVES>
+// What the fused query/key/value product needs beside the product itself: the rotation
+// tables, the cache pages and where each token goes in them.
+struct QkvTarget {
+  const float* cos;  // [M, head_dim / 2], or null: no rotation
+  const float* sin;
+  const int* slots;  // [M] cache slot of each token (negative: none), or null: no cache write
+  bf16* key_pages;   // [page, kv_head, offset, head_dim]
+  bf16* value_pages; // [page, kv_head, head_dim, offset]
+  bf16* q_out;       // [M, heads * head_dim]
+  int heads, kv_heads, head_dim, block_size, num_pages;
+};
+
+// QKV: w is [(heads + 2 kv_heads) * head_dim, K], the rows of the query heads, then the key
+// heads, then the value heads.  A workgroup of the rotated part owns 8 dims j..j+7 of a head
+// AND their partners j + head_dim/2 .. (src/mini_llm_runtime/qwen_model_runner.py:56-61 pairs
+// dim j with j + head_dim/2), so the rotation happens on the sums before anything is stored:
+// queries go to q_out, keys and values straight into their pages (:105-109).
+template <int WAVES, bool QKV>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf16* __restrict__ x,
                                                                        const bf16* __restrict__ w,
-                                                                       GemmEpilogue ep, int M, int N, int K) {
+                                                                       GemmEpilogue ep, QkvTarget qkv, int M, int N,
+                                                                       int K) {
   constexpr int U = 8;  // k-steps in flight per wavefront
   __shared__ float red[WAVES][kWave][4];
   const int lane = threadIdx.x % kWave;
@@ -132,7 +150,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   const int per = (ksteps + slices - 1) / slices;
   const int sb = blockIdx.y * per;
   const int se = min(ksteps, sb + per);
-  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(n0 + r, N - 1)) * K);
+  // the weight row behind accumulator row `slot` of this workgroup
+  int head = 0, block_in_head = 0;
+  bool rotated = false;
+  if constexpr (QKV) {
+    const int per_head = qkv.head_dim / 16;
+    head = blockIdx.x / per_head;
+    block_in_head = blockIdx.x - head * per_head;
+    rotated = qkv.cos != nullptr && head < qkv.heads + qkv.kv_heads;
+  }
+  auto row_of = [&](int slot) {
+    if (!rotated) return n0 + slot;
+    return head * qkv.head_dim + block_in_head * 8 + (slot < 8 ? slot : qkv.head_dim / 2 + slot - 8);
+  };
+  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(row_of(r), N - 1)) * K);
   const bf16x8_t* xp = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(r, M - 1)) * K);
   const bool xok = r < M;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -158,12 +189,59 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
   __syncthreads();
-  if (wave == 0) {
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int ww = 0; ww < WAVES; ++ww)
+  if (wave != 0) return;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] += red[ww][lane][i];
+    for (int i = 0; i < 4; ++i) v[i] += red[ww][lane][i];
+  if constexpr (!QKV) {
     finish4(ep, blockIdx.y, slices, r, n0 + q * 4, M, N, v);
+  } else {
+    // the lane holds token r, accumulator rows 4q..4q+3: four consecutive dims of one head
+    const int D = qkv.head_dim;
+    const int d0 = row_of(q * 4) - head * D;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (ep.bias != nullptr) v[i] += load_as_f32(ep.bias, head * D + d0 + i, ep.bias_is_f32);
+      v[i] = to_f32(f32_to_bf16(v[i]));  // the product as bfloat16, as the unfused kernels hand it on
+    }
+    if (rotated) {
+      // lanes q and q ^ 2 of a token hold the two halves of the same pairs
+      const int half = D / 2;
+      const int j0 = block_in_head * 8 + (q & 1) * 4;
+      const int t = min(r, M - 1);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float partner = __shfl_xor(v[i], 32, kWave);
+        const float c = qkv.cos[static_cast<int64_t>(t) * half + j0 + i];
+        const float sn = qkv.sin[static_cast<int64_t>(t) * half + j0 + i];
+        v[i] = q < 2 ? v[i] * c - partner * sn : v[i] * c + partner * sn;
+      }
+    }
+    if (r >= M) return;
+    u16x4_t packed;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(v[i]).bits;
+    if (head < qkv.heads) {
+      *reinterpret_cast<u16x4_t*>(qkv.q_out + (static_cast<int64_t>(r) * qkv.heads + head) * D + d0) = packed;
+      return;
+    }
+    if (qkv.slots == nullptr) return;
+    const int slot = qkv.slots[r];
+    if (slot < 0) return;
+    const int page = slot / qkv.block_size;
+    const int off = slot - page * qkv.block_size;
+    if (page >= qkv.num_pages) return;
+    if (head < qkv.heads + qkv.kv_heads) {
+      const int kvh = head - qkv.heads;
+      bf16* dst = qkv.key_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * qkv.block_size + off) * D + d0;
+      *reinterpret_cast<u16x4_t*>(dst) = packed;
+    } else {
+      const int kvh = head - qkv.heads - qkv.kv_heads;
+      bf16* dst = qkv.value_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * D + d0) * qkv.block_size + off;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[static_cast<int64_t>(i) * qkv.block_size].bits = packed[i];
+    }
   }
 }
 
@@ -400,7 +478,7 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
         return -1;
       }
       dim3 grid((n + 15) / 16, slices);
-      gemm_skinny_split_kernel<4><<<grid, 256, 0, stream>>>(xb, wb, ep, m, n, k);
+      gemm_skinny_split_kernel<4, false><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
       return 0;
     }
     case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
@@ -445,6 +523,36 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   if (kernel == 0) kernel = choose_kernel(m, n, slices);
   if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, kernel, stream) != 0)
     return -1;
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+// The query/key/value product of up to 16 tokens with everything that follows it before
+// attention: bias, rotation of the query and key heads (cos, sin: [m, head_dim / 2] float32,
+// or null for none), queries to q_out [m, heads * head_dim], keys and values into the slots
+// of their pages (`write` 0: another layer owns the pages).  w is [(heads + 2 kv_heads) *
+// head_dim, k]; head_dim a multiple of 16, k of 8.
+int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
+                            const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
+                            int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
+                            int write, hipStream_t stream) {
+  MLR_REQUIRE(x && w && q_out, "null pointer");
+  MLR_REQUIRE(m > 0 && m <= 16, "the fused product takes 1..16 tokens");
+  MLR_REQUIRE(k > 0 && k % 8 == 0, "k must be a positive multiple of 8");
+  MLR_REQUIRE(heads > 0 && kv_heads > 0 && head_dim >= 16 && head_dim % 16 == 0, "head_dim must be a multiple of 16");
+  MLR_REQUIRE((cos == nullptr) == (sin == nullptr), "cos and sin come together");
+  MLR_REQUIRE(!write || (slots && key_pages && value_pages && block_size > 0 && num_pages > 0),
+              "a cache write needs slots, pages and their sizes");
+  MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(q_out) % 8 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 8 == 0,
+              "operands must be 16-byte aligned");
+  const int64_t n = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  MLR_REQUIRE(n / 16 < (1ll << 31), "too many rows for one launch");
+  GemmEpilogue ep{bias, bias_is_f32, nullptr, 0, 0};
+  QkvTarget target{cos, sin, write ? slots : nullptr, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages),
+                   static_cast<bf16*>(q_out), heads, kv_heads, head_dim, block_size, num_pages};
+  gemm_skinny_split_kernel<4, true><<<dim3(static_cast<unsigned>(n / 16)), 256, 0, stream>>>(
+      static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, target, m, static_cast<int>(n), k);
   MLR_LAUNCH_CHECK();
   return 0;
 }

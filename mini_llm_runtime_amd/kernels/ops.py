@@ -37,6 +37,10 @@ _SIGNATURES = {
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
+    "mlr_qkv_rope_write_bf16": (
+        [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        _I,
+    ),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
         _I,
@@ -351,6 +355,73 @@ class HipOps:
             self._ptr(value_pages if write else None), tokens, num_heads, num_kv_heads, head_dim, rotary_dim,
             block_size, num_pages, int(write), self._stream(),
         )
+
+    def qkv_rope_write(
+        self,
+        x: torch.Tensor,
+        weight: torch.Tensor,
+        bias: Optional[torch.Tensor],
+        rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+        slot_mapping: torch.Tensor,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        *,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        block_size: int,
+        write: bool = True,
+        fused: Optional[bool] = None,
+    ) -> torch.Tensor:
+        """Query/key/value product, rotation of queries and keys, keys and values into the cache.
+
+        Returns a tensor whose leading num_heads * head_dim columns are the position-encoded
+        queries, for `paged_attention`.  Up to 16 bfloat16 tokens (decoding) run as ONE kernel
+        that rotates the sums and stores them where they belong; everything else is the product
+        followed by `rope_kv_write`.  `fused` forces one of the two ways (tests).
+        """
+        m, k = x.shape
+        can_fuse = (
+            self.dtype == torch.bfloat16
+            and m <= 16
+            and k % 8 == 0
+            and head_dim % 16 == 0
+            and (rotation is None or rotation[2] == head_dim)
+        )
+        if fused is None:
+            fused = can_fuse
+        elif fused and not can_fuse:
+            raise KernelError("the fused query/key/value kernel takes up to 16 bfloat16 tokens and a full rotation")
+        if not fused:
+            qkv = self.linear(x, weight, bias)
+            self.rope_kv_write(
+                qkv, rotation, slot_mapping, key_pages, value_pages, num_heads=num_heads,
+                num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size, write=write,
+            )
+            return qkv
+        width = (num_heads + 2 * num_kv_heads) * head_dim
+        self._check(x, "linear input", self.dtype, (None, None))
+        self._check(weight, "qkv weight", self.dtype, (width, k))
+        if bias is not None:
+            self._check(bias, "qkv bias", (torch.float32, self.dtype), (width,))
+        cos = sin = None
+        if rotation is not None:
+            cos, sin, _ = rotation
+            self._check(cos, "rotary cos", torch.float32, (m, head_dim // 2))
+            self._check(sin, "rotary sin", torch.float32, (m, head_dim // 2))
+        num_pages = 0
+        if write:
+            num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
+            self._check(slot_mapping, "slot mapping", torch.int32, (m,))
+        q = self._empty((m, num_heads * head_dim), self.dtype)
+        self._call(
+            "mlr_qkv_rope_write_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias),
+            int(bias is not None and bias.dtype == torch.float32), self._ptr(cos), self._ptr(sin),
+            self._ptr(slot_mapping if write else None), self._ptr(key_pages if write else None),
+            self._ptr(value_pages if write else None), self._ptr(q), m, k, num_heads, num_kv_heads, head_dim,
+            block_size, num_pages, int(write), self._stream(),
+        )
+        return q
 
     def paged_attention(
         self,

@@ -94,25 +94,27 @@ class GQAAttention(Mixer):
     def forward(self, ctx: StepContext, h: torch.Tensor, site: int) -> torch.Tensor:
         ops = ctx.ops
         cache = ctx.kv(site)
-        qkv = ops.linear(h, self.qkv_weight, self.qkv_bias_vec)
         rotation = self.position.rotation(ctx) if self.position is not None else None
-        if self.position is not None and rotation is None:
-            tokens = qkv.shape[0]
-            q = qkv[:, : self.q_size].view(tokens, self.num_heads, self.head_dim)
-            k = qkv[:, self.q_size : self.q_size + self.kv_size].view(tokens, self.num_kv_heads, self.head_dim)
-            self.position.apply(ctx, q, k)
-        ops.rope_kv_write(
-            qkv,
-            rotation,
-            cache.slot_mapping,
-            cache.key,
-            cache.value,
+        pages = dict(
             num_heads=self.num_heads,
             num_kv_heads=self.num_kv_heads,
             head_dim=self.head_dim,
             block_size=cache.block_size,
             write=cache.writable,
         )
+        if self.position is not None and rotation is None:
+            # a position encoding with a rule of its own: it sees the queries and keys between
+            # the product and the cache write
+            qkv = ops.linear(h, self.qkv_weight, self.qkv_bias_vec)
+            tokens = qkv.shape[0]
+            q = qkv[:, : self.q_size].view(tokens, self.num_heads, self.head_dim)
+            k = qkv[:, self.q_size : self.q_size + self.kv_size].view(tokens, self.num_kv_heads, self.head_dim)
+            self.position.apply(ctx, q, k)
+            ops.rope_kv_write(qkv, None, cache.slot_mapping, cache.key, cache.value, **pages)
+        else:
+            qkv = ops.qkv_rope_write(
+                h, self.qkv_weight, self.qkv_bias_vec, rotation, cache.slot_mapping, cache.key, cache.value, **pages
+            )
         attended = ops.paged_attention(
             qkv,
             cache.key,

@@ -96,6 +96,11 @@ class TorchOps:
             key_pages[page, :, off, :] = k[ok]
             value_pages[page, :, :, off] = v[ok]
 
+    def qkv_rope_write(self, x, weight, bias, rotation, slot_mapping, key_pages, value_pages, **sizes):
+        qkv = self.linear(x, weight, bias)
+        self.rope_kv_write(qkv, rotation, slot_mapping, key_pages, value_pages, **sizes)
+        return qkv
+
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window
     ):

@@ -288,6 +288,45 @@ def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
     assert torch.equal(out[0, : heads * head_dim], qkv[0, : heads * head_dim])
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,tokens,rotate,write", [
+    (14, 2, 64, 896, 8, True, True), (3, 1, 16, 40, 1, True, True), (6, 3, 48, 104, 16, True, True),
+    (4, 4, 80, 72, 5, False, True), (5, 1, 128, 136, 13, True, False),
+])
+def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write):
+    """Decoding runs product, bias, rotation and cache write as one kernel; it has to leave the
+    queries and the pages exactly as the product followed by the rotation kernel does, and must
+    not touch any slot but the tokens' own (a token without a slot writes nothing)."""
+    ops = ops_for(torch.bfloat16)
+    bs, pages = 8, 7
+    width = (heads + 2 * kv_heads) * head_dim
+    x = _rand((tokens, hidden), torch.bfloat16, 71).cuda()
+    w = _rand((width, hidden), torch.bfloat16, 72, 0.2).cuda()
+    b = _rand((width,), torch.float32, 73).cuda()
+    rotation = None
+    if rotate:
+        pos = torch.tensor([3, 0, 911, 17, 40000, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15][:tokens], dtype=torch.int32).cuda()
+        inv = (1.0 / (1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))).cuda()
+        cos, sin = ops.rope_table(pos, inv)
+        rotation = (cos, sin, head_dim)
+    g = torch.Generator().manual_seed(74)
+    slots = torch.randperm(pages * bs, generator=g)[:tokens].to(torch.int32)
+    if tokens > 2:
+        slots[2] = -1
+    slots = slots.cuda()
+    out = {}
+    for fused in (False, True):
+        kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=torch.bfloat16).cuda()
+        vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=torch.bfloat16).cuda()
+        q = ops.qkv_rope_write(x, w, b, rotation, slots, kp, vp, num_heads=heads, num_kv_heads=kv_heads,
+                               head_dim=head_dim, block_size=bs, write=write, fused=fused)
+        out[fused] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
+    for name, a, c in zip(("queries", "key pages", "value pages"), out[False], out[True]):
+        assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
+        # the rotation's two products may be contracted differently: a last-place difference at most
+        torch.testing.assert_close(torch.nan_to_num(c), torch.nan_to_num(a), atol=0, rtol=2 ** -7, msg=lambda m: f"{name}: {m}")
+    assert torch.isnan(out[True][1]).all() == (not write)
+
+
 # ---- attention ----------------------------------------------------------------------------------------
 def _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, seed, extra_pages=3, spike=False):
     """entries: list of (context_len, q_len).  Returns device inputs and the float64 expectation."""
