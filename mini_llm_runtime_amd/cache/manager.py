@@ -116,6 +116,33 @@ class RequestCache:
     def live_blocks(self, group: int) -> list[int]:
         return [b for b in self.tables[group] if b >= 0]
 
+    def table_array(self, group: int) -> np.ndarray:
+        """`tables[group]` as int32; kept between steps and only extended when pages were
+        appended, rebuilt when the table changed in any other way."""
+        table = self.tables[group]
+        cache = self.__dict__.setdefault("_table_arrays", {})
+        kept = cache.get(group)
+        n = len(table)
+        if kept is not None:
+            array, length, stamp = kept
+            if stamp == self.__dict__.get("_table_stamp", 0) and length <= n:
+                if length < n:
+                    if n > array.shape[0]:
+                        grown = np.empty(max(n, 2 * array.shape[0]), dtype=np.int32)
+                        grown[:length] = array[:length]
+                        array = grown
+                    array[length:n] = table[length:]
+                    cache[group] = (array, n, stamp)
+                return array[:n]
+        array = np.empty(max(16, 2 * n), dtype=np.int32)
+        array[:n] = table
+        cache[group] = (array, n, self.__dict__.get("_table_stamp", 0))
+        return array[:n]
+
+    def tables_changed(self) -> None:
+        """Entries of `tables` were overwritten or removed (not just appended)."""
+        self.__dict__["_table_stamp"] = self.__dict__.get("_table_stamp", 0) + 1
+
 
 @dataclass
 class _PendingEntry:
@@ -356,6 +383,7 @@ class CacheManager:
                 if request.tables[i][-len(ids) :] != ids:
                     raise RuntimeError("pages of an aborted step are no longer the table's tail")
                 del request.tables[i][-len(ids) :]
+                request.tables_changed()
                 g.allocator.free(ids, to_reserved=entry.from_reserved[i])
                 request.reserved[i] += entry.from_reserved[i]
             request.pending_tokens = 0
@@ -387,6 +415,7 @@ class CacheManager:
                 request.reserved[i] += keep
                 for j in range(dead):
                     request.tables[i][j] = -1
+                request.tables_changed()
                 passed.setdefault(request.request_id, {})[i] = tuple(ids)
         return passed
 
@@ -399,30 +428,31 @@ class CacheManager:
         cu_q = np.zeros(count + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu_q[1:])
         total = int(cu_q[-1])
-        positions = np.empty(total, dtype=np.int32)
-        token_entry = np.empty(total, dtype=np.int32)
-        for r in range(count):
-            a, b = int(cu_q[r]), int(cu_q[r + 1])
-            positions[a:b] = np.arange(q_starts[r], context[r], dtype=np.int32)
-            token_entry[a:b] = r
+        if total == count:  # one token each
+            positions = q_starts.copy()
+            token_entry = np.arange(count, dtype=np.int32)
+        else:
+            positions = np.empty(total, dtype=np.int32)
+            token_entry = np.empty(total, dtype=np.int32)
+            for r in range(count):
+                a, b = int(cu_q[r]), int(cu_q[r + 1])
+                positions[a:b] = np.arange(q_starts[r], context[r], dtype=np.int32)
+                token_entry[a:b] = r
+        used = (context + (bs - 1)) // bs  # pages each entry has with this step's tokens
+        width = max(1, int(used.max()))
         block_tables: list[np.ndarray] = []
         slot_mappings: list[np.ndarray] = []
         for i, g in enumerate(self.groups):
-            width = max(1, max(blocks_for(int(c), bs) for c in context))
             table = np.full((count, width), -1, dtype=np.int32)
-            slots = np.empty(total, dtype=np.int32)
             for r, e in enumerate(pending):
-                row = e.request.tables[i]
-                used = blocks_for(int(context[r]), bs)
-                table[r, :used] = row[:used]
-                a, b = int(cu_q[r]), int(cu_q[r + 1])
-                pos = positions[a:b]
-                pages = table[r, pos // bs]
-                if (pages < 0).any():
-                    raise RuntimeError(f"request {e.request.request_id!r}: a new token has no page")
-                slots[a:b] = pages * bs + pos % bs
+                n = int(used[r])
+                table[r, :n] = e.request.table_array(i)[:n]
+            pages = table[token_entry, positions // bs]
+            if (pages < 0).any():
+                r = int(token_entry[int(np.argmax(pages < 0))])
+                raise RuntimeError(f"request {pending[r].request.request_id!r}: a new token has no page")
             block_tables.append(table)
-            slot_mappings.append(slots)
+            slot_mappings.append((pages * bs + positions % bs).astype(np.int32))
         slot_ids = np.array([e.request.slot for e in pending], dtype=np.int32)
         parity = np.array([e.request.state_parity for e in pending], dtype=np.int32)
         return StepLayout(

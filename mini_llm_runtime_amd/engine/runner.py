@@ -95,6 +95,7 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
         self.max_graph_batch = int(max_graph_batch)
         self._graphs: dict[tuple[int, int], tuple] = {}
+        self._staging: dict[tuple[int, int], list] = {}
 
     # -------------------------------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -243,16 +244,62 @@ class ModelRunner:
         quantum = max(1, 1024 // bs)  # table widths in steps of 1,024 tokens
         return padded, -(-pages // quantum) * quantum
 
+    def _graph_staging(self, key: tuple[int, int], spans, size: int):
+        """Two pinned host buffers per graph (a step fills one while the other may still be
+        read by the previous step's copy), each with int32 views in the order of `_arrays`."""
+        staging = self._staging.get(key)
+        if staging is None:
+            buffers = []
+            for _ in range(2):
+                host = torch.zeros(size, dtype=torch.int32, pin_memory=self._pinned)
+                flat = host.numpy()
+                views = [flat[start : start + (int(np.prod(shape)) if shape else 1)].reshape(shape) for start, shape in spans]
+                buffers.append([host, views, None])
+            staging = [buffers, 0]
+            self._staging[key] = staging
+        buffers, turn = staging
+        staging[1] = turn ^ 1
+        slot = buffers[turn]
+        if slot[2] is not None:
+            slot[2].synchronize()  # the copy that last read this buffer
+        return slot
+
+    def _fill_padded(self, views, layout: StepLayout, token_ids: np.ndarray) -> None:
+        """`_arrays(..., pad_entries, table_width)` written into the views of a staging buffer.
+        The views of the constant arrays (token_entry, cu_q, logit rows) were set when the
+        buffer was made."""
+        count = layout.num_entries
+        for view, values, fill in (
+            (views[0], token_ids, 0), (views[1], layout.positions, 0), (views[4], layout.q_starts, 0),
+            (views[5], layout.context_lens, 0), (views[6], layout.state_read, 0), (views[7], layout.state_write, 0),
+        ):
+            view[:count] = values
+            view[count:] = fill
+        groups = len(layout.slot_mappings)
+        for g in range(groups):
+            view = views[10 + g]
+            view[:count] = layout.slot_mappings[g]
+            view[count:] = -1
+            table = views[10 + groups + g]
+            t = layout.block_tables[g]
+            table[:count, : t.shape[1]] = t
+            table[:count, t.shape[1] :] = -1
+            table[count:] = -1
+
     def _forward_graph(
         self, key: tuple[int, int], layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray
     ) -> torch.Tensor:
         padded, width = key
-        empty = np.zeros((0, 2), dtype=np.int32)
-        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, empty, padded, width))
         graph = self._graphs.get(key)
         if graph is None:
-            static = torch.empty_like(host, device=self.device)
-            static.copy_(host, non_blocking=True)
+            empty = np.zeros((0, 2), dtype=np.int32)
+            arrays = self._arrays(layout, token_ids, logit_rows, empty, padded, width)
+            buf, spans = _pack_int32(arrays)
+            slot = self._graph_staging(key, spans, buf.size)
+            for other in self._staging[key][0]:
+                other[0].numpy()[:] = buf  # the constant arrays, once
+            static = torch.empty(buf.size, dtype=torch.int32, device=self.device)
+            static.copy_(slot[0], non_blocking=True)
             ctx = self._context(
                 static,
                 spans,
@@ -272,10 +319,16 @@ class ModelRunner:
             captured = torch.cuda.CUDAGraph()
             with torch.cuda.graph(captured):
                 out = self.model.forward(ctx, ctx.memo["logit_rows"])
-            graph = (captured, static, out)
+            graph = (captured, static, out, spans, buf.size)
             self._graphs[key] = graph
-        captured, static, out = graph
-        static.copy_(host, non_blocking=True)
+        captured, static, out, spans, size = graph
+        slot = self._graph_staging(key, spans, size)
+        self._fill_padded(slot[1], layout, token_ids)
+        static.copy_(slot[0], non_blocking=True)
+        if self._pinned:
+            done = slot[2] or torch.cuda.Event()
+            done.record(torch.cuda.current_stream(self.device))
+            slot[2] = done
         captured.replay()
         if logit_rows.size == layout.num_entries and (logit_rows == np.arange(layout.num_entries)).all():
             return out[: layout.num_entries]
