@@ -4,8 +4,8 @@
 
 Default run: the Qwen2.5-0.5B shape in bfloat16, 8 requests with 2,048-token
 random-id prompts (context capacity 4,096, KV block 16).  A step is one decode
-step of the whole engine: the step function over the batch, sampling on the GPU
-and the copy of the chosen tokens to the host.  W warm-up steps, then exactly K
+step of the whole continuous-batching engine: scheduling, the step function over
+the batch, sampling on the GPU and the copy of the chosen tokens to the host.  W warm-up steps, then exactly K
 timed steps between device synchronisations.  One JSON line is printed:
 `value` is decoded tokens per second at batch 8; `points` holds batch 1 and 64;
 `prefill` is one 2,048-token prompt; `roofline` prices the decode step by the
@@ -57,6 +57,7 @@ def main() -> int:
     import mini_llm_runtime_amd  # noqa: F401
     from mini_llm_runtime_amd.config.presets import load_preset
     from mini_llm_runtime_amd.engine.factory import default_ops, load_model, make_cache, parse_dtype
+    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
     from mini_llm_runtime_amd.engine.runner import ModelRunner, StepEntry
     from mini_llm_runtime_amd.models.registry import config_from_dict
     from mini_llm_runtime_amd.sampling.sampler import Sampler
@@ -78,7 +79,7 @@ def main() -> int:
 
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
     steps_total = args.warmup + args.steps
-    capacity = max(CONTEXT_LEN, args.prompt_len + steps_total + 1)
+    capacity = max(CONTEXT_LEN, args.prompt_len + steps_total + max(batches) + 9)
     pages = max(batches) * (-(-capacity // BLOCK_SIZE)) + 8
     cache = make_cache(model, block_size=BLOCK_SIZE, num_blocks=pages, max_requests=max(batches))
     runner = ModelRunner(model, cache, ops)
@@ -93,31 +94,31 @@ def main() -> int:
         torch.cuda.synchronize(device)
 
     def decode(batch: int, warmup: int, steps: int) -> float:
-        """ms per decode step at this batch size, contexts starting at prompt_len."""
-        ids = [f"b{batch}-{i}" for i in range(batch)]
-        last = []
-        for rid in ids:
-            cache.create_request(rid)
-            out = runner.step([StepEntry.of(rid, prompt(), (args.prompt_len - 1,))])
-            last.append(int(sampler.sample(out.logits, [_GREEDY], [0]).cpu()[0]))
-        params = [_GREEDY] * batch
-        counts = [1] * batch
-
-        def one_step() -> None:
-            nonlocal last
-            out = runner.step([StepEntry(rid, (tok,), (0,)) for rid, tok in zip(ids, last)])
-            last = sampler.sample(out.logits, params, counts).cpu().tolist()
-
+        """ms per decode step of the continuous-batching engine at this batch size, contexts
+        starting at prompt_len: scheduler, step function, sampling on the GPU, tokens to the host."""
+        admission = PagedBlockAdmissionController(cache, max_step_tokens=args.prompt_len)
+        scheduler = RequestScheduler(
+            max_running_requests=batch,
+            max_batch_tokens=max(args.prompt_len, batch),
+            admission_callback=admission.try_admit,
+        )
+        engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
+        for i in range(batch):
+            engine.submit(f"b{batch}-{i}", prompt(), max_new_tokens=warmup + steps + batch + 8)
+        while True:  # prompts, until a step is nothing but one token for every request
+            result = engine.step()
+            if len(result.batch.decode_request_ids) == batch:
+                break
         for _ in range(warmup):
-            one_step()
+            engine.step()
         sync()
         t0 = time.perf_counter()
         for _ in range(steps):
-            one_step()
+            result = engine.step()
         sync()
         elapsed = time.perf_counter() - t0
-        for rid in ids:
-            cache.release_request(rid)
+        assert len(result.batch.decode_request_ids) == batch and len(result.update.emitted_tokens) == batch
+        engine.run_until_done()
         return elapsed * 1e3 / steps
 
     from mini_llm_runtime_amd.sampling.sampler import GREEDY as _GREEDY

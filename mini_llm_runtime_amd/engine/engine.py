@@ -9,6 +9,18 @@ On any exception the step's newly admitted requests are released and the
 scheduler's batch is undone, so the same step can be tried again
 (engine.py:249-254).  Unlike the reference, which runs prompts and decodes as two
 forwards (engine.py:186-248), a step here is one forward over the whole batch.
+
+Decoding one step ahead.  The host's share of a decode step (scheduling, block
+tables, the launch itself, waiting for the chosen tokens) is a good part of the
+step's time for a small model, and the GPU would idle through it.  So, before it
+waits for the tokens of step k, the engine launches step k+1 for the same requests
+with the token ids taken on the device from the sampler's output; nothing about
+that step counts yet.  When the scheduler, now knowing step k's tokens, asks for
+exactly that step, it is committed and only its tokens are waited for; when it
+asks for anything else (a request finished, another was admitted) the launch is
+abandoned: its pages go back, and what it wrote is overwritten by the steps that
+follow it on the stream.  Results, their order and the scheduler's decisions are
+those of the plain loop.
 """
 
 from __future__ import annotations
@@ -24,7 +36,7 @@ import torch
 from ..sampling.sampler import GREEDY, Sampler, SamplingParams
 from .admission import PagedBlockAdmissionController
 from .metrics import RequestMetricsCollector
-from .runner import ModelRunner, StepEntry
+from .runner import ModelRunner, StepEntry, StepOutput
 from .scheduler import (
     BatchingPolicy,
     RequestScheduler,
@@ -45,6 +57,35 @@ def _trace_range(enabled: bool, message: str) -> Iterator[None]:
     finally:
         if enabled:
             torch.cuda.nvtx.range_pop()
+
+
+class _TokensOnTheWay:
+    """The chosen tokens of one step, being copied to the host.  The copy is put on the
+    stream right behind the sampling, BEFORE any later step is launched, and waited for by
+    its own event: waiting for it then does not wait for what was launched after it."""
+
+    def __init__(self, chosen: torch.Tensor) -> None:
+        self.device_tokens = chosen
+        self._event = None
+        if chosen.device.type == "cuda":
+            self._host = torch.empty(chosen.shape, dtype=chosen.dtype, pin_memory=True)
+            self._host.copy_(chosen, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record(torch.cuda.current_stream(chosen.device))
+        else:
+            self._host = chosen
+
+    def wait(self) -> list[int]:
+        if self._event is not None:
+            self._event.synchronize()
+        return self._host.tolist()
+
+
+@dataclass
+class _LaunchedAhead:
+    request_ids: tuple[str, ...]
+    output: "StepOutput"
+    chosen: _TokensOnTheWay
 
 
 @dataclass(frozen=True)
@@ -68,6 +109,7 @@ class ContinuousBatchEngine:
         clock_ns: Callable[[], int] = time.perf_counter_ns,
         metrics: Optional[RequestMetricsCollector] = None,
         enable_tracing: bool = False,
+        lookahead: bool = True,
     ) -> None:
         if admission.manager is not runner.cache:
             raise ValueError("the admission controller and the runner must share one cache manager")
@@ -82,6 +124,11 @@ class ContinuousBatchEngine:
         self._clock_ns = clock_ns
         self.metrics = metrics or RequestMetricsCollector()
         self.enable_tracing = enable_tracing
+        self.lookahead = bool(lookahead)
+        self._ahead: Optional[_LaunchedAhead] = None
+        self.lookahead_hits = 0
+        self.lookahead_misses = 0
+        self.lookahead_error: Optional[Exception] = None  # what switched the lookahead off, if anything did
 
     @property
     def manager(self):
@@ -158,6 +205,7 @@ class ContinuousBatchEngine:
         with _trace_range(self.enable_tracing, "scheduler.schedule_step"):
             batch = self.scheduler.schedule_step()
         if batch is None:
+            self._drop_ahead()
             return None
         label = (
             f"engine.step:{batch.step_index}:prefill={len(batch.prefill_request_ids)}:"
@@ -181,23 +229,40 @@ class ContinuousBatchEngine:
                 if item.produces_token:
                     params.append(request.sampling)
                     indices.append(len(request.generated_token_ids))
-            with _trace_range(self.enable_tracing, f"model.step:tokens={batch.token_count}"):
-                output = self.runner.step(entries)
-            chosen = None
-            if output.logits is not None:
-                chosen = self.sampler.sample(output.logits, params, indices)
+            ahead = self._take_ahead(batch)
+            if ahead is not None:
+                output = self.runner.commit(ahead.output)
+                chosen = ahead.chosen
+            else:
+                with _trace_range(self.enable_tracing, f"model.step:tokens={batch.token_count}"):
+                    output = self.runner.step(entries)
+                chosen = None
+                if output.logits is not None:
+                    chosen = _TokensOnTheWay(self.sampler.sample(output.logits, params, indices))
         except Exception:
+            self._drop_ahead()
             with _trace_range(self.enable_tracing, "engine.rollback"):
                 self.admission.release_admitted(batch.admitted_request_ids)
                 self.scheduler.abort_step()
             raise
 
+        if self.lookahead and chosen is not None:
+            # step k is launched and counted; a failure to launch k+1 early must not undo it
+            try:
+                with _trace_range(self.enable_tracing, "model.step:ahead"):
+                    self._ahead = self._launch_ahead(batch, output, chosen.device_tokens, params, indices)
+            except Exception as error:  # noqa: BLE001 - decoding goes on without the lookahead
+                self._ahead = None
+                self.lookahead = False
+                self.lookahead_error = error
         with _trace_range(self.enable_tracing, "token.d2h_sync"):
-            host_tokens = chosen.cpu().tolist() if chosen is not None else []
+            host_tokens = chosen.wait() if chosen is not None else []
         tokens_ready_ns = self._clock_ns()
         generated = {rid: int(tok) for (rid, _), tok in zip(output.rows, host_tokens)}
         with _trace_range(self.enable_tracing, "scheduler.apply_and_release"):
             update = self.scheduler.apply_step_results(generated)
+            if update.finished_request_ids:
+                self._drop_ahead()  # it holds pages of a request that is about to be released
             released = self.admission.release_finished(update.finished_request_ids)
         completed_ns = self._clock_ns()
         self.metrics.record_tokens(update.emitted_tokens, tokens_ready_ns)
@@ -210,6 +275,63 @@ class ContinuousBatchEngine:
             tokens_ready_ns=tokens_ready_ns,
             completed_ns=completed_ns,
         )
+
+    # ---- the step launched ahead ----------------------------------------------------------------------
+    def _launch_ahead(self, batch, output: StepOutput, chosen, params, indices) -> Optional[_LaunchedAhead]:
+        """Launch the next step now if it is bound to be one token for each request of this
+        batch: all running requests produced a token here, none of them ends by length with
+        it, and nobody waits who could be admitted.  (A request may still end on an
+        end-of-sequence token; then the launch is abandoned.)"""
+        scheduler = self.scheduler
+        running = scheduler.running_request_ids
+        produced = [rid for rid, _ in output.rows]
+        if not running or sorted(running) != sorted(produced):
+            return None
+        if scheduler.waiting_request_ids and len(running) < scheduler.max_running_requests:
+            return None
+        by_id = {rid: i for i, rid in enumerate(produced)}
+        order = [by_id[rid] for rid in running]
+        for i in order:
+            request = scheduler.get_request(produced[i])
+            if indices[i] + 1 >= request.max_new_tokens:
+                return None
+        tokens = chosen
+        if order != list(range(len(order))):
+            tokens = chosen[torch.tensor(order, dtype=torch.int64, device=chosen.device)]
+        launched = self.runner.launch_decode(running, tokens)
+        if launched is None:
+            return None
+        try:
+            ahead = _TokensOnTheWay(
+                self.sampler.sample(launched.logits, [params[i] for i in order], [indices[i] + 1 for i in order])
+            )
+        except BaseException:
+            self.runner.abort(launched)
+            raise
+        return _LaunchedAhead(tuple(running), launched, ahead)
+
+    def _take_ahead(self, batch: SchedulerBatch) -> Optional[_LaunchedAhead]:
+        """The step launched ahead if `batch` is that step; otherwise it is abandoned."""
+        ahead = self._ahead
+        if ahead is None:
+            return None
+        same = (
+            not batch.admitted_request_ids
+            and all(i.kind is WorkKind.DECODE for i in batch.items)
+            and tuple(i.request_id for i in batch.items) == ahead.request_ids
+        )
+        if not same:
+            self._drop_ahead()
+            return None
+        self._ahead = None
+        self.lookahead_hits += 1
+        return ahead
+
+    def _drop_ahead(self) -> None:
+        if self._ahead is not None:
+            ahead, self._ahead = self._ahead, None
+            self.lookahead_misses += 1
+            self.runner.abort(ahead.output)
 
     def run_until_done(self) -> list[EngineStepResult]:
         """Step until every submitted request has finished."""

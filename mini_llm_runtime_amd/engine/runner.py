@@ -321,6 +321,16 @@ class ModelRunner:
                 out = self.model.forward(ctx, ctx.memo["logit_rows"])
             graph = (captured, static, out, spans, buf.size)
             self._graphs[key] = graph
+        out = self._replay(key, graph, layout, token_ids, None)
+        if logit_rows.size == layout.num_entries and (logit_rows == np.arange(layout.num_entries)).all():
+            return out[: layout.num_entries]
+        if logit_rows.size == 0:
+            return None
+        return out[torch.from_numpy(logit_rows.astype(np.int64)).to(self.device)]
+
+    def _replay(self, key, graph, layout: StepLayout, token_ids: np.ndarray, device_tokens: Optional[torch.Tensor]):
+        """Upload the step's metadata into the graph's static buffer and replay it; token ids
+        come from the host array or, stream-ordered after the upload, from a device tensor."""
         captured, static, out, spans, size = graph
         slot = self._graph_staging(key, spans, size)
         self._fill_padded(slot[1], layout, token_ids)
@@ -329,12 +339,49 @@ class ModelRunner:
             done = slot[2] or torch.cuda.Event()
             done.record(torch.cuda.current_stream(self.device))
             slot[2] = done
+        if device_tokens is not None:
+            start = spans[0][0]
+            static[start : start + layout.num_entries].copy_(device_tokens)
         captured.replay()
-        if logit_rows.size == layout.num_entries and (logit_rows == np.arange(layout.num_entries)).all():
-            return out[: layout.num_entries]
-        if logit_rows.size == 0:
+        return out
+
+    # ---- a decode step launched ahead of its tokens ---------------------------------------------------
+    @torch.inference_mode()
+    def launch_decode(self, request_ids: Sequence[str], device_tokens: torch.Tensor) -> Optional[StepOutput]:
+        """Launch one token per request whose ids are still on the device (the sampler's output
+        of the step before), without waiting for them on the host.  The step's pages are taken
+        but nothing counts until `commit`; `abort` gives them back (whatever the GPU then still
+        writes lands in pages that later steps, ordered behind it on the stream, overwrite).
+        Returns None when such a step cannot replay an already captured graph."""
+        count = len(request_ids)
+        if not self.use_graphs or self.cache.state_banks or not 0 < count <= self.max_graph_batch:
             return None
-        return out[torch.from_numpy(logit_rows.astype(np.int64)).to(self.device)]
+        if device_tokens.shape != (count,) or device_tokens.dtype != torch.int32 or device_tokens.device != self.device:
+            raise ValueError("device_tokens must be int32 [requests] on the runner's device")
+        for rid in request_ids:
+            if self.cache.get_request(rid).num_tokens + 1 > self.max_positions:
+                return None
+        layout = self.cache.begin_step([(rid, 1) for rid in request_ids])
+        try:
+            key = self._graph_key(layout)
+            graph = self._graphs.get(key) if key is not None else None
+            if graph is None:
+                self.cache.abort_step()
+                return None
+            out = self._replay(key, graph, layout, np.zeros(count, dtype=np.int32), device_tokens)
+        except BaseException:
+            self.cache.abort_step()
+            raise
+        return StepOutput(logits=out[:count], rows=tuple((rid, 0) for rid in request_ids), layout=layout)
+
+    def commit(self, launched: StepOutput) -> StepOutput:
+        """Make a step from `launch_decode` count."""
+        launched.passed_pages = self.cache.commit_step()
+        return launched
+
+    def abort(self, launched: StepOutput) -> None:
+        """Give back what a step from `launch_decode` took."""
+        self.cache.abort_step()
 
     # -------------------------------------------------------------------------------------------
     @torch.inference_mode()

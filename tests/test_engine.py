@@ -213,6 +213,59 @@ def test_failed_step_rolls_back_and_can_be_retried(tmp_path, backend, dtype):
     _check_greedy(engine.scheduler.get_request("C").generated_token_ids, pc, w, cfg, dtype)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_decoding_one_step_ahead_changes_nothing_but_the_waiting(tmp_path, dtype):
+    """The engine launches the next decode step before it has seen the last one's tokens.  With
+    requests that end on an end-of-sequence token at different times, late arrivals and few
+    pages, every request's tokens, every batch and every released page must be those of the
+    plain loop; launches are both confirmed and abandoned on the way; no page is lost."""
+    d = make_model_dir(tmp_path, "B", seed=29)
+    cfg, w = read_weights(d)
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    lengths = {"r0": 3, "r1": 9, "r2": 24, "r3": 17, "r4": 30, "r5": 2}
+    arrivals = {"r0": 0, "r1": 0, "r2": 1, "r3": 9, "r4": 9, "r5": 30}
+    prompts = {rid: random_tokens(n, cfg["vocab_size"], 60 + i) for i, (rid, n) in enumerate(lengths.items())}
+
+    def run(lookahead, eos):
+        engine = _engine(d, HipOps(dtype, "cuda"), block_size=BLOCK_SIZE["B"], num_blocks=30, max_running=3,
+                         max_batch_tokens=32, lookahead=lookahead)
+        trace = []
+        step = 0
+        while step < 300:
+            for rid, at in arrivals.items():
+                if at == step:
+                    engine.submit(rid, prompts[rid], max_new_tokens=24, temperature=0.7 if rid == "r1" else 0.0,
+                                  seed=5, eos_token_ids=eos)
+            if not engine.scheduler.has_unfinished_requests and step > max(arrivals.values()):
+                break
+            result = engine.step()
+            step += 1
+            if result is not None:
+                trace.append((tuple((i.request_id, i.kind.value, i.input_token_ids) for i in result.batch.items),
+                              result.update.emitted_tokens, result.update.finished_request_ids, result.released_blocks))
+        assert engine.lookahead_error is None
+        assert engine.manager.request_ids == () and engine.admission.reservations == ()
+        assert not engine.manager.step_in_flight
+        engine.manager.check_invariants()
+        assert engine.manager.groups[0].allocator.free_count == 30
+        tokens = {rid: engine.scheduler.get_request(rid).generated_token_ids for rid in prompts}
+        return tokens, trace, engine
+
+    plain_tokens, _, _ = run(False, None)
+    # end-of-sequence tokens taken from what the requests really generate, so that they end at
+    # different steps, some of them while a launch for the next step is out
+    eos = {plain_tokens["r0"][5], plain_tokens["r2"][11], plain_tokens["r4"][3]}
+    want_tokens, want_trace, off = run(False, eos)
+    got_tokens, got_trace, on = run(True, eos)
+    assert off.lookahead_hits == 0 and off.lookahead_misses == 0
+    assert on.lookahead_hits > 5 and on.lookahead_misses > 0
+    assert got_tokens == want_tokens
+    assert got_trace == want_trace
+    assert any(len(t) < 24 for t in got_tokens.values()), "no request ended on an end-of-sequence token"
+
+
 def test_static_policy_does_not_refill(tmp_path):
     d = make_model_dir(tmp_path, "A", seed=26)
     cfg, _ = read_weights(d)
