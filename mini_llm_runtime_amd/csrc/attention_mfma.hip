@@ -16,8 +16,9 @@
 //    KV head, partition of the keys); the g query heads that share the KV head
 //    are the 16 columns of the MFMA tile, so keys and values are read once per
 //    KV head (the reference's kernel reads them once per query head,
-//    csrc/paged_attention_cuda.cu:44-46).  Four wavefronts take 16-key tiles in
-//    turn and merge through LDS; partitions merge in attn_decode_merge with the
+//    csrc/paged_attention_cuda.cu:44-46).  Four wavefronts take 32-key tiles in
+//    turn, all of a wavefront's loads in flight before it computes, one softmax
+//    update per tile, and merge through LDS; partitions merge in attn_decode_merge with the
 //    reference's rule m = max m_j, O = sum w_j a_j / sum w_j l_j, w_j = exp(m_j - m)
 //    (csrc/paged_attention_split_cuda.cu:66-88).
 //  * attn_prefill: entries with several new tokens (prompt portions), in tiles of
@@ -43,21 +44,6 @@ static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple 
 constexpr int kSteps = (D + 31) / 32;
 constexpr bool kHalfLast = (D % 32) != 0;
 constexpr int kDimTiles = D / 16;
-
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ f32x4_t mfma_16x16x16(s16x4_t a, s16x4_t b, f32x4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
-}
-
-__device__ __forceinline__ s16x4_t pack_bf16x4(float a, float b, float c, float d) {
-  s16x4_t r;
-  r[0] = static_cast<short>(f32_to_bf16(a).bits);
-  r[1] = static_cast<short>(f32_to_bf16(b).bits);
-  r[2] = static_cast<short>(f32_to_bf16(c).bits);
-  r[3] = static_cast<short>(f32_to_bf16(d).bits);
-  return r;
-}
 
 // One row of D dims (a query, or a key) as the operand chunks of the score product.
 struct RowOperand {
@@ -87,96 +73,78 @@ __device__ __forceinline__ f32x4_t score_tile(const RowOperand& k, const RowOper
 // m is the running maximum of score * scale * log2(e).
 struct Softmax {
   float m;
-  float l;  // this lane's share of the sum (its own 4 keys of every tile)
+  float l;  // this lane's share of the sum (its own keys of every tile)
 };
-
-// Fold a tile of 4 scores into the state; returns the probabilities as the B
-// operand of the value product and the factor the accumulator must be scaled by.
-__device__ __forceinline__ s16x4_t softmax_tile(Softmax& st, f32x4_t s, const bool (&ok)[4], float scale2,
-                                                float& alpha) {
-  float tmax = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (!ok[i]) s[i] = -INFINITY;
-    tmax = fmaxf(tmax, s[i]);
-  }
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-  const float m_new = fmaxf(st.m, tmax * scale2);
-  const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-  alpha = fast_exp2(st.m - m_use);
-  float p[4];
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    p[i] = fast_exp2(fmaf(s[i], scale2, -m_use));
-    sum += p[i];
-  }
-  st.l = st.l * alpha + sum;
-  st.m = m_new;
-  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-  const u32x2_t packed = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3])};
-  return __builtin_bit_cast(s16x4_t, packed);
-}
 
 // ---- decode ---------------------------------------------------------------------------------
 constexpr int kDecodeWaves = D > 128 ? 2 : 4;  // bounded by the LDS the merge needs
 constexpr int kPartialStride = D + 2;  // numerator[D], max, denominator
-constexpr int kDecodeDepth = D > 128 ? 2 : 4;  // tiles of a wavefront in flight at once (registers)
+constexpr int kMaxDecodeDepth = D > 128 ? 1 : (D > 64 ? 2 : 4);  // 32-key tiles of a wavefront in flight at once (registers)
 
-// Operands of one 16-key tile, loaded ahead of their use.
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4v_t __attribute__((ext_vector_type(4)));
+
+// Operands of one 32-key tile (two 16-key halves), loaded ahead of their use.
 struct DecodeTile {
-  RowOperand k;
-  s16x4_t v[kDimTiles];
+  RowOperand k[2];
+  u32x2_t v[kDimTiles][2];  // per 16 dims: this lane's 4 keys of each half
   bool bad;
 };
 
+// Where one 32-key tile's operands lie: the page of this lane's key row and of its 4 value
+// keys, per half.  Looked up for ALL of a wavefront's tiles before any operand is loaded, and
+// without branches: the wait for a later tile's table entry would otherwise also wait for
+// every operand load issued before it, one trip to memory after the other.
+struct DecodeTilePages {
+  int key_page[2], value_page[2];
+};
+
+__device__ __forceinline__ DecodeTilePages find_decode_tile(const int* __restrict__ table, int ts, int ke,
+                                                            int block_size, int col, int quarter) {
+  DecodeTilePages p;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    // positions past the end look at the last position's entry instead: always inside the table
+    p.key_page[half] = table[min(ts + half * 16 + col, ke - 1) / block_size];
+    p.value_page[half] = table[min(ts + half * 16 + quarter * 4, ke - 1) / block_size];
+  }
+  return p;
+}
+
+// Loads are unconditional (what is absent reads page 0 instead): a key outside first..ke-1 is
+// masked by its position and its values are cleared there; a missing page inside that range
+// poisons the output.
 __device__ __forceinline__ DecodeTile load_decode_tile(const bf16* __restrict__ key_pages,
                                                        const bf16* __restrict__ value_pages,
-                                                       const int* __restrict__ table, int ts, int ke, int first,
+                                                       const DecodeTilePages& pages, int ts, int ke, int first,
                                                        int kvh, int kv_heads, int block_size, int num_pages,
                                                        int col, int quarter) {
   DecodeTile t;
   t.bad = false;
-  // key operand: this lane's row is key ts + col
-  const int key_a = ts + col;
-  bool valid_a = key_a < ke;
-  const bf16* krow = key_pages;
-  if (valid_a) {
-    const int logical = key_a / block_size;
-    const int page = table[logical];
-    if (page < 0 || page >= num_pages) {
-      t.bad = key_a >= first;
-      valid_a = false;
-    } else {
-      krow = key_pages +
-             ((static_cast<int64_t>(page) * kv_heads + kvh) * block_size + (key_a - logical * block_size)) * D;
-    }
-  }
-  t.k = load_row(krow, valid_a, quarter);
-  // value operand: this lane's 4 keys are ts + quarter * 4 .. + 3, inside one page
-  const int key_v = ts + quarter * 4;
-  bool valid_v = key_v < ke;
-  const bf16* vbase = value_pages;
-  if (valid_v) {
-    const int logical = key_v / block_size;
-    const int page = table[logical];
-    if (page < 0 || page >= num_pages) {
-      valid_v = false;
-    } else {
-      vbase = value_pages + (static_cast<int64_t>(page) * kv_heads + kvh) * D * block_size +
-              (key_v - logical * block_size);
-    }
-  }
 #pragma unroll
-  for (int dt = 0; dt < kDimTiles; ++dt) {
-    t.v[dt] = s16x4_t{0, 0, 0, 0};
-    if (valid_v)
-      t.v[dt] = *reinterpret_cast<const s16x4_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size);
+  for (int half = 0; half < 2; ++half) {
+    // key operand: this lane's row is key ts + half * 16 + col
+    const int key_a = ts + half * 16 + col;
+    const bool here_a = static_cast<unsigned>(pages.key_page[half]) < static_cast<unsigned>(num_pages);
+    t.bad = t.bad || (!here_a && key_a >= first && key_a < ke);
+    const int page_a = here_a ? pages.key_page[half] : 0;
+    const int off_a = min(key_a, ke - 1) % block_size;
+    t.k[half] = load_row(key_pages + ((static_cast<int64_t>(page_a) * kv_heads + kvh) * block_size + off_a) * D,
+                         true, quarter);
+    // value operand: this lane's 4 keys are ts + half * 16 + quarter * 4 .. + 3, inside one page
+    const int key_v = ts + half * 16 + quarter * 4;
+    const bool here_v = static_cast<unsigned>(pages.value_page[half]) < static_cast<unsigned>(num_pages);
+    const int page_v = here_v ? pages.value_page[half] : 0;
+    const int off_v = key_v < ke ? key_v % block_size : 0;
+    const bf16* vbase = value_pages + (static_cast<int64_t>(page_v) * kv_heads + kvh) * D * block_size + off_v;
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt)
+      t.v[dt][half] = *reinterpret_cast<const u32x2_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size);
   }
   return t;
 }
 
+template <int kDecodeDepth>
 __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
@@ -211,6 +179,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int base = (first / 16) * 16;
   const int kb = base + split * part;
   const int ke = min(kb + part, ctx);
+  if (kb >= ke) return;  // a partition past this entry's keys: the merge does not look at it
   const int* table = block_table + static_cast<int64_t>(entry) * table_width;
   if (tid == 0) sm_bad = 0;
   __syncthreads();
@@ -224,42 +193,77 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   bool bad = false;
 
-  // The wavefronts take the partition's 16-key tiles in turn.  A tile's work is far shorter
+  // The wavefronts take the partition's 32-key tiles in turn.  A tile's work is far shorter
   // than a trip to memory, so a wavefront first issues the loads of up to kDecodeDepth of
-  // its tiles (a 256-key partition: all of them) and only then starts on the first.
-  constexpr int kStride = kDecodeWaves * 16;
+  // its tiles (the host picks the depth so that this is all of them whenever registers allow;
+  // tiles past the end would be loaded all the same) and only then starts on the first.
+  // Per tile: scores of both halves, ONE softmax update, one 32-key value product per 16 dims.
+  constexpr int kStride = kDecodeWaves * 32;
   const float scale2 = scale * 1.44269504088896340736f;
-  for (int ts0 = kb + wave * 16; ts0 < ke; ts0 += kDecodeDepth * kStride) {
+  for (int ts0 = kb + wave * 32; ts0 < ke; ts0 += kDecodeDepth * kStride) {
+    DecodeTilePages pages[kDecodeDepth];
+#pragma unroll
+    for (int j = 0; j < kDecodeDepth; ++j)
+      pages[j] = find_decode_tile(table, ts0 + j * kStride, ke, block_size, col, quarter);
     DecodeTile tile[kDecodeDepth];
 #pragma unroll
     for (int j = 0; j < kDecodeDepth; ++j)
-      if (ts0 + j * kStride < ke)
-        tile[j] = load_decode_tile(key_pages, value_pages, table, ts0 + j * kStride, ke, first, kvh, kv_heads,
-                                   block_size, num_pages, col, quarter);
+      tile[j] = load_decode_tile(key_pages, value_pages, pages[j], ts0 + j * kStride, ke, first, kvh, kv_heads,
+                                 block_size, num_pages, col, quarter);
 #pragma unroll
     for (int j = 0; j < kDecodeDepth; ++j) {
       const int ts = ts0 + j * kStride;
       if (ts >= ke) break;
       DecodeTile& cur = tile[j];
       bad = bad || cur.bad;
-      const f32x4_t s = score_tile(cur.k, qo);
-      bool ok[4];
+      f32x4_t sc[2];
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = ts + quarter * 4 + i;
-        ok[i] = key >= first && key < ke;
-        if (!ok[i]) {
+      for (int half = 0; half < 2; ++half) {
+        sc[half] = score_tile(cur.k[half], qo);
 #pragma unroll
-          for (int dt = 0; dt < kDimTiles; ++dt) cur.v[dt][i] = 0;  // unwritten slots may hold NaN
+        for (int i = 0; i < 4; ++i) {
+          const int key = ts + half * 16 + quarter * 4 + i;
+          if (!(key >= first && key < ke)) {
+            sc[half][i] = -INFINITY;
+            // unwritten slots may hold NaN, and 0 * NaN would reach the output
+            const uint32_t keep = (i & 1) ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+            for (int dt = 0; dt < kDimTiles; ++dt) cur.v[dt][half][i / 2] &= keep;
+          }
+          tmax = fmaxf(tmax, sc[half][i]);
         }
       }
-      float alpha;
-      const s16x4_t pb = softmax_tile(sm, s, ok, scale2, alpha);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(sm.m, tmax * scale2);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
+      const float alpha = fast_exp2(sm.m - m_use);
+      float sum = 0.f;
+      float pr[2][4];
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pr[half][i] = fast_exp2(fmaf(sc[half][i], scale2, -m_use));
+          sum += pr[half][i];
+        }
+      sm.l = sm.l * alpha + sum;
+      sm.m = m_new;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+      }
+      // k-slots 0..3 of a lane are its 4 keys of the first half, slots 4..7 those of the second
+      const u32x4v_t pb = {pack_bf16x2(pr[0][0], pr[0][1]), pack_bf16x2(pr[0][2], pr[0][3]),
+                           pack_bf16x2(pr[1][0], pr[1][1]), pack_bf16x2(pr[1][2], pr[1][3])};
+      const bf16x8_t pop = __builtin_bit_cast(bf16x8_t, pb);
 #pragma unroll
       for (int dt = 0; dt < kDimTiles; ++dt) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
-        acc[dt] = mfma_16x16x16(cur.v[dt], pb, acc[dt]);
+        const u32x4v_t va = {cur.v[dt][0][0], cur.v[dt][0][1], cur.v[dt][1][0], cur.v[dt][1][1]};
+        acc[dt] = mfma_16x16x32(__builtin_bit_cast(bf16x8_t, va), pop, acc[dt]);
       }
     }
   }
@@ -316,38 +320,66 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
 // with independent loads.
 __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* __restrict__ partial,
                                                                   const int* __restrict__ cu_q,
-                                                                  bf16* __restrict__ out, int heads, int splits) {
+                                                                  const int* __restrict__ context_lens,
+                                                                  bf16* __restrict__ out, int heads, int window,
+                                                                  int part, int all_splits) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
   const int t = cu_q[entry];
   if (cu_q[entry + 1] - t != 1) return;
-  const float* src = partial + (static_cast<int64_t>(entry) * heads + h) * splits * kPartialStride;
+  const float* src = partial + (static_cast<int64_t>(entry) * heads + h) * all_splits * kPartialStride;
+  // the partitions that hold keys of this entry (the others wrote nothing), as attn_decode cuts them
+  const int ctx = context_lens[entry];
+  const int first = window > 0 ? max(0, ctx - window) : 0;
+  const int splits = min(all_splits, (ctx - (first / 16) * 16 + part - 1) / part);
+  // The numerators are read kMergeBatch partitions at a time, all loads of a batch issued
+  // before the first is used, and the first batch before the reductions below: this kernel's
+  // time is the latency of its loads, so they must not wait for one another.
+  constexpr int kPerLane = (D + kWave - 1) / kWave;
+  constexpr int kMergeBatch = D <= 128 ? 16 : 8;
+  float ms[kMergeBatch], piece[kMergeBatch][kPerLane];
+  auto load_batch = [&](int s0) {
+#pragma unroll
+    for (int u = 0; u < kMergeBatch; ++u) {
+      const int sp = min(s0 + u, splits - 1);
+      ms[u] = src[sp * kPartialStride + D];
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) {
+        const int d = lane + j * kWave;
+        piece[u][j] = d < D ? src[sp * kPartialStride + d] : 0.f;
+      }
+    }
+  };
+  load_batch(0);
+
   float mstar = -INFINITY;
   float den = 0.f;
   // more than 64 partitions: several rounds of the same two reductions
   for (int s0 = 0; s0 < splits; s0 += kWave) {
     const int sp = s0 + lane;
-    const float ms = sp < splits ? src[sp * kPartialStride + D] : -INFINITY;
-    const float ls = sp < splits ? src[sp * kPartialStride + D + 1] : 0.f;
-    const float round_max = wave_max(ms);
+    const float m_sp = sp < splits ? src[sp * kPartialStride + D] : -INFINITY;
+    const float l_sp = sp < splits ? src[sp * kPartialStride + D + 1] : 0.f;
+    const float round_max = wave_max(m_sp);
     const float m_new = fmaxf(mstar, round_max);
-    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - m_new);
+    const float w = (m_sp == -INFINITY) ? 0.f : fast_exp2(m_sp - m_new);
     const float rescale = (mstar == -INFINITY) ? 0.f : fast_exp2(mstar - m_new);
-    den = den * rescale + wave_sum(w * ls);
+    den = den * rescale + wave_sum(w * l_sp);
     mstar = m_new;
   }
-  float num[(D + kWave - 1) / kWave];
+  float num[kPerLane];
 #pragma unroll
-  for (int j = 0; j < (D + kWave - 1) / kWave; ++j) num[j] = 0.f;
-  for (int sp = 0; sp < splits; ++sp) {
-    const float ms = src[sp * kPartialStride + D];
-    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - mstar);
+  for (int j = 0; j < kPerLane; ++j) num[j] = 0.f;
+  for (int s0 = 0;;) {
 #pragma unroll
-    for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
-      const int d = lane + j * kWave;
-      if (d < D) num[j] += w * src[sp * kPartialStride + d];
+    for (int u = 0; u < kMergeBatch; ++u) {
+      const float w = (s0 + u >= splits || ms[u] == -INFINITY) ? 0.f : fast_exp2(ms[u] - mstar);
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) num[j] += w * piece[u][j];
     }
+    s0 += kMergeBatch;
+    if (s0 >= splits) break;
+    load_batch(s0);
   }
 #pragma unroll
   for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
@@ -649,15 +681,34 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   const int head_tiles = (group + 15) / 16;
   MLR_REQUIRE(kv_heads * head_tiles <= 65535, "too many heads for one launch");
   dim3 grid(entries, kv_heads * head_tiles, splits);
-  attn_decode_kernel<<<grid, kDecodeWaves * kWave, 0, stream>>>(
-      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
-      static_cast<const bf16*>(value_pages), block_table, table_width, cu_q, context_lens,
-      static_cast<bf16*>(out), partial, heads, kv_heads, head_tiles, block_size, num_pages, scale, window, part,
-      splits);
+  const bf16* qp = static_cast<const bf16*>(q);
+  const bf16* kp = static_cast<const bf16*>(key_pages);
+  const bf16* vp = static_cast<const bf16*>(value_pages);
+  bf16* op = static_cast<bf16*>(out);
+  const int tiles_per_wave = (part + 32 * kDecodeWaves - 1) / (32 * kDecodeWaves);
+#define MLR_DECODE(depth)                                                                                       \
+  attn_decode_kernel<depth><<<grid, kDecodeWaves * kWave, 0, stream>>>(                                         \
+      qp, q_stride, kp, vp, block_table, table_width, cu_q, context_lens, op, partial, heads, kv_heads,         \
+      head_tiles, block_size, num_pages, scale, window, part, splits)
+  bool launched = false;
+  if constexpr (kMaxDecodeDepth >= 4) {
+    if (tiles_per_wave >= 4) {
+      MLR_DECODE(4);
+      launched = true;
+    }
+  }
+  if constexpr (kMaxDecodeDepth >= 2) {
+    if (!launched && tiles_per_wave >= 2) {
+      MLR_DECODE(2);
+      launched = true;
+    }
+  }
+  if (!launched) MLR_DECODE(1);
+#undef MLR_DECODE
   MLR_LAUNCH_CHECK();
   if (splits > 1) {
-    attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, static_cast<bf16*>(out),
-                                                                         heads, splits);
+    attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(
+        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, part, splits);
     MLR_LAUNCH_CHECK();
   }
   return 0;

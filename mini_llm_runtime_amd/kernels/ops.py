@@ -500,6 +500,8 @@ class HipOps:
             group_tiles = -(-(num_heads // num_kv_heads) // 16)
             base = num_decode * num_kv_heads * group_tiles
             part = max(64, self.decode_partition // 64 * 64)
+            if part > 128 and base * -(-span // part) < 256:
+                part = 128  # few entries: more, smaller partitions so that the compute units fill
             splits = max(1, min(-(-span // part), -(-1024 // base)))
             part = -(-(-(-span // splits)) // 64) * 64
             splits = -(-span // part)
