@@ -390,7 +390,7 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 
 // ---- prefill ----------------------------------------------------------------------------------
 constexpr int kTileQ = 64;                 // queries per workgroup (16 per wavefront)
-constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounded by LDS)
+constexpr int kTileK = D > 192 ? 32 : (D > 64 ? 64 : 128);  // key positions per LDS tile (bounded by LDS)
 constexpr int kSubTiles = kTileK / 16;
 constexpr int kPairs = kSubTiles / 2;      // the value product takes 32 key positions per MFMA
 constexpr int kKLd = D + 8;                // padded key row in LDS (elements)
@@ -409,7 +409,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
-    bf16* __restrict__ out, int heads, int kv_heads, int bs_shift, int num_pages, float scale, int window) {
+    bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
+    int window) {
   // two buffers of (key tile, value tile), then a flag; offsets from one array keep LDS addressing
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   bf16* const lds = reinterpret_cast<bf16*>(prefill_lds);
@@ -417,9 +418,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   int& sm_bad = *reinterpret_cast<int*>(prefill_lds + 2 * kBuffer * 2);
 
   const int block_size = 1 << bs_shift;
-  const int entry = tiles[2 * blockIdx.x];
-  const int q0 = tiles[2 * blockIdx.x + 1];
-  const int head = blockIdx.y;
+  // Workgroup -> (tile, head).  The tile list comes heaviest first (a tile late in a long
+  // prompt has many key tiles before it, an early one few), and all heads of a tile weigh the
+  // same.  Workgroups are handed out round-robin, 256 to a round of the compute units, and
+  // usually all are resident at once: even rounds take work from the heavy end of the list,
+  // odd rounds from the light end, so that a compute unit's workgroups add up alike.
+  const int total = num_tiles * heads;
+  const int round = blockIdx.x / 256, in_round = blockIdx.x % 256;
+  const int work = (round & 1) == 0 ? (round / 2) * 256 + in_round : total - 1 - ((round / 2) * 256 + in_round);
+  const int tile = work / heads;
+  const int head = work - tile * heads;
+  const int entry = tiles[2 * tile];
+  const int q0 = tiles[2 * tile + 1];
   const int kvh = head / (heads / kv_heads);
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
@@ -732,7 +742,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
                   reinterpret_cast<uintptr_t>(value_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
               "operands must be 16-byte aligned");
   MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0, "bad scale or window");
-  MLR_REQUIRE(heads <= 65535, "too many heads for one launch");
+  MLR_REQUIRE(static_cast<int64_t>(num_tiles) * heads < (1ll << 31), "too many tiles for one launch");
   static bool configured = false;
   if (!configured) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel),
@@ -743,10 +753,10 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
     }
     configured = true;
   }
-  attn_prefill_kernel<<<dim3(num_tiles, heads), 256, kPrefillLds, stream>>>(
+  attn_prefill_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256, kPrefillLds, stream>>>(
       static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
       static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,
-      static_cast<bf16*>(out), heads, kv_heads, bs_shift, num_pages, scale, window);
+      static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -22,10 +22,9 @@ import torch
 
 from ..cache.manager import CacheManager, StepLayout
 from ..cache.spec import PagedKVSpec, SlotStateSpec
-from ..parts.context import KVView, StateView, StepContext
+from ..parts.context import QUERY_TILE, KVView, StateView, StepContext, query_tiles
 from ..parts.model import DecoderModel
 
-QUERY_TILE = 64  # queries per tile of the attention plan
 
 
 @dataclass(frozen=True)
@@ -210,8 +209,8 @@ class ModelRunner:
 
     def _forward_eager(self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray) -> Optional[torch.Tensor]:
         single = layout.q_lens == 1
-        tiles = [(r, q0) for r, n in enumerate(layout.q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
-        tile_array = np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+        tile_array = query_tiles(layout.q_lens, layout.q_starts)
+        tiles = tile_array
         host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, tile_array))
         dev = host.to(self.device, non_blocking=True)
         ctx = self._context(

@@ -60,15 +60,7 @@ _SIGNATURES = {
     ),
 }
 
-QUERY_TILE = 64  # queries per workgroup of the prefill attention kernel
-
-
-def query_tiles(q_lens) -> "np.ndarray":
-    """[num_tiles, 2] int32 (entry, first query) covering every entry with more than one new token."""
-    import numpy as np
-
-    tiles = [(r, q0) for r, n in enumerate(q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
-    return np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+from ..parts.context import QUERY_TILE, query_tiles  # noqa: F401  (the plan the prefill kernel runs)
 
 
 class KernelError(RuntimeError):

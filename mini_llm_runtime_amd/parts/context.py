@@ -8,7 +8,21 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Optional
 
+import numpy as np
 import torch
+
+QUERY_TILE = 64  # queries of one request that a mixer's prompt kernel takes together
+
+
+def query_tiles(q_lens, q_starts=None) -> np.ndarray:
+    """[num_tiles, 2] int32 (entry, first query) covering every entry with more than one new
+    token, the tiles with the most keys before them first: a kernel that hands them to the
+    compute units in that order can start the heavy ones early and pair them with light ones."""
+    tiles = [(r, q0) for r, n in enumerate(q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
+    if q_starts is None:
+        q_starts = [0] * len(q_lens)
+    tiles.sort(key=lambda t: -(int(q_starts[t[0]]) + t[1]))
+    return np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
 
 
 @dataclass
