@@ -511,12 +511,23 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   // that the tile loop stays free of branches.  Keys read that way need no clearing: their
   // scores are masked by position.  Values are cleared, since 0 * NaN would reach the output;
   // that can only happen in the last tile and under a window, whose early pages may be gone.
-  auto fetch = [&](int kt0, TileInFlight& t) {
-    const int lim = k_end - kt0;  // positions of this tile that exist
+  // The page ids of a tile are looked up one tile ahead of its loads (two ahead of its use):
+  // a lookup right before the loads that need it would put two trips to memory, one after the
+  // other, into every turn of the loop.
+  int k_ids[kPieces], v_ids[kPieces];
+  auto lookup = [&](int kt0) {
     const int page0 = kt0 >> bs_shift;
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
-      const int page = table[min(page0 + k_page[i], last_page)];
+      k_ids[i] = table[min(page0 + k_page[i], last_page)];
+      v_ids[i] = table[min(page0 + v_page[i], last_page)];
+    }
+  };
+  auto fetch = [&](int kt0, TileInFlight& t) {  // with the ids that lookup(kt0) left
+    const int lim = k_end - kt0;  // positions of this tile that exist
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const int page = k_ids[i];
       const bool in = static_cast<unsigned>(page) < static_cast<unsigned>(num_pages);
       bad = bad || (!in && k_row[i] < lim && kt0 + k_row[i] >= k_begin_raw);
       t.k[i] = load_bf16x8(key_pages + ((in ? page : 0) * page_elems + k_in_page[i]));
@@ -524,7 +535,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bool guard = lim < kTileK || window > 0;  // uniform
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
-      const int page = table[min(page0 + v_page[i], last_page)];
+      const int page = v_ids[i];
       const bool in = static_cast<unsigned>(page) < static_cast<unsigned>(num_pages);
       bf16x8_t val = load_bf16x8(value_pages + ((in ? page : 0) * page_elems + v_in_page[i]));
       if (guard) {
@@ -547,13 +558,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   };
 
   TileInFlight flight;
+  lookup(k_begin);
   fetch(k_begin, flight);
+  lookup(k_begin + kTileK);
   stash(flight, 0);
   __syncthreads();
   int buf = 0;
   for (int kt0 = k_begin; kt0 < k_end; kt0 += kTileK, buf ^= 1) {
     const bool more = kt0 + kTileK < k_end;
-    if (more) fetch(kt0 + kTileK, flight);  // in flight while this tile is computed
+    if (more) {
+      fetch(kt0 + kTileK, flight);  // in flight while this tile is computed
+      lookup(kt0 + 2 * kTileK);
+    }
     const bf16* ks = lds + buf * kBuffer;
     const bf16* vs = ks + kTileK * kKLd;
 
