@@ -390,14 +390,16 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 
 // ---- prefill ----------------------------------------------------------------------------------
 constexpr int kTileQ = 64;                 // queries per workgroup (16 per wavefront)
-constexpr int kTileK = D > 192 ? 32 : (D > 64 ? 64 : 128);  // key positions per LDS tile (bounded by LDS)
+constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounded by LDS)
+constexpr int kKeyGroups = D <= 64 ? 2 : 1;  // wavefront groups of a workgroup that take key tiles in turn (registers allow
+                                            // two resident groups per SIMD only for the small head sizes)
 constexpr int kSubTiles = kTileK / 16;
 constexpr int kPairs = kSubTiles / 2;      // the value product takes 32 key positions per MFMA
 constexpr int kKLd = D + 8;                // padded key row in LDS (elements)
 constexpr int kVLd = kTileK + 8;
 constexpr int kPieces = (kTileK * (D / 8) + 255) / 256;  // 16-byte pieces per thread, of the key and of the value tile
 constexpr int kNoPiece = 0x3fffffff;                      // position of a piece that a thread does not have
-constexpr int kPrefillLds = 2 * (kTileK * kKLd + D * kVLd) * 2 + 16;  // bytes: two buffers and a flag
+constexpr int kPrefillLds = 2 * kKeyGroups * (kTileK * kKLd + D * kVLd) * 2 + 16;  // bytes: two buffers per group, a flag
 
 // One key/value tile on its way from the pages to LDS.
 struct TileInFlight {
@@ -405,17 +407,22 @@ struct TileInFlight {
   bf16x8_t v[kPieces];
 };
 
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+__global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
     int window) {
-  // two buffers of (key tile, value tile), then a flag; offsets from one array keep LDS addressing
+  // Two groups of four wavefronts work on the same 64 queries; group g takes the key tiles
+  // g, g + 2, g + 4, ... and the groups' states are merged at the end.  The heaviest tiles (the
+  // end of a long prompt) bound the kernel's time by their chain of key tiles, one after the
+  // other; this halves the chain and doubles the wavefronts that hide each other's latencies.
+  // LDS: per group two buffers of (key tile, value tile), then a flag; offsets from one array
+  // keep LDS addressing.
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   bf16* const lds = reinterpret_cast<bf16*>(prefill_lds);
   constexpr int kBuffer = kTileK * kKLd + D * kVLd;  // elements
-  int& sm_bad = *reinterpret_cast<int*>(prefill_lds + 2 * kBuffer * 2);
+  int& sm_bad = *reinterpret_cast<int*>(prefill_lds + 2 * kKeyGroups * kBuffer * 2);
 
   const int block_size = 1 << bs_shift;
   // Workgroup -> (tile, head).  The tile list comes heaviest first (a tile late in a long
@@ -431,9 +438,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int entry = tiles[2 * tile];
   const int q0 = tiles[2 * tile + 1];
   const int kvh = head / (heads / kv_heads);
-  const int tid = threadIdx.x;
+  const int group = threadIdx.x / 256;  // key group
+  const int tid = threadIdx.x % 256;    // thread within the group
   const int lane = tid % kWave;
-  const int wave = tid / kWave;
+  const int wave = tid / kWave;  // which 16 queries
   const int col = lane % 16;
   const int quarter = lane / 16;
 
@@ -442,7 +450,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int ctx = context_lens[entry];
   const int pos0 = ctx - q_len;  // position of the entry's first new token
   const int* table = block_table + static_cast<int64_t>(entry) * table_width;
-  if (tid == 0) sm_bad = 0;
+  if (threadIdx.x == 0) sm_bad = 0;
 
   // this lane's query (a column of S^T)
   const int qi = q0 + wave * 16 + col;
@@ -552,28 +560,33 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < kPieces; ++i)
       if (k_row[i] != kNoPiece) {
-        *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + k_lds[i]) = t.k[i];
-        *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + v_lds[i]) = t.v[i];
+        *reinterpret_cast<bf16x8_t*>(lds + (buf * kKeyGroups + group) * kBuffer + k_lds[i]) = t.k[i];
+        *reinterpret_cast<bf16x8_t*>(lds + (buf * kKeyGroups + group) * kBuffer + v_lds[i]) = t.v[i];
       }
   };
 
   TileInFlight flight;
-  lookup(k_begin);
-  fetch(k_begin, flight);
-  lookup(k_begin + kTileK);
-  stash(flight, 0);
+  constexpr int kStep = kKeyGroups * kTileK;  // keys per turn of the loop, all groups together
+  const int k_mine = k_begin + group * kTileK;  // this group's first tile
+  if (k_mine < k_end) {
+    lookup(k_mine);
+    fetch(k_mine, flight);
+    lookup(k_mine + kStep);
+    stash(flight, 0);
+  }
   __syncthreads();
   int buf = 0;
-  for (int kt0 = k_begin; kt0 < k_end; kt0 += kTileK, buf ^= 1) {
-    const bool more = kt0 + kTileK < k_end;
+  for (int kt0 = k_mine; kt0 - group * kTileK < k_end; kt0 += kStep, buf ^= 1) {  // as many turns for every group
+    const bool mine = kt0 < k_end;
+    const bool more = kt0 + kStep < k_end;
     if (more) {
-      fetch(kt0 + kTileK, flight);  // in flight while this tile is computed
-      lookup(kt0 + 2 * kTileK);
+      fetch(kt0 + kStep, flight);  // in flight while this tile is computed
+      lookup(kt0 + 2 * kStep);
     }
-    const bf16* ks = lds + buf * kBuffer;
+    const bf16* ks = lds + (buf * kKeyGroups + group) * kBuffer;
     const bf16* vs = ks + kTileK * kKLd;
 
-    if (wave_has_queries && kt0 <= w_last && kt0 + kTileK - 1 >= w_first) {
+    if (mine && wave_has_queries && kt0 <= w_last && kt0 + kTileK - 1 >= w_first) {
       // Scores of the whole tile, then ONE softmax update for its kTileK positions.  The
       // vector ALU, not the matrix core, bounds this loop (a wavefront instruction takes four
       // cycles, an exponential sixteen), so every per-score operation counts: the scale is
@@ -648,8 +661,30 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     __syncthreads();
   }
 
+  // merge the key groups: the second hands its state over through LDS (the tiles are done with)
+  float* const handover = reinterpret_cast<float*>(prefill_lds);  // [component][thread of the group]
+  if (kKeyGroups > 1 && group == 1) {
+    handover[tid] = m_run;
+    handover[256 + tid] = l_run;
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) handover[(2 + dt * 4 + i) * 256 + tid] = acc[dt][i];
+  }
   if (bad) atomicOr(&sm_bad, 1);
   __syncthreads();
+  if (group != 0) return;
+  if constexpr (kKeyGroups > 1) {
+    const float m_other = handover[tid];
+    const float m_new = fmaxf(m_run, m_other);
+    const float w_mine = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);
+    const float w_other = (m_other == -INFINITY) ? 0.f : fast_exp2(m_other - m_new);
+    l_run = l_run * w_mine + handover[256 + tid] * w_other;
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[dt][i] = acc[dt][i] * w_mine + handover[(2 + dt * 4 + i) * 256 + tid] * w_other;
+  }
   const bool poisoned = sm_bad != 0;
   l_run += __shfl_xor(l_run, 16, kWave);
   l_run += __shfl_xor(l_run, 32, kWave);
@@ -769,7 +804,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
     }
     configured = true;
   }
-  attn_prefill_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256, kPrefillLds, stream>>>(
+  attn_prefill_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256 * kKeyGroups, kPrefillLds, stream>>>(
       static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
       static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,
       static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);
