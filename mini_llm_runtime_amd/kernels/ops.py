@@ -124,6 +124,11 @@ class HipOps:
 
     # ---- helpers --------------------------------------------------------------------------
     def _stream(self) -> _VP:
+        """The HIP stream torch currently runs on for this device (a capture stream inside a
+        graph capture); asked for at every launch, so by the cheapest route torch offers."""
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        if raw is not None:
+            return _VP(raw(self.device.index))
         return _VP(torch.cuda.current_stream(self.device).cuda_stream)
 
     def _call(self, name: str, *args: Any, lib: Optional[ctypes.CDLL] = None) -> None:
@@ -139,19 +144,27 @@ class HipOps:
         dtype: Optional[Union[torch.dtype, Sequence[torch.dtype]]] = None,
         shape: Optional[Sequence[Optional[int]]] = None,
     ) -> torch.Tensor:
+        # runs several times per kernel launch: the passing case takes the short way
         if not isinstance(t, torch.Tensor):
             raise KernelError(f"{name} must be a tensor")
         if t.device != self.device:
             raise KernelError(f"{name} is on {t.device}, the kernels run on {self.device}")
         if not t.is_contiguous():
             raise KernelError(f"{name} must be contiguous")
-        if dtype is not None:
+        if dtype is not None and t.dtype is not dtype:
             allowed = (dtype,) if isinstance(dtype, torch.dtype) else tuple(dtype)
             if t.dtype not in allowed:
                 raise KernelError(f"{name} has dtype {t.dtype}, expected {' or '.join(map(str, allowed))}")
         if shape is not None:
-            if t.dim() != len(shape) or any(s is not None and s != d for s, d in zip(shape, t.shape)):
-                raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+            actual = t.shape
+            ok = len(actual) == len(shape)
+            if ok:
+                for want, have in zip(shape, actual):
+                    if want is not None and want != have:
+                        ok = False
+                        break
+            if not ok:
+                raise KernelError(f"{name} has shape {tuple(actual)}, expected {tuple(shape)}")
         return t
 
     @staticmethod
