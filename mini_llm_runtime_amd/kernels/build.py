@@ -68,7 +68,7 @@ CORE = Module(
 )
 
 
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
 
 
 def attention_module(head_dim: int) -> Module:

@@ -536,11 +536,14 @@ def test_decode_attention_partitions(ops_for, heads, kv_heads, head_dim, partiti
     torch.testing.assert_close(got.double(), fma.double(), **_tol(torch.bfloat16))
 
 
-def test_prefill_attention_long_prompt_and_portion(ops_for):
-    """The tiled prefill kernel on a 2,048-token prompt and on a 300-token portion behind 1,500 cached tokens."""
+@pytest.mark.parametrize("heads,kv_heads,head_dim,bs,long", [
+    (14, 2, 64, 16, 2048), (8, 2, 128, 16, 1100), (3, 1, 96, 8, 700), (2, 1, 256, 32, 600), (5, 5, 16, 64, 900),
+])
+def test_prefill_attention_long_prompt_and_portion(ops_for, heads, kv_heads, head_dim, bs, long):
+    """The tiled prefill kernel on a long prompt (many key tiles, both key groups, tiles handed out
+    heavy first) and on a 300-token portion behind cached tokens, at several head and page sizes."""
     ops = ops_for(torch.bfloat16)
-    heads, kv_heads, head_dim, bs = 14, 2, 64, 16
-    entries = [(2048, 2048), (1800, 300), (77, 77)]
+    entries = [(long, long), (long - 250, 300), (77, 77)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 27, spike=True)
     scale = head_dim**-0.5
     got = ops.paged_attention(
