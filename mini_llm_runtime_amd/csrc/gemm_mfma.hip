@@ -498,8 +498,17 @@ extern "C" {
 int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
   if (k % 8 != 0) return 1;
   if (m > 64 && tiles_128(m, n) >= 256) return 1;
-  const int groups = m <= 16 ? (n + 15) / 16 : tiles_64(m, n);
-  return choose_slices(groups, (k / 8 + 3) / 4, m > 64 ? min(max_slices, 4) : max_slices);
+  if (m <= 16) {
+    // Measured with the norm kernel that adds the slices up (its cost grows with their number):
+    // a weight of 64 MB or more streams fastest through the LDS-tiled kernel cut into 8 slices;
+    // smaller ones through the 16-feature kernel, cut until the compute units are filled and at
+    // least once per 2,560 of k (up to 4 times).
+    const int64_t bytes = static_cast<int64_t>(n) * k * 2;
+    if (bytes >= (64ll << 20) && max_slices >= 8 && k >= 8 * 256 && few_tokens_tiled(n, 8)) return 8;
+    const int by_fill = choose_slices((n + 15) / 16, (k / 8 + 3) / 4, max_slices);
+    return max(by_fill, min(min(4, max_slices), k / 2560));
+  }
+  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, m > 64 ? min(max_slices, 4) : max_slices);
 }
 
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
