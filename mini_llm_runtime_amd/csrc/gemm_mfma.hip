@@ -328,8 +328,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
   for (int it = 0; it < PIECES; ++it) {
     const int idx = tid + it * 256;
-    const int row = idx / 8;
-    const int ch = idx % 8;
+    const int row = idx / (kBK / 8);
+    const int ch = idx % (kBK / 8);
     piece_off[it] = static_cast<unsigned>(row < BN ? row : row - BN) * K * 2u + ch * 16u;
     lds_off[it] = row * kLd + ch * 8;
     piece_chunk[it] = ch;
@@ -353,7 +353,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) {
       const unsigned off = piece_chunk[it] < left ? piece_off[it] + slice * (kBK * 2u) : kOutOfBuffer;
-      reg[it] = buffer_load_bf16x8(it * 256 / 8 < BN ? w_buf : x_buf, off);
+      reg[it] = buffer_load_bf16x8(it * 256 / (kBK / 8) < BN ? w_buf : x_buf, off);
     }
     // the loads are issued here, ahead of the products: the instruction scheduler would
     // otherwise move them down next to the LDS stores that consume them
