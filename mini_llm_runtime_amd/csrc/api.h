@@ -73,7 +73,7 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                   int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k, hipStream_t stream);
 
-// The query/key/value product of up to 16 tokens fused with bias, rotation (cos, sin:
+// The query/key/value product of up to 64 tokens fused with bias, rotation (cos, sin:
 // [m, head_dim / 2] float32, or null), the queries' store to q_out [m, heads * head_dim] and
 // the keys' and values' store into their cache slots (`write` 0: no cache write).
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,

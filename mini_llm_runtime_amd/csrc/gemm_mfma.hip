@@ -132,13 +132,62 @@ struct QkvTarget {
 // AND their partners j + head_dim/2 .. (src/mini_llm_runtime/qwen_model_runner.py:56-61 pairs
 // dim j with j + head_dim/2), so the rotation happens on the sums before anything is stored:
 // queries go to q_out, keys and values straight into their pages (:105-109).
-template <int WAVES, bool QKV>
+// Rotation and stores of the fused query/key/value product for one token: the lane holds the
+// sums of four consecutive dims d0..d0+3 of `head`; lanes q and q ^ 2 of a token hold the two
+// halves of the same rotation pairs.  Called by all lanes (it shuffles); `live` guards the stores.
+__device__ __forceinline__ void qkv_finish(const GemmEpilogue& ep, const QkvTarget& qkv, int head, int block_in_head,
+                                           bool rotated, int d0, int q, int token, bool live, float (&v)[4]) {
+  const int D = qkv.head_dim;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (ep.bias != nullptr) v[i] += load_as_f32(ep.bias, head * D + d0 + i, ep.bias_is_f32);
+    v[i] = to_f32(f32_to_bf16(v[i]));  // the product as bfloat16, as the unfused kernels hand it on
+  }
+  if (rotated) {
+    const int half = D / 2;
+    const int j0 = block_in_head * 8 + (q & 1) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float partner = __shfl_xor(v[i], 32, kWave);
+      const float c = qkv.cos[static_cast<int64_t>(token) * half + j0 + i];
+      const float sn = qkv.sin[static_cast<int64_t>(token) * half + j0 + i];
+      v[i] = q < 2 ? v[i] * c - partner * sn : v[i] * c + partner * sn;
+    }
+  }
+  if (!live) return;
+  u16x4_t packed;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(v[i]).bits;
+  if (head < qkv.heads) {
+    *reinterpret_cast<u16x4_t*>(qkv.q_out + (static_cast<int64_t>(token) * qkv.heads + head) * D + d0) = packed;
+    return;
+  }
+  if (qkv.slots == nullptr) return;
+  const int slot = qkv.slots[token];
+  if (slot < 0) return;
+  const int page = slot / qkv.block_size;
+  const int off = slot - page * qkv.block_size;
+  if (page >= qkv.num_pages) return;
+  if (head < qkv.heads + qkv.kv_heads) {
+    const int kvh = head - qkv.heads;
+    bf16* dst = qkv.key_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * qkv.block_size + off) * D + d0;
+    *reinterpret_cast<u16x4_t*>(dst) = packed;
+  } else {
+    const int kvh = head - qkv.heads - qkv.kv_heads;
+    bf16* dst = qkv.value_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * D + d0) * qkv.block_size + off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[static_cast<int64_t>(i) * qkv.block_size].bits = packed[i];
+  }
+}
+
+// MT: slabs of 16 tokens a workgroup multiplies its weight rows with (1 for the plain product).
+template <int WAVES, bool QKV, int MT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf16* __restrict__ x,
                                                                        const bf16* __restrict__ w,
                                                                        GemmEpilogue ep, QkvTarget qkv, int M, int N,
                                                                        int K) {
-  constexpr int U = 8;  // k-steps in flight per wavefront
-  __shared__ float red[WAVES][kWave][4];
+  constexpr int U = MT > 2 ? 4 : 8;  // k-steps in flight per wavefront
+  __shared__ float red[WAVES][MT][kWave][4];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int r = lane % 16;
@@ -164,12 +213,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
     return head * qkv.head_dim + block_in_head * 8 + (slot < 8 ? slot : qkv.head_dim / 2 + slot - 8);
   };
   const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(row_of(r), N - 1)) * K);
-  const bf16x8_t* xp = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(r, M - 1)) * K);
-  const bool xok = r < M;
-  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t* xp[MT];
+  bool xok[MT];
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    xp[mt] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K);
+    xok[mt] = mt * 16 + r < M;
+    acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
 
   for (int s0 = sb + wave; s0 < se; s0 += WAVES * U) {
-    bf16x8_t a[U], b[U];
+    bf16x8_t a[U], b[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s0 + u * WAVES;
@@ -180,67 +235,34 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
     for (int u = 0; u < U; ++u) {
       const int s = s0 + u * WAVES;
       const int c = s * 4 + q;
-      b[u] = (xok && s < se && c < chunks) ? xp[c] : zero_bf16x8();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = (xok[mt] && s < se && c < chunks) ? xp[mt][c] : zero_bf16x8();
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u) acc = mfma_16x16x32(a[u], b[u], acc);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = mfma_16x16x32(a[u], b[u][mt], acc[mt]);
   }
 
 #pragma unroll
-  for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][mt][lane][i] = acc[mt][i];
   __syncthreads();
   if (wave != 0) return;
-  float v[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] += red[ww][lane][i];
-  if constexpr (!QKV) {
-    finish4(ep, blockIdx.y, slices, r, n0 + q * 4, M, N, v);
-  } else {
-    // the lane holds token r, accumulator rows 4q..4q+3: four consecutive dims of one head
-    const int D = qkv.head_dim;
-    const int d0 = row_of(q * 4) - head * D;
+  for (int mt = 0; mt < MT; ++mt) {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (ep.bias != nullptr) v[i] += load_as_f32(ep.bias, head * D + d0 + i, ep.bias_is_f32);
-      v[i] = to_f32(f32_to_bf16(v[i]));  // the product as bfloat16, as the unfused kernels hand it on
-    }
-    if (rotated) {
-      // lanes q and q ^ 2 of a token hold the two halves of the same pairs
-      const int half = D / 2;
-      const int j0 = block_in_head * 8 + (q & 1) * 4;
-      const int t = min(r, M - 1);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float partner = __shfl_xor(v[i], 32, kWave);
-        const float c = qkv.cos[static_cast<int64_t>(t) * half + j0 + i];
-        const float sn = qkv.sin[static_cast<int64_t>(t) * half + j0 + i];
-        v[i] = q < 2 ? v[i] * c - partner * sn : v[i] * c + partner * sn;
-      }
-    }
-    if (r >= M) return;
-    u16x4_t packed;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(v[i]).bits;
-    if (head < qkv.heads) {
-      *reinterpret_cast<u16x4_t*>(qkv.q_out + (static_cast<int64_t>(r) * qkv.heads + head) * D + d0) = packed;
-      return;
-    }
-    if (qkv.slots == nullptr) return;
-    const int slot = qkv.slots[r];
-    if (slot < 0) return;
-    const int page = slot / qkv.block_size;
-    const int off = slot - page * qkv.block_size;
-    if (page >= qkv.num_pages) return;
-    if (head < qkv.heads + qkv.kv_heads) {
-      const int kvh = head - qkv.heads;
-      bf16* dst = qkv.key_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * qkv.block_size + off) * D + d0;
-      *reinterpret_cast<u16x4_t*>(dst) = packed;
+      for (int i = 0; i < 4; ++i) v[i] += red[ww][mt][lane][i];
+    const int token = mt * 16 + r;
+    if constexpr (!QKV) {
+      finish4(ep, blockIdx.y, slices, token, n0 + q * 4, M, N, v);
     } else {
-      const int kvh = head - qkv.heads - qkv.kv_heads;
-      bf16* dst = qkv.value_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * D + d0) * qkv.block_size + off;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) dst[static_cast<int64_t>(i) * qkv.block_size].bits = packed[i];
+      // the lane holds accumulator rows 4q..4q+3 of its token: four consecutive dims of one head
+      qkv_finish(ep, qkv, head, block_in_head, rotated, row_of(q * 4) - head * qkv.head_dim, q, min(token, M - 1),
+                 token < M, v);
     }
   }
 }
@@ -478,7 +500,7 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
         return -1;
       }
       dim3 grid((n + 15) / 16, slices);
-      gemm_skinny_split_kernel<4, false><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
+      gemm_skinny_split_kernel<4, false, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
       return 0;
     }
     case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
@@ -536,7 +558,7 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   return 0;
 }
 
-// The query/key/value product of up to 16 tokens with everything that follows it before
+// The query/key/value product of up to 64 tokens with everything that follows it before
 // attention: bias, rotation of the query and key heads (cos, sin: [m, head_dim / 2] float32,
 // or null for none), queries to q_out [m, heads * head_dim], keys and values into the slots
 // of their pages (`write` 0: another layer owns the pages).  w is [(heads + 2 kv_heads) *
@@ -546,7 +568,7 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
                             int write, hipStream_t stream) {
   MLR_REQUIRE(x && w && q_out, "null pointer");
-  MLR_REQUIRE(m > 0 && m <= 16, "the fused product takes 1..16 tokens");
+  MLR_REQUIRE(m > 0 && m <= 64, "the fused product takes 1..64 tokens");
   MLR_REQUIRE(k > 0 && k % 8 == 0, "k must be a positive multiple of 8");
   MLR_REQUIRE(heads > 0 && kv_heads > 0 && head_dim >= 16 && head_dim % 16 == 0, "head_dim must be a multiple of 16");
   MLR_REQUIRE((cos == nullptr) == (sin == nullptr), "cos and sin come together");
@@ -560,8 +582,15 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
   GemmEpilogue ep{bias, bias_is_f32, nullptr, 0, 0};
   QkvTarget target{cos, sin, write ? slots : nullptr, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages),
                    static_cast<bf16*>(q_out), heads, kv_heads, head_dim, block_size, num_pages};
-  gemm_skinny_split_kernel<4, true><<<dim3(static_cast<unsigned>(n / 16)), 256, 0, stream>>>(
-      static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, target, m, static_cast<int>(n), k);
+  const dim3 grid(static_cast<unsigned>(n / 16));
+  const bf16* xb = static_cast<const bf16*>(x);
+  const bf16* wb = static_cast<const bf16*>(w);
+  if (m <= 16)
+    gemm_skinny_split_kernel<4, true, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+  else if (m <= 32)
+    gemm_skinny_split_kernel<4, true, 2><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+  else
+    gemm_skinny_split_kernel<4, true, 4><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -381,22 +381,25 @@ class HipOps:
         """Query/key/value product, rotation of queries and keys, keys and values into the cache.
 
         Returns a tensor whose leading num_heads * head_dim columns are the position-encoded
-        queries, for `paged_attention`.  Up to 16 bfloat16 tokens (decoding) run as ONE kernel
+        queries, for `paged_attention`.  Up to 64 bfloat16 tokens (decoding) run as ONE kernel
         that rotates the sums and stores them where they belong; everything else is the product
         followed by `rope_kv_write`.  `fused` forces one of the two ways (tests).
         """
         m, k = x.shape
+        width = (num_heads + 2 * num_kv_heads) * head_dim
         can_fuse = (
             self.dtype == torch.bfloat16
-            and m <= 16
+            and m <= 64
             and k % 8 == 0
             and head_dim % 16 == 0
             and (rotation is None or rotation[2] == head_dim)
         )
         if fused is None:
-            fused = can_fuse
+            # every 16 features' workgroup reads all the tokens: beyond 16 tokens that pays only
+            # while this re-reading stays small beside the caches
+            fused = can_fuse and (m <= 16 or (width // 16) * m * k * 2 <= 32 << 20)
         elif fused and not can_fuse:
-            raise KernelError("the fused query/key/value kernel takes up to 16 bfloat16 tokens and a full rotation")
+            raise KernelError("the fused query/key/value kernel takes up to 64 bfloat16 tokens and a full rotation")
         if not fused:
             qkv = self.linear(x, weight, bias)
             self.rope_kv_write(
@@ -404,7 +407,6 @@ class HipOps:
                 num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size, write=write,
             )
             return qkv
-        width = (num_heads + 2 * num_kv_heads) * head_dim
         self._check(x, "linear input", self.dtype, (None, None))
         self._check(weight, "qkv weight", self.dtype, (width, k))
         if bias is not None:

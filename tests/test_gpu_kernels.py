@@ -291,20 +291,21 @@ def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
 @pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,tokens,rotate,write", [
     (14, 2, 64, 896, 8, True, True), (3, 1, 16, 40, 1, True, True), (6, 3, 48, 104, 16, True, True),
     (4, 4, 80, 72, 5, False, True), (5, 1, 128, 136, 13, True, False),
+    (14, 2, 64, 896, 64, True, True), (3, 1, 32, 104, 17, True, True), (2, 2, 16, 40, 33, True, True),
 ])
 def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write):
     """Decoding runs product, bias, rotation and cache write as one kernel; it has to leave the
     queries and the pages exactly as the product followed by the rotation kernel does, and must
     not touch any slot but the tokens' own (a token without a slot writes nothing)."""
     ops = ops_for(torch.bfloat16)
-    bs, pages = 8, 7
+    bs, pages = 8, 9
     width = (heads + 2 * kv_heads) * head_dim
     x = _rand((tokens, hidden), torch.bfloat16, 71).cuda()
     w = _rand((width, hidden), torch.bfloat16, 72, 0.2).cuda()
     b = _rand((width,), torch.float32, 73).cuda()
     rotation = None
     if rotate:
-        pos = torch.tensor([3, 0, 911, 17, 40000, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15][:tokens], dtype=torch.int32).cuda()
+        pos = torch.tensor(([3, 0, 911, 17, 40000] + list(range(5, 64)))[:tokens], dtype=torch.int32).cuda()
         inv = (1.0 / (1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))).cuda()
         cos, sin = ops.rope_table(pos, inv)
         rotation = (cos, sin, head_dim)
@@ -322,8 +323,15 @@ def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads,
         out[fused] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
     for name, a, c in zip(("queries", "key pages", "value pages"), out[False], out[True]):
         assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
-        # the rotation's two products may be contracted differently: a last-place difference at most
-        torch.testing.assert_close(torch.nan_to_num(c), torch.nan_to_num(a), atol=0, rtol=2 ** -7, msg=lambda m: f"{name}: {m}")
+        if tokens <= 16:
+            # both ways sum the product in the same order; the rotation's two products may be
+            # contracted differently: a last-place difference at most
+            tol = dict(atol=0, rtol=2 ** -7)
+        else:
+            # the unfused product comes from another kernel with another order of summation: sums may
+            # round to neighbouring bfloat16 values, and the rotation subtracts
+            tol = _tol(torch.bfloat16)
+        torch.testing.assert_close(torch.nan_to_num(c), torch.nan_to_num(a), msg=lambda m: f"{name}: {m}", **tol)
     assert torch.isnan(out[True][1]).all() == (not write)
 
 
