@@ -111,6 +111,7 @@ class HipOps:
         self._attention_libs: dict[int, ctypes.CDLL] = {}
         self.decode_partition = int(os.environ.get("MLR_DECODE_PARTITION", "256"))
         self.max_k_slices = int(os.environ.get("MLR_MAX_K_SLICES", "16"))
+        self.decode_max_groups = int(os.environ.get("MLR_DECODE_MAX_GROUPS", "1024"))
 
     def attention_library(self, head_dim: int) -> ctypes.CDLL:
         """The MFMA attention kernels of one head size, compiled on first use."""
@@ -509,7 +510,7 @@ class HipOps:
             part = max(64, self.decode_partition // 64 * 64)
             if part > 128 and base * -(-span // part) < 256:
                 part = 128  # few entries: more, smaller partitions so that the compute units fill
-            splits = max(1, min(-(-span // part), -(-1024 // base)))
+            splits = max(1, min(-(-span // part), -(-self.decode_max_groups // base)))
             part = -(-(-(-span // splits)) // 64) * 64
             splits = -(-span // part)
             partial = None
