@@ -46,14 +46,12 @@ FLAGS = [
     "-mllvm",
     "-amdgpu-mfma-vgpr-form",
 ]
-HEADERS = ["api.h", "common.h", "mfma.h"]
-
-
 @dataclass(frozen=True)
 class Module:
     name: str
     sources: tuple[str, ...]
     defines: tuple[str, ...] = field(default_factory=tuple)
+    headers: tuple[str, ...] = ("api.h", "common.h", "mfma.h")  # what the sources include: part of the stamp
 
 
 CORE = Module(
@@ -75,7 +73,9 @@ def attention_module(head_dim: int) -> Module:
     """The MFMA attention kernels for one head size (a multiple of 16 within 16..256)."""
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise ValueError("the MFMA attention kernels take head sizes in steps of 16 up to 256")
-    return Module(f"attention_d{head_dim}", ("attention_mfma.hip",), (f"MLR_HEAD_DIM={head_dim}",))
+    return Module(
+        f"attention_d{head_dim}", ("attention_mfma.hip",), (f"MLR_HEAD_DIM={head_dim}",), ("common.h", "mfma.h")
+    )
 
 
 def all_modules() -> list[Module]:
@@ -124,7 +124,7 @@ def _source_hash(module: Module) -> str:
     h = hashlib.sha256()
     h.update(" ".join(FLAGS).encode())
     h.update(" ".join(module.defines).encode())
-    for name in list(module.sources) + HEADERS:
+    for name in list(module.sources) + list(module.headers):
         path = CSRC / name
         if path.exists():
             h.update(name.encode())
