@@ -95,6 +95,13 @@ class ModelRunner:
         self.max_graph_batch = int(max_graph_batch)
         self._graphs: dict[tuple[int, int], tuple] = {}
         self._staging: dict[tuple[int, int], list] = {}
+        # Any other step (prompt portions, mixed batches) is recorded when its sizes come a second
+        # time, and replayed from then on, if every part of the model allows it; a bounded number
+        # of such recordings is kept, the least recently used one goes first.
+        self.max_step_graphs = 16
+        self.max_graph_tokens = 8192
+        self._step_graphs: dict[tuple, tuple] = {}
+        self._step_seen: dict[tuple, int] = {}
 
     # -------------------------------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -207,11 +214,11 @@ class ModelRunner:
             host = host.pin_memory()
         return host, spans
 
-    def _forward_eager(self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray) -> Optional[torch.Tensor]:
+    def _forward_eager(
+        self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray, tiles: np.ndarray
+    ) -> Optional[torch.Tensor]:
         single = layout.q_lens == 1
-        tile_array = query_tiles(layout.q_lens, layout.q_starts)
-        tiles = tile_array
-        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, tile_array))
+        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, tiles))
         dev = host.to(self.device, non_blocking=True)
         ctx = self._context(
             dev,
@@ -227,6 +234,84 @@ class ModelRunner:
         )
         return self.model.forward(ctx, ctx.memo["logit_rows"] if logit_rows.size else None)
 
+    # ---- steps of sizes seen before, as HIP graphs ----------------------------------------------------
+    def _table_quantum(self) -> int:
+        return max(1, 1024 // self.cache.block_size)  # table widths in steps of 1,024 tokens
+
+    def _step_key(self, layout: StepLayout, logit_rows: np.ndarray, tiles: np.ndarray) -> Optional[tuple]:
+        """The sizes that fix every launch of a step; None when such steps are not recorded."""
+        if (
+            not self.use_graphs
+            or self.cache.state_banks
+            or not self.model.replayable
+            or layout.num_tokens > self.max_graph_tokens
+        ):
+            return None
+        pages = -(-int(layout.context_lens.max()) // self.cache.block_size)
+        quantum = self._table_quantum()
+        width = -(-pages // quantum) * quantum
+        decodes = int((layout.q_lens == 1).sum())
+        return ("step", layout.num_tokens, layout.num_entries, len(tiles), decodes, width, int(logit_rows.size))
+
+    def _forward_recorded(
+        self, key: tuple, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray, tiles: np.ndarray
+    ) -> Optional[torch.Tensor]:
+        """Replay (recording first, if need be) the graph of a step of these sizes."""
+        width = key[5]
+        span = width * self.cache.block_size
+        arrays = self._arrays(layout, token_ids, logit_rows, tiles)
+        groups = len(layout.block_tables)
+        for g in range(groups):  # block tables as wide as the graph was recorded with
+            table = arrays[len(arrays) - groups + g]
+            wide = np.full((table.shape[0], width), -1, dtype=np.int32)
+            wide[:, : table.shape[1]] = table
+            arrays[len(arrays) - groups + g] = wide
+        graph = self._step_graphs.pop(key, None)
+        if graph is None:
+            buf, spans = _pack_int32(arrays)
+            static = torch.empty(buf.size, dtype=torch.int32, device=self.device)
+            static.copy_(torch.from_numpy(buf))
+            ctx = self._context(
+                static,
+                spans,
+                layout,
+                num_tokens=layout.num_tokens,
+                num_entries=layout.num_entries,
+                max_q_len=layout.num_tokens,
+                max_context_len=span,
+                num_query_tiles=len(tiles),
+                num_decode_entries=key[4],
+                max_decode_context=span if key[4] else 0,
+            )
+            ctx.host = None  # what a recording bakes in must not come from this one step's layout
+            wanted = ctx.memo["logit_rows"] if logit_rows.size else None
+            # one plain run with exactly these launch sizes first: whatever is set up at a
+            # kernel's first use must exist before the recording (the run writes the same cache
+            # entries the replay will write again)
+            self.model.forward(ctx, wanted)
+            torch.cuda.synchronize(self.device)
+            ctx.memo = {"logit_rows": ctx.memo["logit_rows"]}
+            captured = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(captured):
+                out = self.model.forward(ctx, wanted)
+            graph = (captured, static, out, spans, buf.size)
+            while len(self._step_graphs) >= self.max_step_graphs:
+                oldest = next(iter(self._step_graphs))
+                del self._step_graphs[oldest]
+                self._staging.pop(oldest, None)
+        self._step_graphs[key] = graph  # most recently used last
+        captured, static, out, spans, size = graph
+        slot = self._graph_staging(key, spans, size)
+        for view, array in zip(slot[1], arrays):
+            view[...] = array.reshape(view.shape)
+        static.copy_(slot[0], non_blocking=True)
+        if self._pinned:
+            done = slot[2] or torch.cuda.Event()
+            done.record(torch.cuda.current_stream(self.device))
+            slot[2] = done
+        captured.replay()
+        return out
+
     # ---- decode steps as HIP graphs ---------------------------------------------------------------
     def _graph_key(self, layout: StepLayout) -> Optional[tuple[int, int]]:
         """(padded batch, block table width) when the step can replay a captured graph."""
@@ -240,7 +325,7 @@ class ModelRunner:
             padded *= 2
         bs = self.cache.block_size
         pages = -(-int(layout.context_lens.max()) // bs)
-        quantum = max(1, 1024 // bs)  # table widths in steps of 1,024 tokens
+        quantum = self._table_quantum()
         return padded, -(-pages // quantum) * quantum
 
     def _graph_staging(self, key: tuple[int, int], spans, size: int):
@@ -403,7 +488,17 @@ class ModelRunner:
             if key is not None:
                 logits = self._forward_graph(key, layout, token_ids, logit_rows)
             else:
-                logits = self._forward_eager(layout, token_ids, logit_rows)
+                tiles = query_tiles(layout.q_lens, layout.q_starts)
+                step_key = self._step_key(layout, logit_rows, tiles)
+                seen = 0
+                if step_key is not None:
+                    seen = self._step_seen[step_key] = self._step_seen.get(step_key, 0) + 1
+                    if len(self._step_seen) > 4096:
+                        self._step_seen.clear()
+                if seen >= 2:
+                    logits = self._forward_recorded(step_key, layout, token_ids, logit_rows, tiles)
+                else:
+                    logits = self._forward_eager(layout, token_ids, logit_rows, tiles)
         except BaseException:
             self.cache.abort_step()
             raise

@@ -33,6 +33,9 @@ class GQAAttention(Mixer):
     [Wq; Wk; Wv] (made by the weight rules at load time).
     """
 
+    replayable = True
+
+
     def __init__(
         self,
         hidden_size: int,

@@ -17,6 +17,13 @@ from .spec import ParamSpec
 
 
 class Part:
+    # True when `forward` does nothing on the host that depends on the step's DATA (which
+    # requests, their lengths, token values): everything of that kind is read on the device from
+    # the tensors of the `StepContext`, and the host only uses the context's sizes (tokens,
+    # entries, tiles, block table width).  A step of such parts can be recorded as a HIP graph
+    # and replayed for later steps of the same sizes.  Off by default: a part has to say so.
+    replayable = False
+
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}
 

@@ -20,6 +20,9 @@ class PreNormBlock(Block):
     hands its last output to the next block (or the model) un-added.
     """
 
+    replayable = True
+
+
     norm_names = ("input", "post_mixer")
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: Mapping[str, Norm]) -> None:

@@ -22,6 +22,9 @@ class SwiGLU(FeedForward):
     silu(gate) * up is that product's epilogue.
     """
 
+    replayable = True
+
+
     def __init__(self, hidden_size: int, intermediate_size: int) -> None:
         if hidden_size <= 0 or intermediate_size <= 0 or intermediate_size % 2:
             raise ValueError("SwiGLU sizes must be > 0 and the intermediate size even")

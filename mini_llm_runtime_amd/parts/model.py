@@ -72,6 +72,11 @@ class DecoderModel:
         src = self.spec.order[site].reads_cache_of
         return site if src is None else src
 
+    @property
+    def replayable(self) -> bool:
+        """Every part says that its steps can be recorded and replayed (`Part.replayable`)."""
+        return all(part.replayable for _, part in self.named_parts())
+
     def named_parts(self) -> Iterator[tuple[str, Part]]:
         for i, layer in enumerate(self.layers):
             yield from _walk(f"layers.{i}", layer)

@@ -21,6 +21,9 @@ class RMSNorm(Norm):
     rounded once to the engine's dtype.
     """
 
+    replayable = True
+
+
     def __init__(self, size: int, eps: float) -> None:
         if size <= 0 or not eps >= 0:
             raise ValueError("RMSNorm needs size > 0 and eps >= 0")

@@ -24,6 +24,9 @@ class RotaryEmbedding(PositionEncoding):
     encoding's constants.
     """
 
+    replayable = True
+
+
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None) -> None:
         rotary_dim = head_dim if rotary_dim is None else int(rotary_dim)
         if rotary_dim <= 0 or rotary_dim % 2 or rotary_dim > head_dim:
@@ -51,6 +54,9 @@ class RotaryEmbedding(PositionEncoding):
 @register_part("position", "none")
 class NoPosition(PositionEncoding):
     """No position encoding at all (order enters through the causal mask only)."""
+
+    replayable = True
+
 
     def __init__(self, head_dim: int = 0) -> None:
         self.head_dim = head_dim

@@ -197,3 +197,47 @@ def test_long_decoding_graph_replays_match_eager(tmp_path, dtype):
     everything = dict(requests)
     everything["x"] = extra[: max(p for r, p in graph if r == "x") + 1]
     _compare(graph, everything, weights, cfg, dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_recorded_prompt_steps_match_plain_steps(tmp_path, dtype):
+    """Steps whose sizes come again are recorded as graphs and replayed.  The same sequence of
+    prompt portions and mixed batches, with other requests, tokens, lengths and pages each time,
+    must give the logits of the unrecorded runner, replay after replay, with plain steps and
+    synchronisations in between."""
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    d = make_model_dir(tmp_path, "A", seed=31)
+    cfg, _ = read_weights(d)
+    vocab = cfg["vocab_size"]
+    outputs = {}
+    for use_graphs in (False, True):
+        _, _, _, runner = make_runner(d, HipOps(dtype, "cuda"), block_size=BLOCK_SIZE["A"], num_blocks=64, max_requests=4)
+        runner.use_graphs = use_graphs
+        got = []
+        for rnd in range(5):
+            a, b = f"a{rnd}", f"b{rnd}"
+            runner.cache.create_request(a)
+            runner.cache.create_request(b)
+            # a prompt step of 40 tokens, a mixed step (a decodes, b brings 23 tokens), a step of two
+            # portions of changing split (same totals: same sizes, other lengths), two decode steps
+            steps = [
+                [StepEntry.of(a, random_tokens(40, vocab, 100 + rnd), (39,))],
+                [StepEntry.of(a, random_tokens(1, vocab, 200 + rnd), (0,)), StepEntry.of(b, random_tokens(23, vocab, 300 + rnd), (22,))],
+                [StepEntry.of(a, random_tokens(5 + rnd, vocab, 400 + rnd), (0, 4)), StepEntry.of(b, random_tokens(12 - rnd, vocab, 500 + rnd), (3,))],
+                [StepEntry.of(a, random_tokens(1, vocab, 600 + rnd), (0,)), StepEntry.of(b, random_tokens(1, vocab, 700 + rnd), (0,))],
+            ]
+            for entries in steps:
+                out = runner.step(entries)
+                got.append(out.logits.float().cpu())
+                torch.cuda.synchronize()
+            runner.cache.release_request(a)
+            runner.cache.release_request(b)
+        outputs[use_graphs] = got
+        if use_graphs:
+            assert len(runner._step_graphs) >= 3, "the repeated prompt and mixed steps were not recorded"
+        else:
+            assert not runner._step_graphs
+    for i, (want, have) in enumerate(zip(outputs[False], outputs[True])):
+        assert torch.equal(want, have), f"step {i}: a replayed step differs from the plain one"
