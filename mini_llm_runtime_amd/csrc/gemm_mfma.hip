@@ -14,11 +14,12 @@
 //    slice between them (interleaved, so the workgroup reads contiguous spans of
 //    every weight row), keep eight 16-byte loads in flight per lane, and add their
 //    partial sums through LDS.  Activations come straight from L2.
-//  * gemm_tiled: everything else.  An output tile per workgroup (128 x 128 when
-//    there are enough of those to fill the compute units, else 64 x 64), K in
+//  * gemm_tiled: everything else.  An output tile per workgroup (256 x 256 with
+//    sixteen wavefronts for large products, 128 x 128 or 64 x 64 with four, whichever
+//    is the largest that still keeps the compute units busy), K in
 //    slices of 64 staged through double-buffered LDS by range-checked
-//    buffer loads (edge tiles and the tail of K read zeros, no branches), four
-//    wavefronts, 32x32x16 MFMA.  Workgroups are placed so that those resident on
+//    buffer loads (edge tiles and the tail of K read zeros, no branches),
+//    32x32x16 MFMA.  Workgroups are placed so that those resident on
 //    one XCD share operands in its L2.  Up to 16 tokens take this kernel too once
 //    its tiles fill the compute units (it streams a wide weight fastest).
 //    With more than one K slice both kernels write float32 partial sums
@@ -275,13 +276,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
 constexpr int kBK = 64;       // k per LDS slice
 constexpr int kLd = kBK + 8;  // padded LDS row, in elements (144 bytes)
 
-template <int WM, int WN>
+template <int WM, int WN, int GM = 2, int GN = 2>
 struct TiledShape {
-  static constexpr int BM = 64 * WM;
-  static constexpr int BN = 64 * WN;
-  static constexpr int kPieces = (BM + BN) * (kBK / 8) / 256;  // 16-byte pieces per thread and slice
-  static constexpr int kLds = 2 * (BM + BN) * kLd * 2;         // bytes, two buffers
-  static constexpr bool kDeep = WM * WN < 4;                   // loads two slices ahead for the small tiles
+  static constexpr int kThreads = 64 * GM * GN;
+  static constexpr int BM = 32 * WM * GM;
+  static constexpr int BN = 32 * WN * GN;
+  static constexpr int kPieces = (BM + BN) * (kBK / 8) / kThreads;  // 16-byte pieces per thread and slice
+  static constexpr int kLds = 2 * (BM + BN) * kLd * 2;              // bytes, two buffers
+  static constexpr bool kDeep = WM * WN < 4 && GM * GN == 4;        // loads two slices ahead for the small tiles
 };
 
 // Workgroup -> (slice, token tile, feature tile).  Consecutive workgroups go to the eight
@@ -310,11 +312,11 @@ __device__ __forceinline__ void place_workgroup(const TileOrder& order, int id, 
   nt = in_group / size;
 }
 
-template <int WM, int WN, bool DEEP>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+template <int WM, int WN, bool DEEP, int GM = 2, int GN = 2>
+__global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                          GemmEpilogue ep, TileOrder order, int M, int N, int K) {
-  using Shape = TiledShape<WM, WN>;
-  constexpr int BM = Shape::BM, BN = Shape::BN, PIECES = Shape::kPieces;
+  using Shape = TiledShape<WM, WN, GM, GN>;
+  constexpr int BM = Shape::BM, BN = Shape::BN, PIECES = Shape::kPieces, THREADS = Shape::kThreads;
   // Two LDS buffers, each BN rows of w and then BM rows of x.  Addressed as offsets from
   // the one shared array so that every access stays an LDS instruction.
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -324,8 +326,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
   const int wave = tid / kWave;
-  const int wn = wave % 2;
-  const int wm = wave / 2;
+  const int wn = wave % GN;
+  const int wm = wave / GN;
   const int r32 = lane % 32;
   const int h = lane / 32;
   int slice, mt, nt;
@@ -349,7 +351,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
   int piece_chunk[PIECES];
 #pragma unroll
   for (int it = 0; it < PIECES; ++it) {
-    const int idx = tid + it * 256;
+    const int idx = tid + it * THREADS;
     const int row = idx / (kBK / 8);
     const int ch = idx % (kBK / 8);
     piece_off[it] = static_cast<unsigned>(row < BN ? row : row - BN) * K * 2u + ch * 16u;
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) {
       const unsigned off = piece_chunk[it] < left ? piece_off[it] + slice * (kBK * 2u) : kOutOfBuffer;
-      reg[it] = buffer_load_bf16x8(it * 256 / (kBK / 8) < BN ? w_buf : x_buf, off);
+      reg[it] = buffer_load_bf16x8(it * THREADS / (kBK / 8) < BN ? w_buf : x_buf, off);
     }
     // the loads are issued here, ahead of the products: the instruction scheduler would
     // otherwise move them down next to the LDS stores that consume them
@@ -442,13 +444,14 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     }
 }
 
-template <int WM, int WN>
+template <int WM, int WN, int GM = 2, int GN = 2>
 static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
                         hipStream_t stream) {
-  using Shape = TiledShape<WM, WN>;
+  using Shape = TiledShape<WM, WN, GM, GN>;
+  constexpr bool kDeep = Shape::kDeep;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, Shape::kDeep>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, kDeep, GM, GN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLds);
     if (e != hipSuccess) {
       set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
@@ -462,7 +465,8 @@ static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, 
     set_error("mlr_gemm_bf16: too many tiles for one launch");
     return -1;
   }
-  gemm_tiled_kernel<WM, WN, Shape::kDeep><<<dim3(static_cast<unsigned>(groups)), 256, Shape::kLds, stream>>>(xb, wb, ep, order, m, n, k);
+  gemm_tiled_kernel<WM, WN, kDeep, GM, GN><<<dim3(static_cast<unsigned>(groups)), Shape::kThreads, Shape::kLds, stream>>>(
+      xb, wb, ep, order, m, n, k);
   return 0;
 }
 
@@ -478,17 +482,22 @@ static int choose_slices(int groups, int ksteps, int allowed) {
 // Tiles of a shape under the 64 x 64 and the 128 x 128 tiling.
 static int tiles_64(int m, int n) { return ((n + 63) / 64) * ((m + 63) / 64); }
 static int tiles_128(int m, int n) { return ((n + 127) / 128) * ((m + 127) / 128); }
+static int tiles_256(int m, int n) { return ((n + 255) / 256) * ((m + 255) / 256); }
 
 // Up to 16 tokens: the LDS-tiled kernel once its 64-feature tiles (times slices) fill the
 // compute units, the 16-feature streaming kernel below that.
 static bool few_tokens_tiled(int n, int slices) { return ((n + 63) / 64) * slices >= 256; }
 
-// The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 = gemm_tiled with 64 x 64 and
-// 128 x 128 tiles.  The large tile needs less L2 traffic per flop and wins whenever there are
-// enough of them to fill the compute units.
-static int choose_kernel(int m, int n, int slices) {
+// The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,
+// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles.  A larger tile
+// needs less L2 traffic per flop and wins once there are enough of them to keep the compute
+// units busy; the largest one wants K long enough to pay for its prologue, or many tiles.
+static int choose_kernel(int m, int n, int k, int slices) {
   if (m <= 16 && !few_tokens_tiled(n, slices)) return 16;
-  return (m > 64 && slices == 1 && tiles_128(m, n) >= 256) ? 22 : 11;
+  if (m <= 64 || slices > 1) return 11;
+  const int big = tiles_256(m, n);
+  if (big >= 144 && (big >= 512 || k >= 2048)) return 44;
+  return tiles_128(m, n) >= 256 ? 22 : 11;
 }
 
 static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
@@ -505,7 +514,8 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
     }
     case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
     case 22: return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 11 or 22"); return -1;
+    case 44: return launch_tiled<2, 2, 4, 4>(xb, wb, ep, m, n, k, slices, stream);
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 11, 22 or 44"); return -1;
   }
 }
 
@@ -551,7 +561,7 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
               "x and w must be 16-byte aligned");
   GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
-  if (kernel == 0) kernel = choose_kernel(m, n, slices);
+  if (kernel == 0) kernel = choose_kernel(m, n, k, slices);
   if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, kernel, stream) != 0)
     return -1;
   MLR_LAUNCH_CHECK();

@@ -209,13 +209,13 @@ def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     assert torch.equal(picked, got.cpu()[..., [m - 1, 0], :])
 
 
-@pytest.mark.parametrize("kernel", [16, 11, 22])
+@pytest.mark.parametrize("kernel", [16, 11, 22, 44])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
     shorter than an LDS slice, whole and cut along k."""
     ops = ops_for(torch.bfloat16)
-    m, n, k = (13 if kernel == 16 else 150), 203, 1208
+    m, n, k = (13 if kernel == 16 else (300 if kernel == 44 else 150)), (203 if kernel != 44 else 530), 1208
     x = _rand((m, k), torch.bfloat16, 61)
     w = _rand((n, k), torch.bfloat16, 62, 0.05)
     b = _rand((n,), torch.float32, 63)
