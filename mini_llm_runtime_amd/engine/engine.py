@@ -64,11 +64,19 @@ class _TokensOnTheWay:
     stream right behind the sampling, BEFORE any later step is launched, and waited for by
     its own event: waiting for it then does not wait for what was launched after it."""
 
+    _landing: list = []  # pinned host buffers that are not in use (allocating one costs a system call)
+
     def __init__(self, chosen: torch.Tensor) -> None:
         self.device_tokens = chosen
         self._event = None
+        self._buffer = None
         if chosen.device.type == "cuda":
-            self._host = torch.empty(chosen.shape, dtype=chosen.dtype, pin_memory=True)
+            count = chosen.numel()
+            pool = _TokensOnTheWay._landing
+            self._buffer = pool.pop() if pool and pool[-1].numel() >= count else torch.empty(
+                max(256, count), dtype=chosen.dtype, pin_memory=True
+            )
+            self._host = self._buffer[:count]
             self._host.copy_(chosen, non_blocking=True)
             self._event = torch.cuda.Event()
             self._event.record(torch.cuda.current_stream(chosen.device))
@@ -78,7 +86,12 @@ class _TokensOnTheWay:
     def wait(self) -> list[int]:
         if self._event is not None:
             self._event.synchronize()
-        return self._host.tolist()
+        tokens = self._host.tolist()
+        if self._buffer is not None:
+            if len(_TokensOnTheWay._landing) < 8:
+                _TokensOnTheWay._landing.append(self._buffer)
+            self._buffer = None
+        return tokens
 
 
 @dataclass
