@@ -563,6 +563,28 @@ def test_prefill_attention_long_prompt_and_portion(ops_for, heads, kv_heads, hea
     torch.testing.assert_close(got.double(), ref, **_tol(torch.bfloat16))
 
 
+def test_attention_at_a_long_context(ops_for):
+    """A decoded token and a 64-token portion behind some 20,000 cached positions: many partitions
+    and key tiles, table rows of over a thousand pages, and a single far key (position 1) that
+    carries the result, which an index or partition mistake would lose among the thousands."""
+    ops = ops_for(torch.bfloat16)
+    heads, kv_heads, head_dim, bs = 4, 2, 64, 16
+    entries = [(20000, 1), (19000, 64), (33, 33)]
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 41, spike=True)
+    scale = head_dim**-0.5
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
+    ).cpu()
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.double(), ref, **_tol(torch.bfloat16))
+    # the far key really decides: the output is close to its value row
+    v1 = dense[0][1][1]  # values at position 1 of the first entry, [kv_heads, d]
+    want = v1.repeat_interleave(heads // kv_heads, dim=0).reshape(-1)
+    assert torch.allclose(got[0].double(), want, atol=0.1), "the far key did not dominate"
+
+
 # ---- sampling ---------------------------------------------------------------------------------------------
 def test_sample_greedy_first_maximum(ops_for):
     ops = ops_for(torch.float32)
