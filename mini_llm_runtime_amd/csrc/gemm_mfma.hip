@@ -540,7 +540,8 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
     const int by_fill = choose_slices((n + 15) / 16, (k / 8 + 3) / 4, max_slices);
     return max(by_fill, min(min(4, max_slices), k / 2560));
   }
-  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, m > 64 ? min(max_slices, 4) : max_slices);
+  // more slices fill the compute units, but the norm that adds them up reads them all
+  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, m > 64 ? 4 : 8));
 }
 
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
