@@ -91,6 +91,7 @@ class ModelRunner:
         # Steps that hold single tokens only are captured once per (padded batch, table
         # width) as a HIP graph and replayed: a decode step of a small model is hundreds of
         # short kernels, and launching them one by one from the host costs more than running them.
+        # Only for models whose parts all say `replayable`.
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
         self.max_graph_batch = int(max_graph_batch)
         self._graphs: dict[tuple[int, int], tuple] = {}
@@ -315,7 +316,7 @@ class ModelRunner:
     # ---- decode steps as HIP graphs ---------------------------------------------------------------
     def _graph_key(self, layout: StepLayout) -> Optional[tuple[int, int]]:
         """(padded batch, block table width) when the step can replay a captured graph."""
-        if not self.use_graphs or self.cache.state_banks or (layout.q_lens != 1).any():
+        if not self.use_graphs or self.cache.state_banks or not self.model.replayable or (layout.q_lens != 1).any():
             return None
         count = layout.num_entries
         if count > self.max_graph_batch:
@@ -438,7 +439,12 @@ class ModelRunner:
         writes lands in pages that later steps, ordered behind it on the stream, overwrite).
         Returns None when such a step cannot replay an already captured graph."""
         count = len(request_ids)
-        if not self.use_graphs or self.cache.state_banks or not 0 < count <= self.max_graph_batch:
+        if (
+            not self.use_graphs
+            or self.cache.state_banks
+            or not self.model.replayable
+            or not 0 < count <= self.max_graph_batch
+        ):
             return None
         if device_tokens.shape != (count,) or device_tokens.dtype != torch.int32 or device_tokens.device != self.device:
             raise ValueError("device_tokens must be int32 [requests] on the runner's device")

@@ -7,7 +7,8 @@ without a change to the framework's files.
 * an execution order that names a layer twice (two sites, two caches) and lets a
   site read another site's cache;
 * attention layers with a window beside layers without (two page pools);
-* another position encoding (a learned-free additive ramp applied to q and k).
+* another position encoding (a learned-free additive ramp applied to q and k);
+* a feed-forward with routing (a router, the two best of four experts per token).
 
 None of them is a model of anybody's; they only show that the interfaces hold.
 Each is compared with a plain computation written out in this file, whole and in
@@ -33,6 +34,7 @@ from mini_llm_runtime_amd.config.model_config import ModelConfig
 from mini_llm_runtime_amd.engine import ModelRunner, StepEntry
 from mini_llm_runtime_amd.models import register_architecture, unregister_architecture
 from mini_llm_runtime_amd.parts import (
+    FeedForward,
     LayerSpec,
     Mixer,
     ModelSpec,
@@ -99,6 +101,8 @@ class RampPosition(PositionEncoding):
     """q and k get `slope * position` added to their first dim: not a rotation, so the
     attention part has to call `apply` and store k without the fused rotation."""
 
+    replayable = True  # nothing here looks at the step's data on the host
+
     def __init__(self, head_dim: int, slope: float) -> None:
         self.head_dim = head_dim
         self.slope = slope
@@ -107,6 +111,39 @@ class RampPosition(PositionEncoding):
         ramp = (ctx.positions.float() * self.slope)[:, None]
         q[:, :, 0] = (q[:, :, 0].float() + ramp).to(q.dtype)
         k[:, :, 0] = (k[:, :, 0].float() + ramp).to(k.dtype)
+
+
+class RoutedFeedForward(FeedForward):
+    """Each token goes to its `top` best of `experts` small two-matrix networks, by a router
+    whose logits and softmax are 32-bit; the experts' outputs are added with the renormalised
+    router weights.  Which rows an expert gets is decided on the host from the step's data, so
+    the part does not say `replayable`."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int, router_scale: float) -> None:
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.experts, self.top, self.router_scale = experts, top, router_scale
+        self.router_weight = self.up_weight = self.down_weight = None
+
+    def param_specs(self):
+        h, i, e = self.hidden_size, self.intermediate_size, self.experts
+        return {"router_weight": ParamSpec((e, h)), "up_weight": ParamSpec((e * i, h)), "down_weight": ParamSpec((e * h, i))}
+
+    def forward(self, ctx, h):
+        ops = ctx.ops
+        i, width = self.intermediate_size, self.hidden_size
+        logits = ops.linear(h, self.router_weight, None, out_dtype=torch.float32) * self.router_scale
+        weights, chosen = torch.softmax(logits, dim=-1).topk(self.top, dim=-1)
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+        out = torch.zeros(h.shape[0], width, dtype=torch.float32, device=h.device)
+        for e in range(self.experts):
+            rows, slot = (chosen == e).nonzero(as_tuple=True)
+            if rows.numel() == 0:
+                continue
+            inner = ops.linear(h.index_select(0, rows).contiguous(), self.up_weight[e * i : (e + 1) * i], None)
+            inner = torch.nn.functional.silu(inner.float()).to(ctx.dtype)
+            y = ops.linear(inner, self.down_weight[e * width : (e + 1) * width], None, out_dtype=torch.float32)
+            out.index_add_(0, rows, y * weights[rows, slot][:, None])
+        return out.to(ctx.dtype)
 
 
 @dataclass(frozen=True)
@@ -126,18 +163,24 @@ class ToyConfig(ModelConfig):
     window: int = 0
     rope_theta: float = 10000.0
     ramp_slope: float = 0.01
+    ffn_kinds: tuple = ()  # per layer "swiglu" or "routed"; empty: all "swiglu"
+    num_experts: int = 0
+    experts_per_token: int = 0
+    router_scale: float = 1.0
 
     @classmethod
     def from_dict(cls, data: Mapping[str, Any]) -> "ToyConfig":
         names = [f.name for f in fields(cls)]
         kw = {n: data[n] for n in names if n in data}
         kw["layer_kinds"] = tuple(kw["layer_kinds"])
+        kw["ffn_kinds"] = tuple(kw.get("ffn_kinds", ()))
         kw["order"] = tuple(tuple(o) for o in kw["order"])
         return cls(**kw)
 
     def to_dict(self):
         d = super().to_dict()
         d["layer_kinds"] = list(self.layer_kinds)
+        d["ffn_kinds"] = list(self.ffn_kinds)
         d["order"] = [list(o) for o in self.order]
         return d
 
@@ -176,14 +219,26 @@ def toy_spec(c: ToyConfig) -> ModelSpec:
                 WeightRule(p + "attn.v", p + "mixer.qkv_weight", q_rows + kv_rows, kv_rows),
                 WeightRule(p + "attn.o", p + "mixer.o_weight"),
             ]
-        rules += [
-            WeightRule(p + "norm1", p + "norm_input.weight"),
-            WeightRule(p + "norm2", p + "norm_post_mixer.weight"),
-            WeightRule(p + "ffn.gate", p + "feed_forward.gate_up_weight", 0, c.intermediate_size, block=2, period=4),
-            WeightRule(p + "ffn.up", p + "feed_forward.gate_up_weight", 2, c.intermediate_size, block=2, period=4),
-            WeightRule(p + "ffn.down", p + "feed_forward.down_weight"),
-        ]
-        layers.append(LayerSpec("pre_norm", mixer, ffn, {"input": norm, "post_mixer": norm}))
+        rules += [WeightRule(p + "norm1", p + "norm_input.weight"), WeightRule(p + "norm2", p + "norm_post_mixer.weight")]
+        layer_ffn = ffn
+        if c.ffn_kinds and c.ffn_kinds[i] == "routed":
+            layer_ffn = PartSpec(
+                "toy_routed",
+                {"hidden_size": c.hidden_size, "intermediate_size": c.intermediate_size, "experts": c.num_experts,
+                 "top": c.experts_per_token, "router_scale": c.router_scale},
+            )
+            rules += [
+                WeightRule(p + "ffn.router", p + "feed_forward.router_weight"),
+                WeightRule(p + "ffn.experts.up", p + "feed_forward.up_weight"),
+                WeightRule(p + "ffn.experts.down", p + "feed_forward.down_weight"),
+            ]
+        else:
+            rules += [
+                WeightRule(p + "ffn.gate", p + "feed_forward.gate_up_weight", 0, c.intermediate_size, block=2, period=4),
+                WeightRule(p + "ffn.up", p + "feed_forward.gate_up_weight", 2, c.intermediate_size, block=2, period=4),
+                WeightRule(p + "ffn.down", p + "feed_forward.down_weight"),
+            ]
+        layers.append(LayerSpec("pre_norm", mixer, layer_ffn, {"input": norm, "post_mixer": norm}))
     return ModelSpec(
         architecture=c.architecture,
         vocab_size=c.vocab_size,
@@ -202,15 +257,19 @@ def toy_spec(c: ToyConfig) -> ModelSpec:
 def toy_registered():
     register_part("mixer", "toy_running_mean", RunningMeanMixer, replace=True)
     register_part("position", "toy_ramp", RampPosition, replace=True)
+    register_part("feed_forward", "toy_routed", RoutedFeedForward, replace=True)
     register_architecture("ToyForCausalLM", ToyConfig, toy_spec, replace=True)
     yield
     unregister_architecture("ToyForCausalLM")
     unregister_part("mixer", "toy_running_mean")
     unregister_part("position", "toy_ramp")
+    unregister_part("feed_forward", "toy_routed")
 
 
 # ---- the plain computation of the same toy model ------------------------------------------------------
-def toy_plain(tokens, w, c: ToyConfig):
+def toy_plain(tokens, w, c: ToyConfig, gaps=None):
+    """Logits of the whole sequence.  `gaps` collects, per routed layer, each token's router
+    logit gap between its last chosen and its first rejected expert, relative to its largest logit."""
     x = w["embed.weight"].double()[torch.tensor(tokens)]
     n = len(tokens)
     pos = torch.arange(n)
@@ -247,6 +306,22 @@ def toy_plain(tokens, w, c: ToyConfig):
             mixed = att.transpose(0, 1).reshape(n, hq * d) @ w[p + "attn.o"].double().t()
         x = x + mixed
         h = plain.rms_norm(x, w[p + "norm2"].double(), c.rms_norm_eps)
+        if c.ffn_kinds and c.ffn_kinds[layer] == "routed":
+            i, width = c.intermediate_size, c.hidden_size
+            logits = (h @ w[p + "ffn.router"].double().t()) * c.router_scale
+            ordered = logits.sort(dim=-1, descending=True).values
+            if gaps is not None:
+                gaps.append((ordered[:, c.experts_per_token - 1] - ordered[:, c.experts_per_token]) / logits.abs().max(-1).values)
+            weights, chosen = torch.softmax(logits, -1).topk(c.experts_per_token, -1)
+            weights = weights / weights.sum(-1, keepdim=True)
+            y = torch.zeros_like(x)
+            for t in range(n):
+                for weight, e in zip(weights[t], chosen[t]):
+                    up = w[p + "ffn.experts.up"].double()[int(e) * i : (int(e) + 1) * i]
+                    down = w[p + "ffn.experts.down"].double()[int(e) * width : (int(e) + 1) * width]
+                    y[t] += weight * (down @ torch.nn.functional.silu(up @ h[t]))
+            x = x + y
+            continue
         g = h @ w[p + "ffn.gate"].double().t()
         x = x + (g * torch.sigmoid(g) * (h @ w[p + "ffn.up"].double().t())) @ w[p + "ffn.down"].double().t()
     x = plain.rms_norm(x, w["norm.weight"].double(), c.rms_norm_eps)
@@ -332,6 +407,76 @@ def test_toy_model_whole_and_in_portions(tmp_path, toy_registered, name, backend
     if name == "window":  # the window pool gave pages back while the full pool kept them
         a = cache.get_request("a")
         assert a.tables[0][0] == -1 and len(a.live_blocks(0)) < len(a.live_blocks(1))
+    for rid in requests:
+        cache.release_request(rid)
+    assert all(g.allocator.free_count == g.num_blocks for g in cache.groups)
+
+
+ROUTED = dict(
+    layer_kinds=["attention", "attention", "attention"], ffn_kinds=["swiglu", "routed", "swiglu"],
+    order=[[0, -1], [1, -1], [2, -1]], window=0, num_experts=4, experts_per_token=2, router_scale=30.0,
+)
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+def test_toy_routed_feed_forward(tmp_path, toy_registered, backend, dtype):
+    """A feed-forward with a router and experts, defined above, in one of three layers: whole
+    prompts, then portions of two requests in one batch with single tokens at the end.  Random
+    weights can leave a token on the edge between two experts, where bfloat16 may choose the
+    other one; the seed is the first whose routing is clear for every token (32-bit needs none)."""
+    base = dict(
+        architectures=["ToyForCausalLM"], model_type="toy", vocab_size=97, hidden_size=48, intermediate_size=40,
+        num_attention_heads=3, num_key_value_heads=1, head_dim=16, max_position_embeddings=256, rms_norm_eps=1e-5,
+    )
+    base.update(ROUTED)
+    config = mlr.models.config_from_dict(base)
+    requests = {"a": random_tokens(23, 97, 11), "b": random_tokens(11, 97, 12)}
+    for seed in range(20, 120):
+        folder = mlr.write_random_model(config, tmp_path / f"routed{seed}", seed=seed)
+        with SafetensorsFile(folder / "model.safetensors") as f:
+            weights = {n: f.tensor(n) for n in f.entries}
+        gaps: list = []
+        refs = {rid: toy_plain(toks, weights, config, gaps) for rid, toks in requests.items()}
+        if min(float(g.min()) for g in gaps) > 0.06:
+            break
+    else:
+        pytest.fail("no seed with clear routing")
+    assert len(gaps) == 2 and {n for n in weights if "router" in n} == {"layers.1.ffn.router"}
+    ops = _ops(backend, dtype)
+    cfg, model = mlr.load_model(folder, dtype=dtype, device=ops.device)
+    assert not model.replayable  # the routed part plans on the host: its steps are never recorded
+    cache = mlr.make_cache(model, block_size=4, num_blocks=24, max_requests=2)
+    cache.poison()
+    runner = ModelRunner(model, cache, ops)
+
+    def check(got, rid, first):
+        ref = refs[rid][first : first + got.shape[0]]
+        err = (got.double().cpu() - ref).abs().max() / ref.abs().max()
+        assert err < (1e-4 if dtype == torch.float32 else 4e-2), (rid, first, float(err))
+
+    for rid, toks in requests.items():
+        cache.create_request(rid)
+        check(runner.step([StepEntry.of(rid, toks, range(len(toks)))]).logits, rid, 0)
+        cache.release_request(rid)
+    fed = {rid: 0 for rid in requests}
+    for rid in requests:
+        cache.create_request(rid)
+    sizes = [6, 1, 3, 9, 1, 1, 2, 5]
+    i = 0
+    while any(fed[r] < len(requests[r]) for r in requests):
+        entries = []
+        for rid, toks in requests.items():
+            n = min(sizes[(i + 3 * (rid == "b")) % len(sizes)], len(toks) - fed[rid])
+            if n > 0:
+                entries.append(StepEntry.of(rid, toks[fed[rid] : fed[rid] + n], range(n)))
+        out = runner.step(entries)  # the same sizes come again and again: still no recording
+        at = 0
+        for e in entries:
+            check(out.logits[at : at + len(e.tokens)], e.request_id, fed[e.request_id])
+            at += len(e.tokens)
+            fed[e.request_id] += len(e.tokens)
+        i += 1
+    assert not getattr(runner, "_step_graphs", {})
     for rid in requests:
         cache.release_request(rid)
     assert all(g.allocator.free_count == g.num_blocks for g in cache.groups)
