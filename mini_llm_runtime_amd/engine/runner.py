@@ -396,6 +396,7 @@ class ModelRunner:
                 num_query_tiles=0,
                 num_decode_entries=padded,
                 max_decode_context=width * self.cache.block_size,
+                logits_for_all=True,
             )
             # one eager run first: everything that is set up lazily must exist before capture
             self.model.forward(ctx, ctx.memo["logit_rows"])

@@ -72,6 +72,7 @@ class StepContext:
     num_query_tiles: int = 0
     num_decode_entries: int = 0
     max_decode_context: int = 0
+    logits_for_all: bool = False  # the wanted rows are all tokens, in order: no gather needed
     kv_views: dict[int, KVView] = field(default_factory=dict)
     state_views: dict[int, StateView] = field(default_factory=dict)
     memo: dict[Any, Any] = field(default_factory=dict)

@@ -128,8 +128,11 @@ class DecoderModel:
             x, delta = self.layers[entry.layer].forward(ctx, x, delta, site)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
-        rows = ops.gather_rows(x, logit_rows)
-        delta_rows = ops.gather_rows(delta, logit_rows) if delta is not None else None
+        if ctx.logits_for_all:
+            rows, delta_rows = x, delta
+        else:
+            rows = ops.gather_rows(x, logit_rows)
+            delta_rows = ops.gather_rows(delta, logit_rows) if delta is not None else None
         h = self.final_norm.forward(ctx, rows, delta_rows)
         return ops.linear(h, self.head_weight, None, out_dtype=torch.float32)
 
