@@ -274,7 +274,7 @@ class ContinuousBatchEngine:
         generated = {rid: int(tok) for (rid, _), tok in zip(output.rows, host_tokens)}
         with _trace_range(self.enable_tracing, "scheduler.apply_and_release"):
             update = self.scheduler.apply_step_results(generated)
-            if update.finished_request_ids:
+            if self._ahead is not None and set(update.finished_request_ids) & set(self._ahead.request_ids):
                 self._drop_ahead()  # it holds pages of a request that is about to be released
             released = self.admission.release_finished(update.finished_request_ids)
         completed_ns = self._clock_ns()
@@ -292,9 +292,9 @@ class ContinuousBatchEngine:
     # ---- the step launched ahead ----------------------------------------------------------------------
     def _launch_ahead(self, batch, output: StepOutput, chosen, params, indices) -> Optional[_LaunchedAhead]:
         """Launch the next step now if it is bound to be one token for each request of this
-        batch: all running requests produced a token here, none of them ends by length with
-        it, and nobody waits who could be admitted.  (A request may still end on an
-        end-of-sequence token; then the launch is abandoned.)"""
+        batch that goes on: all running requests produced a token here, nobody waits who could
+        be admitted, and those that end by length with this token are left out.  (A request may
+        still end on an end-of-sequence token; then the launch is abandoned.)"""
         scheduler = self.scheduler
         running = scheduler.running_request_ids
         produced = [rid for rid, _ in output.rows]
@@ -303,15 +303,14 @@ class ContinuousBatchEngine:
         if scheduler.waiting_request_ids and len(running) < scheduler.max_running_requests:
             return None
         by_id = {rid: i for i, rid in enumerate(produced)}
-        order = [by_id[rid] for rid in running]
-        for i in order:
-            request = scheduler.get_request(produced[i])
-            if indices[i] + 1 >= request.max_new_tokens:
-                return None
+        going_on = [rid for rid in running if indices[by_id[rid]] + 1 < scheduler.get_request(rid).max_new_tokens]
+        if not going_on:
+            return None
+        order = [by_id[rid] for rid in going_on]
         tokens = chosen
-        if order != list(range(len(order))):
+        if order != list(range(len(produced))):
             tokens = chosen[torch.tensor(order, dtype=torch.int64, device=chosen.device)]
-        launched = self.runner.launch_decode(running, tokens)
+        launched = self.runner.launch_decode(going_on, tokens)
         if launched is None:
             return None
         try:
@@ -321,7 +320,7 @@ class ContinuousBatchEngine:
         except BaseException:
             self.runner.abort(launched)
             raise
-        return _LaunchedAhead(tuple(running), launched, ahead)
+        return _LaunchedAhead(tuple(going_on), launched, ahead)
 
     def _take_ahead(self, batch: SchedulerBatch) -> Optional[_LaunchedAhead]:
         """The step launched ahead if `batch` is that step; otherwise it is abandoned."""
