@@ -22,7 +22,7 @@ import torch
 
 from ..cache.manager import CacheManager, StepLayout
 from ..cache.spec import PagedKVSpec, SlotStateSpec
-from ..parts.context import QUERY_TILE, KVView, StateView, StepContext, query_tiles
+from ..parts.context import KVView, StateView, StepContext, query_tiles
 from ..parts.model import DecoderModel
 
 

@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 import math
-from typing import Mapping, Optional
+from typing import Optional
 
 import torch
 

@@ -27,7 +27,6 @@ import sys
 from pathlib import Path
 from typing import Any, Optional, Sequence, TextIO
 
-import numpy as np
 
 PAGE_TOKENS = 16  # tokens per page of the replay pool
 ROUNDING = 64  # the caller counts every request's tokens rounded up to this

@@ -12,7 +12,7 @@ cut into steps.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Optional, Sequence
+from typing import Any, Sequence
 
 import numpy as np
 import torch

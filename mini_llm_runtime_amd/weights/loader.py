@@ -16,7 +16,7 @@ from __future__ import annotations
 
 import json
 from pathlib import Path
-from typing import Mapping, Union
+from typing import Union
 
 import torch
 

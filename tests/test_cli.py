@@ -9,7 +9,6 @@ import sys
 from pathlib import Path
 
 import pytest
-import torch
 
 import plain_qwen2 as plain
 from helpers import read_weights

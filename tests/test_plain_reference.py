@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import plain_qwen2 as plain
-from helpers import TINY, make_model_dir, random_tokens, read_weights
+from helpers import make_model_dir, random_tokens, read_weights
 
 
 def test_rotate_half_vector():

@@ -12,7 +12,6 @@ from mini_llm_runtime_amd.engine.scheduler import (
     FinishReason,
     RequestScheduler,
     RequestStatus,
-    WorkKind,
 )
 
 

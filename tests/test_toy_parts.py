@@ -18,7 +18,6 @@ portions.
 from __future__ import annotations
 
 import json
-import math
 from dataclasses import dataclass, fields
 from typing import Any, ClassVar, Mapping
 

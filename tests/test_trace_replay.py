@@ -8,7 +8,6 @@ from __future__ import annotations
 import io
 import json
 import subprocess
-import sys
 from pathlib import Path
 
 import numpy as np
