@@ -73,13 +73,14 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                   int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k, hipStream_t stream);
 
-// The query/key/value product of up to 64 tokens fused with bias, rotation (cos, sin:
-// [m, head_dim / 2] float32, or null), the queries' store to q_out [m, heads * head_dim] and
-// the keys' and values' store into their cache slots (`write` 0: no cache write).
+// The query/key/value product fused with bias, rotation (cos, sin: [m, head_dim / 2] float32,
+// or null), the queries' store to q_out [m, heads * head_dim] and the keys' and values' store
+// into their cache slots (`write` 0: no cache write).  kernel: 0 chooses; 16 the row-splitting
+// kernel (up to 64 tokens); 11, 22, 44 the tiled kernels as in mlr_gemm_bf16.
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
                             const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
-                            int write, hipStream_t stream);
+                            int write, int kernel, hipStream_t stream);
 
 // Attention of every token over its request's pages: token t (entry
 // token_entry[t], absolute position positions[t]) sees the keys

@@ -133,6 +133,34 @@ struct QkvTarget {
 // AND their partners j + head_dim/2 .. (src/mini_llm_runtime/qwen_model_runner.py:56-61 pairs
 // dim j with j + head_dim/2), so the rotation happens on the sums before anything is stored:
 // queries go to q_out, keys and values straight into their pages (:105-109).
+// Four consecutive features row0..row0+3 of the fused product of `token` go where they belong:
+// query heads to q_out, key and value heads into the token's cache slot (if it has one).
+__device__ __forceinline__ void qkv_store4(const QkvTarget& qkv, int row0, int token, u16x4_t packed) {
+  const int D = qkv.head_dim;
+  const int head = row0 / D;
+  const int d0 = row0 - head * D;
+  if (head < qkv.heads) {
+    *reinterpret_cast<u16x4_t*>(qkv.q_out + (static_cast<int64_t>(token) * qkv.heads + head) * D + d0) = packed;
+    return;
+  }
+  if (qkv.slots == nullptr) return;
+  const int slot = qkv.slots[token];
+  if (slot < 0) return;
+  const int page = slot / qkv.block_size;
+  const int off = slot - page * qkv.block_size;
+  if (page >= qkv.num_pages) return;
+  if (head < qkv.heads + qkv.kv_heads) {
+    const int kvh = head - qkv.heads;
+    bf16* dst = qkv.key_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * qkv.block_size + off) * D + d0;
+    *reinterpret_cast<u16x4_t*>(dst) = packed;
+  } else {
+    const int kvh = head - qkv.heads - qkv.kv_heads;
+    bf16* dst = qkv.value_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * D + d0) * qkv.block_size + off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[static_cast<int64_t>(i) * qkv.block_size].bits = packed[i];
+  }
+}
+
 // Rotation and stores of the fused query/key/value product for one token: the lane holds the
 // sums of four consecutive dims d0..d0+3 of `head`; lanes q and q ^ 2 of a token hold the two
 // halves of the same rotation pairs.  Called by all lanes (it shuffles); `live` guards the stores.
@@ -159,26 +187,7 @@ __device__ __forceinline__ void qkv_finish(const GemmEpilogue& ep, const QkvTarg
   u16x4_t packed;
 #pragma unroll
   for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(v[i]).bits;
-  if (head < qkv.heads) {
-    *reinterpret_cast<u16x4_t*>(qkv.q_out + (static_cast<int64_t>(token) * qkv.heads + head) * D + d0) = packed;
-    return;
-  }
-  if (qkv.slots == nullptr) return;
-  const int slot = qkv.slots[token];
-  if (slot < 0) return;
-  const int page = slot / qkv.block_size;
-  const int off = slot - page * qkv.block_size;
-  if (page >= qkv.num_pages) return;
-  if (head < qkv.heads + qkv.kv_heads) {
-    const int kvh = head - qkv.heads;
-    bf16* dst = qkv.key_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * qkv.block_size + off) * D + d0;
-    *reinterpret_cast<u16x4_t*>(dst) = packed;
-  } else {
-    const int kvh = head - qkv.heads - qkv.kv_heads;
-    bf16* dst = qkv.value_pages + ((static_cast<int64_t>(page) * qkv.kv_heads + kvh) * D + d0) * qkv.block_size + off;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) dst[static_cast<int64_t>(i) * qkv.block_size].bits = packed[i];
-  }
+  qkv_store4(qkv, head * D + d0, token, packed);
 }
 
 // MT: slabs of 16 tokens a workgroup multiplies its weight rows with (1 for the plain product).
@@ -312,9 +321,14 @@ __device__ __forceinline__ void place_workgroup(const TileOrder& order, int id, 
   nt = in_group / size;
 }
 
-template <int WM, int WN, bool DEEP, int GM = 2, int GN = 2>
+// QKV: the fused query/key/value product (see QkvTarget).  The 32-feature blocks of a tile of
+// the rotated part (query and key heads) come in pairs: an even block holds 32 dims j of the
+// first half of their heads, the odd block after it their partners j + head_dim/2; tiles of the
+// value heads (and all tiles, without rotation) hold consecutive rows.
+template <int WM, int WN, bool DEEP, int GM = 2, int GN = 2, bool QKV = false>
 __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
-                                                         GemmEpilogue ep, TileOrder order, int M, int N, int K) {
+                                                                  GemmEpilogue ep, QkvTarget qkv, TileOrder order, int M,
+                                                                  int N, int K) {
   using Shape = TiledShape<WM, WN, GM, GN>;
   constexpr int BM = Shape::BM, BN = Shape::BN, PIECES = Shape::kPieces, THREADS = Shape::kThreads;
   // Two LDS buffers, each BN rows of w and then BM rows of x.  Addressed as offsets from
@@ -341,10 +355,37 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
   const int s_begin = slice * per;
   const int s_end = min(k_slices, s_begin + per);
 
-  // global -> register staging through two buffer resources that cover exactly this tile's
-  // rows: rows past the end of the matrix, and the tail of K, read as zeros.
+  // which weight row stands behind feature slot `slot` of this tile (-1: none)
+  bool rotated = false;
+  int pair_base = 0, row_base = n0, rot_pairs = 0;
+  if constexpr (QKV) {
+    rot_pairs = qkv.cos != nullptr ? (qkv.heads + qkv.kv_heads) * (qkv.head_dim / 2) : 0;
+    const int rot_tiles = (rot_pairs + BN / 2 - 1) / (BN / 2);
+    rotated = nt < rot_tiles;
+    pair_base = nt * (BN / 2);
+    row_base = 2 * rot_pairs + (nt - rot_tiles) * BN;
+  }
+  auto row_of = [&](int slot) {
+    if constexpr (QKV) {
+      if (rotated) {
+        const int block = slot / 32;
+        const int pair = pair_base + (block / 2) * 32 + slot % 32;
+        if (pair >= rot_pairs) return -1;
+        const int half = qkv.head_dim / 2;
+        const int head = pair / half;
+        return head * qkv.head_dim + (pair - head * half) + ((block & 1) ? half : 0);
+      }
+    }
+    return row_base + slot < N ? row_base + slot : -1;
+  };
+
+  // global -> register staging through two buffer resources: rows past the end of the
+  // matrix, and the tail of K, read as zeros.  The weight resource covers this tile's rows
+  // (QKV: the whole matrix, since a tile's rows lie apart).
   const int w_rows = min(BN, N - n0), x_rows = min(BM, M - m0);
-  const __amdgpu_buffer_rsrc_t w_buf = make_buffer(w + static_cast<int64_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2u);
+  const __amdgpu_buffer_rsrc_t w_buf =
+      QKV ? make_buffer(w, static_cast<unsigned>(N) * K * 2u)
+          : make_buffer(w + static_cast<int64_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2u);
   const __amdgpu_buffer_rsrc_t x_buf = make_buffer(x + static_cast<int64_t>(m0) * K, static_cast<unsigned>(x_rows) * K * 2u);
   unsigned piece_off[PIECES];  // byte offset of the piece in slice 0
   int lds_off[PIECES];
@@ -355,6 +396,12 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
     const int row = idx / (kBK / 8);
     const int ch = idx % (kBK / 8);
     piece_off[it] = static_cast<unsigned>(row < BN ? row : row - BN) * K * 2u + ch * 16u;
+    if constexpr (QKV) {
+      if (row < BN) {
+        const int weight_row = row_of(row);
+        piece_off[it] = weight_row >= 0 ? static_cast<unsigned>(weight_row) * K * 2u + ch * 16u : kOutOfBuffer;
+      }
+    }
     lds_off[it] = row * kLd + ch * 8;
     piece_chunk[it] = ch;
   }
@@ -430,18 +477,85 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
     }
   }
 
+  if constexpr (!QKV) {
 #pragma unroll
-  for (int i = 0; i < WN; ++i)
+    for (int i = 0; i < WN; ++i)
 #pragma unroll
-    for (int j = 0; j < WM; ++j) {
-      const int m = m0 + (wm * WM + j) * 32 + r32;
+      for (int j = 0; j < WM; ++j) {
+        const int m = m0 + (wm * WM + j) * 32 + r32;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = n0 + (wn * WN + i) * 32 + g * 8 + h * 4;
+          const float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+          finish4(ep, slice, slices, m, n, M, N, v);
+        }
+      }
+  } else {
+    // sums -> bias -> bfloat16 (as the unfused kernels hand the product on)
+    int row0[WN][4];  // weight row of the lane's first feature in group g of block i
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int n = n0 + (wn * WN + i) * 32 + g * 8 + h * 4;
-        const float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-        finish4(ep, slice, slices, m, n, M, N, v);
+        row0[i][g] = row_of((wn * WN + i) * 32 + g * 8 + h * 4);
+#pragma unroll
+        for (int j = 0; j < WM; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v = acc[i][j][g * 4 + e];
+            if (ep.bias != nullptr && row0[i][g] >= 0) v += load_as_f32(ep.bias, row0[i][g] + e, ep.bias_is_f32);
+            acc[i][j][g * 4 + e] = to_f32(f32_to_bf16(v));
+          }
+      }
+    // a rotated block needs its partner block: in the same wavefront when it holds two blocks
+    // side by side, else in the neighbouring wavefront, through LDS (the tiles are done with)
+    float* const exchange = reinterpret_cast<float*>(smem);
+    if constexpr (WN == 1) {
+      if (rotated) {
+        __syncthreads();  // every wavefront has read its last tile
+#pragma unroll
+        for (int j = 0; j < WM; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) exchange[((wave * WM + j) * 16 + e) * kWave + lane] = acc[0][j][e];
+        __syncthreads();
       }
     }
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        const int m = m0 + (wm * WM + j) * 32 + r32;
+        const int token = min(m, M - 1);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          if (row0[i][g] < 0) continue;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
+          if (rotated) {
+            const int D = qkv.head_dim, half = D / 2;
+            const int d = row0[i][g] % D;
+            const bool low = d < half;
+            const float* cs = qkv.cos + static_cast<int64_t>(token) * half + (low ? d : d - half);
+            const float* sn = qkv.sin + static_cast<int64_t>(token) * half + (low ? d : d - half);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float partner;
+              if constexpr (WN == 1)
+                partner = exchange[(((wave ^ 1) * WM + j) * 16 + g * 4 + e) * kWave + lane];
+              else
+                partner = acc[i ^ 1][j][g * 4 + e];
+              v[e] = low ? v[e] * cs[e] - partner * sn[e] : v[e] * cs[e] + partner * sn[e];
+            }
+          }
+          if (m >= M) continue;
+          u16x4_t packed;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) packed[e] = f32_to_bf16(v[e]).bits;
+          qkv_store4(qkv, row0[i][g], m, packed);
+        }
+      }
+  }
 }
 
 template <int WM, int WN, int GM = 2, int GN = 2>
@@ -466,7 +580,37 @@ static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, 
     return -1;
   }
   gemm_tiled_kernel<WM, WN, kDeep, GM, GN><<<dim3(static_cast<unsigned>(groups)), Shape::kThreads, Shape::kLds, stream>>>(
-      xb, wb, ep, order, m, n, k);
+      xb, wb, ep, QkvTarget{}, order, m, n, k);
+  return 0;
+}
+
+// The fused query/key/value product on the tiled kernel: tiles of the rotated part first
+// (pairs of 32-dim blocks), then tiles of consecutive rows for the rest.
+template <int WM, int WN, int GM = 2, int GN = 2>
+static int launch_tiled_qkv(const bf16* xb, const bf16* wb, GemmEpilogue ep, const QkvTarget& qkv, int m, int n, int k,
+                            hipStream_t stream) {
+  using Shape = TiledShape<WM, WN, GM, GN>;
+  constexpr bool kDeep = Shape::kDeep;
+  static_assert(WN == 1 || WN == 2, "a rotated block finds its partner beside it or in the next wavefront");
+  const int rot_pairs = qkv.cos != nullptr ? (qkv.heads + qkv.kv_heads) * (qkv.head_dim / 2) : 0;
+  const int rot_tiles = (rot_pairs + Shape::BN / 2 - 1) / (Shape::BN / 2);
+  const int rest_tiles = (n - 2 * rot_pairs + Shape::BN - 1) / Shape::BN;
+  const TileOrder order{(m + Shape::BM - 1) / Shape::BM, rot_tiles + rest_tiles, 1};
+  const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles;
+  MLR_REQUIRE(groups < (1ll << 31), "too many tiles for one launch");
+  static bool prepared = false;
+  if (!prepared) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, kDeep, GM, GN, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLds);
+    if (e != hipSuccess) {
+      set_error(std::string("mlr_qkv_rope_write_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
+      return -1;
+    }
+    prepared = true;
+  }
+  gemm_tiled_kernel<WM, WN, kDeep, GM, GN, true>
+      <<<dim3(static_cast<unsigned>(groups)), Shape::kThreads, Shape::kLds, stream>>>(xb, wb, ep, qkv, order, m, n, k);
+  MLR_LAUNCH_CHECK();
   return 0;
 }
 
@@ -577,32 +721,49 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
                             const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
-                            int write, hipStream_t stream) {
+                            int write, int kernel, hipStream_t stream) {
   MLR_REQUIRE(x && w && q_out, "null pointer");
-  MLR_REQUIRE(m > 0 && m <= 64, "the fused product takes 1..64 tokens");
-  MLR_REQUIRE(k > 0 && k % 8 == 0, "k must be a positive multiple of 8");
+  MLR_REQUIRE(m > 0, "no tokens");
+  MLR_REQUIRE(k > 0 && k % 8 == 0 && k <= (1 << 20), "k must be a positive multiple of 8, at most 2^20");
   MLR_REQUIRE(heads > 0 && kv_heads > 0 && head_dim >= 16 && head_dim % 16 == 0, "head_dim must be a multiple of 16");
   MLR_REQUIRE((cos == nullptr) == (sin == nullptr), "cos and sin come together");
   MLR_REQUIRE(!write || (slots && key_pages && value_pages && block_size > 0 && num_pages > 0),
               "a cache write needs slots, pages and their sizes");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
-                  reinterpret_cast<uintptr_t>(q_out) % 8 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 8 == 0,
+                  reinterpret_cast<uintptr_t>(q_out) % 8 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 8 == 0 &&
+                  reinterpret_cast<uintptr_t>(cos) % 16 == 0 && reinterpret_cast<uintptr_t>(sin) % 16 == 0,
               "operands must be 16-byte aligned");
   const int64_t n = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
   MLR_REQUIRE(n / 16 < (1ll << 31), "too many rows for one launch");
   GemmEpilogue ep{bias, bias_is_f32, nullptr, 0, 0};
   QkvTarget target{cos, sin, write ? slots : nullptr, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages),
                    static_cast<bf16*>(q_out), heads, kv_heads, head_dim, block_size, num_pages};
-  const dim3 grid(static_cast<unsigned>(n / 16));
   const bf16* xb = static_cast<const bf16*>(x);
   const bf16* wb = static_cast<const bf16*>(w);
-  if (m <= 16)
-    gemm_skinny_split_kernel<4, true, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
-  else if (m <= 32)
-    gemm_skinny_split_kernel<4, true, 2><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
-  else
-    gemm_skinny_split_kernel<4, true, 4><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
-  MLR_LAUNCH_CHECK();
+  if (kernel == 0) {
+    kernel = m <= 64 ? 16 : choose_kernel(m, static_cast<int>(n), k, 1);
+    if (kernel == 16 && m > 16 && (n / 16) * m * k * 2 > (32ll << 20)) kernel = 11;  // too many passes over x
+  }
+  if (kernel == 16) {
+    MLR_REQUIRE(m <= 64, "the row-splitting kernel takes 1..64 tokens");
+    const dim3 grid(static_cast<unsigned>(n / 16));
+    if (m <= 16)
+      gemm_skinny_split_kernel<4, true, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+    else if (m <= 32)
+      gemm_skinny_split_kernel<4, true, 2><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+    else
+      gemm_skinny_split_kernel<4, true, 4><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
+  // the tiled kernels address the whole weight matrix, and one token's rows of x, with 31-bit offsets
+  MLR_REQUIRE(n * k * 2 < (1ll << 31), "the weight matrix is too large for the tiled fused product");
+  switch (kernel) {
+    case 11: return launch_tiled_qkv<1, 1>(xb, wb, ep, target, m, static_cast<int>(n), k, stream);
+    case 22: return launch_tiled_qkv<2, 2>(xb, wb, ep, target, m, static_cast<int>(n), k, stream);
+    case 44: return launch_tiled_qkv<2, 2, 4, 4>(xb, wb, ep, target, m, static_cast<int>(n), k, stream);
+    default: MLR_REQUIRE(false, "unknown kernel");
+  }
   return 0;
 }
 

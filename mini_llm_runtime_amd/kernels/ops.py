@@ -38,7 +38,7 @@ _SIGNATURES = {
     "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
     "mlr_qkv_rope_write_bf16": (
-        [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
         _I,
     ),
     "mlr_paged_attention_simple": (
@@ -378,29 +378,30 @@ class HipOps:
         block_size: int,
         write: bool = True,
         fused: Optional[bool] = None,
+        mfma_kernel: int = 0,
     ) -> torch.Tensor:
         """Query/key/value product, rotation of queries and keys, keys and values into the cache.
 
         Returns a tensor whose leading num_heads * head_dim columns are the position-encoded
-        queries, for `paged_attention`.  Up to 64 bfloat16 tokens (decoding) run as ONE kernel
-        that rotates the sums and stores them where they belong; everything else is the product
-        followed by `rope_kv_write`.  `fused` forces one of the two ways (tests).
+        queries, for `paged_attention`.  In bfloat16 with a full rotation this is ONE kernel
+        that rotates the sums and stores them where they belong (a row-splitting kernel for up
+        to 64 tokens, a tiled one beyond); everything else is the product followed by
+        `rope_kv_write`.  `fused` forces one of the two ways, `mfma_kernel` the fused kernel
+        (tests).
         """
         m, k = x.shape
         width = (num_heads + 2 * num_kv_heads) * head_dim
         can_fuse = (
             self.dtype == torch.bfloat16
-            and m <= 64
             and k % 8 == 0
             and head_dim % 16 == 0
             and (rotation is None or rotation[2] == head_dim)
+            and (m <= 16 or width * k * 2 < 1 << 31)
         )
         if fused is None:
-            # every 16 features' workgroup reads all the tokens: beyond 16 tokens that pays only
-            # while this re-reading stays small beside the caches
-            fused = can_fuse and (m <= 16 or (width // 16) * m * k * 2 <= 32 << 20)
+            fused = can_fuse
         elif fused and not can_fuse:
-            raise KernelError("the fused query/key/value kernel takes up to 64 bfloat16 tokens and a full rotation")
+            raise KernelError("the fused query/key/value kernel takes bfloat16 tokens and a full rotation")
         if not fused:
             qkv = self.linear(x, weight, bias)
             self.rope_kv_write(
@@ -427,7 +428,7 @@ class HipOps:
             int(bias is not None and bias.dtype == torch.float32), self._ptr(cos), self._ptr(sin),
             self._ptr(slot_mapping if write else None), self._ptr(key_pages if write else None),
             self._ptr(value_pages if write else None), self._ptr(q), m, k, num_heads, num_kv_heads, head_dim,
-            block_size, num_pages, int(write), self._stream(),
+            block_size, num_pages, int(write), mfma_kernel, self._stream(),
         )
         return q
 

@@ -288,24 +288,34 @@ def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
     assert torch.equal(out[0, : heads * head_dim], qkv[0, : heads * head_dim])
 
 
-@pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,tokens,rotate,write", [
+_QKV_CASES = [
     (14, 2, 64, 896, 8, True, True), (3, 1, 16, 40, 1, True, True), (6, 3, 48, 104, 16, True, True),
     (4, 4, 80, 72, 5, False, True), (5, 1, 128, 136, 13, True, False),
     (14, 2, 64, 896, 64, True, True), (3, 1, 32, 104, 17, True, True), (2, 2, 16, 40, 33, True, True),
-])
-def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write):
-    """Decoding runs product, bias, rotation and cache write as one kernel; it has to leave the
-    queries and the pages exactly as the product followed by the rotation kernel does, and must
-    not touch any slot but the tokens' own (a token without a slot writes nothing)."""
+    (14, 2, 64, 896, 300, True, True, 0), (14, 2, 64, 896, 130, True, True, 11), (14, 2, 64, 896, 130, True, True, 22),
+    (14, 2, 64, 896, 300, True, True, 44), (3, 1, 48, 104, 70, True, True, 11), (3, 1, 48, 104, 70, True, True, 22),
+    (5, 3, 16, 40, 200, True, True, 44), (7, 1, 80, 72, 99, True, True, 22), (2, 2, 96, 136, 65, True, False, 11),
+    (4, 4, 80, 72, 77, False, True, 22), (5, 1, 256, 136, 40, True, True, 11), (3, 3, 128, 264, 150, True, True, 44),
+]
+
+
+@pytest.mark.parametrize(
+    "heads,kv_heads,head_dim,hidden,tokens,rotate,write,kernel", [c if len(c) == 8 else c + (0,) for c in _QKV_CASES]
+)
+def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write, kernel):
+    """Product, bias, rotation and cache write run as one kernel (a row-splitting one for few
+    tokens, the tiled ones, each forced here, for many); it has to leave the queries and the
+    pages as the product followed by the rotation kernel does, and must not touch any slot but
+    the tokens' own (a token without a slot writes nothing)."""
     ops = ops_for(torch.bfloat16)
-    bs, pages = 8, 9
+    bs, pages = 8, max(9, tokens // 8 + 2)
     width = (heads + 2 * kv_heads) * head_dim
     x = _rand((tokens, hidden), torch.bfloat16, 71).cuda()
     w = _rand((width, hidden), torch.bfloat16, 72, 0.2).cuda()
     b = _rand((width,), torch.float32, 73).cuda()
     rotation = None
     if rotate:
-        pos = torch.tensor(([3, 0, 911, 17, 40000] + list(range(5, 64)))[:tokens], dtype=torch.int32).cuda()
+        pos = torch.tensor(([3, 0, 911, 17, 40000] + list(range(5, tokens)))[:tokens], dtype=torch.int32).cuda()
         inv = (1.0 / (1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))).cuda()
         cos, sin = ops.rope_table(pos, inv)
         rotation = (cos, sin, head_dim)
@@ -319,11 +329,12 @@ def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads,
         kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=torch.bfloat16).cuda()
         vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=torch.bfloat16).cuda()
         q = ops.qkv_rope_write(x, w, b, rotation, slots, kp, vp, num_heads=heads, num_kv_heads=kv_heads,
-                               head_dim=head_dim, block_size=bs, write=write, fused=fused)
+                               head_dim=head_dim, block_size=bs, write=write, fused=fused,
+                               mfma_kernel=kernel if fused else 0)
         out[fused] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
     for name, a, c in zip(("queries", "key pages", "value pages"), out[False], out[True]):
         assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
-        if tokens <= 16:
+        if tokens <= 16 and kernel == 0:
             # both ways sum the product in the same order; the rotation's two products may be
             # contracted differently: a last-place difference at most
             tol = dict(atol=0, rtol=2 ** -7)
