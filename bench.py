@@ -11,6 +11,13 @@ timed steps between device synchronisations.  One JSON line is printed:
 `prefill` is one 2,048-token prompt; `roofline` prices the decode step by the
 bytes it must read (every weight once and the live requests' cache) against
 8 TB/s.  Peaks are MI355X's published dense figures.
+
+Two further workloads print a JSON line of their own (`--workload`):
+`burst`: 64 requests arrive at once, prompt lengths uniform in [128, 2048], 32/64/128/256 new
+tokens in turn, 2,048 tokens a step: generated tokens a second, medians of the time to the
+first token and of the time between tokens.  `chunked`: 32 requests decode at context 2,048
+while one 8,192-token prompt is taken in four portions of 2,048 tokens beside them: the time of
+such a mixed step, which is also the time between the decoding requests' tokens.
 """
 
 from __future__ import annotations
@@ -42,7 +49,180 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--prompt-len", type=int, default=PROMPT_LEN)
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked"))
     return p.parse_args()
+
+
+def median(values):
+    ordered = sorted(values)
+    return ordered[len(ordered) // 2]
+
+
+def workload_config(args, config, full_layers: int) -> dict:
+    return {
+        "model": f"{args.config} shape",
+        "layers": config.num_hidden_layers,
+        "layers_full_model": full_layers,
+        "hidden_size": config.hidden_size,
+        "num_attention_heads": config.num_attention_heads,
+        "num_key_value_heads": config.num_key_value_heads,
+        "head_dim": config.head_dim,
+        "intermediate_size": config.intermediate_size,
+        "vocab_size": config.vocab_size,
+        "kv_block_size": BLOCK_SIZE,
+    }
+
+
+def burst(args, config, full_layers, model, ops, device) -> dict:
+    """64 requests at once through the continuous-batching engine, 2,048 tokens a step."""
+    import random
+
+    import torch
+
+    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
+    from mini_llm_runtime_amd.engine.factory import make_cache
+    from mini_llm_runtime_amd.engine.runner import ModelRunner
+    from mini_llm_runtime_amd.sampling.sampler import Sampler
+
+    requests, budget = 64, 2048
+    pages = requests * (-(-(2048 + 256) // BLOCK_SIZE)) + 8
+    cache = make_cache(model, block_size=BLOCK_SIZE, num_blocks=pages, max_requests=requests)
+    runner = ModelRunner(model, cache, ops)
+    sampler = Sampler(ops, device)
+
+    def run(seed: int):
+        admission = PagedBlockAdmissionController(cache, max_step_tokens=budget)
+        scheduler = RequestScheduler(
+            max_running_requests=requests, max_batch_tokens=budget, admission_callback=admission.try_admit
+        )
+        engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
+        rng = random.Random(seed)
+        prompt_tokens = generated = 0
+        torch.cuda.synchronize(device)
+        t0 = time.perf_counter()
+        for i in range(requests):
+            n, new = rng.randint(128, 2048), (32, 64, 128, 256)[i % 4]
+            engine.submit(f"s{seed}-{i}", [rng.randrange(config.vocab_size) for _ in range(n)], max_new_tokens=new)
+            prompt_tokens += n
+            generated += new
+        steps = 0
+        while engine.scheduler.has_unfinished_requests:
+            engine.step()
+            steps += 1
+        torch.cuda.synchronize(device)
+        seconds = time.perf_counter() - t0
+        shots = engine.metrics.snapshots()
+        return {
+            "seconds": seconds,
+            "steps": steps,
+            "prompt_tokens": prompt_tokens,
+            "generated": generated,
+            "ttft_ms": median([m.ttft_ms for m in shots]),
+            "tpot_ms": median([m.median_tpot_ms for m in shots]),
+        }
+
+    if args.warmup:
+        run(args.seed + 1000)  # libraries loaded, the decode steps' graphs recorded
+    runs = [run(args.seed + r) for r in range(3)]
+    best = median([(r["seconds"], i) for i, r in enumerate(runs)])[1]
+    r = runs[best]
+    return {
+        "metric": "burst generated tokens/s",
+        "value": round(r["generated"] / r["seconds"], 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "higher_is_better": True,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights, uniform random token ids)",
+        "seconds": round(r["seconds"], 4),
+        "engine_steps": r["steps"],
+        "prompt_tokens": r["prompt_tokens"],
+        "generated_tokens": r["generated"],
+        "total_tokens_per_s": round((r["prompt_tokens"] + r["generated"]) / r["seconds"], 1),
+        "median_ttft_ms": round(r["ttft_ms"], 2),
+        "median_tpot_ms": round(r["tpot_ms"], 3),
+        "runs_seconds": [round(x["seconds"], 4) for x in runs],
+        "config": dict(workload_config(args, config, full_layers), requests=requests, max_batch_tokens=budget),
+    }
+
+
+def chunked(args, config, full_layers, model, ops, device) -> dict:
+    """One 8,192-token prompt in portions of 2,048 tokens beside 32 decoding requests."""
+    import torch
+
+    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
+    from mini_llm_runtime_amd.engine.factory import make_cache
+    from mini_llm_runtime_amd.engine.runner import ModelRunner
+    from mini_llm_runtime_amd.sampling.sampler import Sampler
+
+    decoders, context, long_prompt, portion, repeats = 32, 2048, 8192, 2048, 3
+    new_tokens = decoders + 64 + (repeats + 2) * (long_prompt // portion + 2)
+    pages = decoders * (-(-(context + new_tokens) // BLOCK_SIZE)) + (long_prompt + 16) // BLOCK_SIZE + 8
+    cache = make_cache(model, block_size=BLOCK_SIZE, num_blocks=pages, max_requests=decoders + 1)
+    runner = ModelRunner(model, cache, ops)
+    sampler = Sampler(ops, device)
+    admission = PagedBlockAdmissionController(cache, max_step_tokens=portion + decoders)
+    scheduler = RequestScheduler(
+        max_running_requests=decoders + 1,
+        max_batch_tokens=portion + decoders,
+        max_mixed_prefill_tokens=portion,
+        admission_callback=admission.try_admit,
+    )
+    engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
+    gen = torch.Generator().manual_seed(args.seed)
+
+    def ids(n: int) -> list[int]:
+        return torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+
+    def timed_step():
+        torch.cuda.synchronize(device)
+        t0 = time.perf_counter()
+        result = engine.step()
+        torch.cuda.synchronize(device)
+        return result, (time.perf_counter() - t0) * 1e3
+
+    for i in range(decoders):
+        engine.submit(f"d{i}", ids(context), max_new_tokens=new_tokens)
+    while len(engine.step().batch.decode_request_ids) < decoders:
+        pass
+    for _ in range(8):
+        engine.step()
+    alone = median([timed_step()[1] for _ in range(16)])
+    portions = long_prompt // portion
+    warmups = 2  # a shape of step is run plainly when it first comes and recorded when it comes again
+    mixed = [[] for _ in range(portions)]
+    for r in range(warmups + repeats):
+        engine.submit(f"long{r}", ids(long_prompt), max_new_tokens=1)
+        for i in range(portions):
+            result, ms = timed_step()
+            batch = result.batch
+            assert batch.prefill_request_ids == (f"long{r}",) and len(batch.decode_request_ids) == decoders
+            assert batch.token_count == portion + decoders
+            if r >= warmups:
+                mixed[i].append(ms)
+        assert not timed_step()[0].batch.prefill_request_ids
+    by_portion = [median(times) for times in mixed]
+    ms = sum(by_portion) / portions
+    return {
+        "metric": "mixed step: 2,048 prompt tokens beside 32 decoding requests (mean over the prompt's portions)",
+        "value": round(ms, 3),
+        "unit": "ms",
+        "n_gpus": 1,
+        "higher_is_better": False,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights, uniform random token ids)",
+        "decoders_tpot_ms_beside_the_prompt": round(ms, 3),
+        "decoders_tpot_ms_alone": round(alone, 3),
+        "prompt_tokens_per_s": round(portion * 1e3 / ms, 1),
+        "mixed_steps_ms_by_portion": [round(x, 3) for x in by_portion],
+        "config": dict(
+            workload_config(args, config, full_layers),
+            decoders=decoders,
+            decoders_context=context,
+            prompt_len=long_prompt,
+            portion=portion,
+        ),
+    }
 
 
 def main() -> int:
@@ -76,6 +256,11 @@ def main() -> int:
     with tempfile.TemporaryDirectory(prefix="mlr_bench_") as tmp:
         folder = write_random_model(config, tmp, seed=args.seed, storage_dtype="bfloat16")
         _, model = load_model(folder, dtype=dtype, device=device)
+
+    if args.workload != "decode":
+        line = (burst if args.workload == "burst" else chunked)(args, config, full_layers, model, ops, device)
+        print(json.dumps(line), flush=True)
+        return 0
 
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
     steps_total = args.warmup + args.steps
