@@ -632,16 +632,35 @@ static int tiles_256(int m, int n) { return ((n + 255) / 256) * ((m + 255) / 256
 // compute units, the 16-feature streaming kernel below that.
 static bool few_tokens_tiled(int n, int slices) { return ((n + 63) / 64) * slices >= 256; }
 
+// Kernel and number of K slices for more than 64 tokens, when the consumer takes up to
+// `max_slices` partial sums.  A larger tile needs less L2 traffic per flop and wins once there
+// are enough of them to keep the compute units busy; the largest one wants K long enough to pay
+// for its prologue, or many tiles.  A narrow output with a long K (the feed-forward's second
+// product) has too few large tiles: cut along K it fills the compute units with large tiles all
+// the same, as long as every slice stays long.
+struct GemmPlan {
+  int kernel, slices;
+};
+static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
+  const int big = tiles_256(m, n), mid = tiles_128(m, n);
+  if (big >= 144 && (big >= 512 || k >= 2048)) return {44, 1};
+  if (max_slices >= 2 && big * 2 >= 192 && k >= 8192) return {44, 2};
+  if (mid >= 256) return {22, 1};
+  if (mid >= 64) {
+    int slices = 1;
+    while (slices < max_slices && slices < 4 && mid * slices < 256 && k / (2 * slices) >= 4096) slices *= 2;
+    if (slices > 1) return {22, slices};
+  }
+  return {11, choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 4))};
+}
+
 // The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,
-// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles.  A larger tile
-// needs less L2 traffic per flop and wins once there are enough of them to keep the compute
-// units busy; the largest one wants K long enough to pay for its prologue, or many tiles.
+// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles.
 static int choose_kernel(int m, int n, int k, int slices) {
   if (m <= 16 && !few_tokens_tiled(n, slices)) return 16;
-  if (m <= 64 || slices > 1) return 11;
-  const int big = tiles_256(m, n);
-  if (big >= 144 && (big >= 512 || k >= 2048)) return 44;
-  return tiles_128(m, n) >= 256 ? 22 : 11;
+  if (m <= 64) return 11;
+  const GemmPlan plan = plan_many_tokens(m, n, k, slices);
+  return plan.slices == slices ? plan.kernel : 11;
 }
 
 static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
@@ -673,7 +692,7 @@ extern "C" {
 // partial sums (at most `max_slices`); 1 means it writes the finished product.
 int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
   if (k % 8 != 0) return 1;
-  if (m > 64 && tiles_128(m, n) >= 256) return 1;
+  if (m > 64) return plan_many_tokens(m, n, k, max_slices).slices;
   if (m <= 16) {
     // Measured with the norm kernel that adds the slices up (its cost grows with their number):
     // a weight of 64 MB or more streams fastest through the LDS-tiled kernel cut into 8 slices;
@@ -685,7 +704,7 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
     return max(by_fill, min(min(4, max_slices), k / 2560));
   }
   // more slices fill the compute units, but the norm that adds them up reads them all
-  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, m > 64 ? 4 : 8));
+  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 8));
 }
 
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the

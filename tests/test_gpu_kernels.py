@@ -175,7 +175,7 @@ def test_linear_swiglu_epilogue(ops_for, dtype, m, inter, k):
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 896, 4864), (8, 896, 896), (16, 130, 2056), (33, 517, 2056), (64, 896, 4864), (8, 151936, 96),
-     (300, 517, 4104), (2048, 896, 4864), (130, 130, 1032)],
+     (300, 517, 4104), (2048, 896, 4864), (130, 130, 1032), (1000, 1030, 8200), (2040, 3000, 8192)],
 )
 def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     """A narrow product of a few tokens may come back as float32 partial sums over slices of k;
@@ -193,8 +193,8 @@ def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
         assert got.shape == (m, n)  # wide enough: not cut
         total = got.cpu().double()
     torch.testing.assert_close(total, ref, **(_tol(torch.bfloat16) if got.dim() == 2 else dict(atol=2e-3, rtol=1e-4)))
-    if k >= 4104 and m <= 300:
-        assert got.dim() == 3, "a long, narrow product of few tokens should be cut along k"
+    if k >= 4104 and (m <= 300 or k >= 8192):
+        assert got.dim() == 3, "a long, narrow product should be cut along k"
     stream = _rand((m, n), torch.float32, 49, 2.0)
     nw = (1 + _rand((n,), torch.float32, 50, 0.1)).to(torch.bfloat16)
     sd = stream.cuda().clone()
