@@ -42,31 +42,53 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
   const int quads = hidden / 4;
+  // Loads first, all of them unconditional (an index past the end is clamped and its value
+  // dropped), so that they are in flight together: a wait per slice would cost more than the
+  // whole kernel otherwise.
+  constexpr int kSliceBatch = 8;
   f32x4 v[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = min(threadIdx.x + j * 256, quads - 1);
+    const int64_t at = row * hidden + 4 * i;
+    v[j] = *reinterpret_cast<const f32x4*>(x + at);
+    if (delta != nullptr) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[j][e] += to_f32(delta[at + e]);
+    }
+  }
+  for (int s0 = 0; s0 < slices; s0 += kSliceBatch) {
+    f32x4 p[VPT][kSliceBatch];
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const int i = min(threadIdx.x + j * 256, quads - 1);
+#pragma unroll
+      for (int u = 0; u < kSliceBatch; ++u) {
+        const int sl = min(s0 + u, slices - 1);
+        p[j][u] = *reinterpret_cast<const f32x4*>(partial + (static_cast<int64_t>(sl) * rows + row) * hidden + 4 * i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kSliceBatch; ++u) {
+      const bool live = s0 + u < slices;
+#pragma unroll
+      for (int j = 0; j < VPT; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[j][e] = live ? v[j][e] + p[j][u][e] : v[j][e];
+    }
+  }
   float ss = 0.f;
+  const bool changed = delta != nullptr || slices > 0;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int i = threadIdx.x + j * 256;
-    v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (i >= quads) continue;
-    const int64_t at = row * hidden + 4 * i;
-    f32x4 a = *reinterpret_cast<const f32x4*>(x + at);
-    bool changed = false;
-    if (delta != nullptr) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) a[e] += to_f32(delta[at + e]);
-      changed = true;
+    if (i >= quads) {
+      v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      continue;
     }
-    for (int s = 0; s < slices; ++s) {
-      const f32x4 p = *reinterpret_cast<const f32x4*>(partial + (static_cast<int64_t>(s) * rows + row) * hidden + 4 * i);
+    if (changed) *reinterpret_cast<f32x4*>(x + row * hidden + 4 * i) = v[j];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) a[e] += p[e];
-      changed = true;
-    }
-    if (changed) *reinterpret_cast<f32x4*>(x + at) = a;
-    v[j] = a;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) ss += a[e] * a[e];
+    for (int e = 0; e < 4; ++e) ss += v[j][e] * v[j][e];
   }
   const float total = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
