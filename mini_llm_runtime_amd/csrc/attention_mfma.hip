@@ -438,10 +438,12 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   const int entry = tiles[2 * tile];
   const int q0 = tiles[2 * tile + 1];
   const int kvh = head / (heads / kv_heads);
-  const int group = threadIdx.x / 256;  // key group
-  const int tid = threadIdx.x % 256;    // thread within the group
+  // uniform in a wavefront, and said so: everything derived from them (tile positions, the
+  // conditions on them) then lives in scalar registers and scalar branches
+  const int group = __builtin_amdgcn_readfirstlane(threadIdx.x / 256);  // key group
+  const int tid = threadIdx.x % 256;                                     // thread within the group
   const int lane = tid % kWave;
-  const int wave = tid / kWave;  // which 16 queries
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // which 16 queries
   const int col = lane % 16;
   const int quarter = lane / 16;
 
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     v_in_page[i] = (kvh * D + d) * block_size + part * 8;
     v_lds[i] = kTileK * kKLd + d * kVLd + pg * block_size + part * 8;
   }
-  const int64_t page_elems = static_cast<int64_t>(kv_heads) * block_size * D;
+  const uint32_t page_elems = static_cast<uint32_t>(kv_heads) * block_size * D;  // one multiply-add per address
   const int last_page = (k_end - 1) >> bs_shift;  // the last table entry that any query here may use
 
   // Loads are unconditional (a page that is absent or past the end reads page 0 instead) so
@@ -537,16 +539,17 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     for (int i = 0; i < kPieces; ++i) {
       const int page = k_ids[i];
       const bool in = static_cast<unsigned>(page) < static_cast<unsigned>(num_pages);
-      bad = bad || (!in && k_row[i] < lim && kt0 + k_row[i] >= k_begin_raw);
-      t.k[i] = load_bf16x8(key_pages + ((in ? page : 0) * page_elems + k_in_page[i]));
+      if (!in) bad = bad || (k_row[i] < lim && kt0 + k_row[i] >= k_begin_raw);
+      t.k[i] = load_bf16x8(key_pages + (static_cast<uint64_t>(in ? static_cast<uint32_t>(page) : 0u) * page_elems + k_in_page[i]));
     }
     const bool guard = lim < kTileK || window > 0;  // uniform
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
       const int page = v_ids[i];
       const bool in = static_cast<unsigned>(page) < static_cast<unsigned>(num_pages);
-      bf16x8_t val = load_bf16x8(value_pages + ((in ? page : 0) * page_elems + v_in_page[i]));
+      bf16x8_t val = load_bf16x8(value_pages + (static_cast<uint64_t>(in ? static_cast<uint32_t>(page) : 0u) * page_elems + v_in_page[i]));
       if (guard) {
+        asm volatile("" ::: "memory");  // keeps this a branch that full tiles skip
         u16x8_t bits = __builtin_bit_cast(u16x8_t, val);
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -564,6 +567,11 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
         *reinterpret_cast<bf16x8_t*>(lds + (buf * kKeyGroups + group) * kBuffer + v_lds[i]) = t.v[i];
       }
   };
+
+  // The query has to be there before the loop: a load still pending at the loop's head makes
+  // the compiler wait, in every turn, for everything in flight, the next tile's loads included.
+#pragma unroll
+  for (int st = 0; st < kSteps; ++st) asm volatile("" ::"v"(qo.step[st]));
 
   TileInFlight flight;
   constexpr int kStep = kKeyGroups * kTileK;  // keys per turn of the loop, all groups together
@@ -598,6 +606,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       for (int sub = 0; sub < kSubTiles; ++sub)
         s[sub] = score_tile(load_row(ks + (sub * 16 + col) * kKLd, true, quarter), qo);
       if (!full) {
+        // a branch of its own: folded into selects, these comparisons would run for every tile
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int sub = 0; sub < kSubTiles; ++sub)
 #pragma unroll
@@ -783,6 +793,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
                           int block_size, int num_pages, float scale, int window, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(num_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad sizes");
+  MLR_REQUIRE(kv_heads <= 65535, "too many key/value heads");  // a page's elements fit 32 bits
   MLR_REQUIRE(block_size >= 8 && (block_size & (block_size - 1)) == 0 && block_size <= kTileK,
               "block_size must be a power of two within 8 and the key tile");
   int bs_shift = 0;
