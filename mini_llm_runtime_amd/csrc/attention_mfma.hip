@@ -391,8 +391,12 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 // ---- prefill ----------------------------------------------------------------------------------
 constexpr int kTileQ = 64;                 // queries per workgroup (16 per wavefront)
 constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounded by LDS)
-constexpr int kKeyGroups = D <= 64 ? 2 : 1;  // wavefront groups of a workgroup that take key tiles in turn (registers allow
-                                            // two resident groups per SIMD only for the small head sizes)
+// Wavefront groups of a workgroup that take the key tiles in turn and merge at the end: a
+// query tile's keys are a chain of dependent steps, and a second group halves it.  Measured:
+// two groups for the small head sizes (where registers allow two workgroups of them per
+// compute unit); four groups, or two for the larger head sizes, leave one workgroup per
+// compute unit and are slower.
+constexpr int kKeyGroups = D <= 64 ? 2 : 1;
 constexpr int kSubTiles = kTileK / 16;
 constexpr int kPairs = kSubTiles / 2;      // the value product takes 32 key positions per MFMA
 constexpr int kKLd = D + 8;                // padded key row in LDS (elements)
@@ -605,6 +609,23 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
 #pragma unroll
       for (int sub = 0; sub < kSubTiles; ++sub)
         s[sub] = score_tile(load_row(ks + (sub * 16 + col) * kKLd, true, quarter), qo);
+      // The value operands of the tile's first 32 keys leave LDS now: the softmax below hides
+      // their way, which would otherwise be waited for once per product.
+      typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+      auto value_operand = [&](int dt, int pr) {
+        const bf16* vrow = vs + (dt * 16 + col) * kVLd + pr * 32 + quarter * 4;
+        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vrow);
+        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vrow + 16);
+        return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+      };
+      constexpr bool kValuesAhead = kDimTiles <= 8;  // registers allow it
+      u32x4_t ahead[kValuesAhead ? kDimTiles : 1];
+      if constexpr (kValuesAhead) {
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt) ahead[dt] = value_operand(dt, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (!full) {
         // a branch of its own: folded into selects, these comparisons would run for every tile
         asm volatile("" ::: "memory");
@@ -649,18 +670,13 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       }
       // O^T += V^T P^T, 32 key positions per MFMA: k-slots 0..3 of a lane are its 4 keys of the
       // pair's first sub-tile, slots 4..7 those of the second; the value operand follows the same map
-      typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
       for (int pr = 0; pr < kPairs; ++pr) {
         const u32x4_t pb = {pw[2 * pr][0], pw[2 * pr][1], pw[2 * pr + 1][0], pw[2 * pr + 1][1]};
         const bf16x8_t pop = __builtin_bit_cast(bf16x8_t, pb);
 #pragma unroll
         for (int dt = 0; dt < kDimTiles; ++dt) {
-          const bf16* vrow = vs + (dt * 16 + col) * kVLd + pr * 32 + quarter * 4;
-          const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vrow);
-          const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vrow + 16);
-          const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
+          const u32x4_t va = (kValuesAhead && pr == 0) ? ahead[dt] : value_operand(dt, pr);
           acc[dt] = mfma_16x16x32(__builtin_bit_cast(bf16x8_t, va), pop, acc[dt]);
         }
       }
@@ -672,28 +688,34 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   }
 
   // merge the key groups: the second hands its state over through LDS (the tiles are done with)
-  float* const handover = reinterpret_cast<float*>(prefill_lds);  // [component][thread of the group]
-  if (kKeyGroups > 1 && group == 1) {
-    handover[tid] = m_run;
-    handover[256 + tid] = l_run;
+  float* const handover = reinterpret_cast<float*>(prefill_lds);  // [group - 1][component][thread of the group]
+  constexpr int kHandover = (2 + kDimTiles * 4) * 256;
+  static_assert((kKeyGroups - 1) * kHandover * 4 <= 2 * kKeyGroups * kBuffer * 2, "the handover fits the tile buffers");
+  if (kKeyGroups > 1 && group > 0) {
+    float* mine = handover + (group - 1) * kHandover;
+    mine[tid] = m_run;
+    mine[256 + tid] = l_run;
 #pragma unroll
     for (int dt = 0; dt < kDimTiles; ++dt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) handover[(2 + dt * 4 + i) * 256 + tid] = acc[dt][i];
+      for (int i = 0; i < 4; ++i) mine[(2 + dt * 4 + i) * 256 + tid] = acc[dt][i];
   }
   if (bad) atomicOr(&sm_bad, 1);
   __syncthreads();
   if (group != 0) return;
-  if constexpr (kKeyGroups > 1) {
-    const float m_other = handover[tid];
+#pragma unroll
+  for (int g = 1; g < kKeyGroups; ++g) {  // in the groups' order, whichever finished first
+    const float* other = handover + (g - 1) * kHandover;
+    const float m_other = other[tid];
     const float m_new = fmaxf(m_run, m_other);
     const float w_mine = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);
     const float w_other = (m_other == -INFINITY) ? 0.f : fast_exp2(m_other - m_new);
-    l_run = l_run * w_mine + handover[256 + tid] * w_other;
+    l_run = l_run * w_mine + other[256 + tid] * w_other;
 #pragma unroll
     for (int dt = 0; dt < kDimTiles; ++dt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[dt][i] = acc[dt][i] * w_mine + handover[(2 + dt * 4 + i) * 256 + tid] * w_other;
+      for (int i = 0; i < 4; ++i) acc[dt][i] = acc[dt][i] * w_mine + other[(2 + dt * 4 + i) * 256 + tid] * w_other;
+    m_run = m_new;
   }
   const bool poisoned = sm_bad != 0;
   l_run += __shfl_xor(l_run, 16, kWave);
