@@ -44,8 +44,43 @@ TINY_B = dict(
     hidden_act="silu",
     tie_word_embeddings=False,
 )
-TINY = {"A": TINY_A, "B": TINY_B}
-BLOCK_SIZE = {"A": 16, "B": 8}
+# Two more, with sizes that kernels dislike.  C: a head size that is not hidden / heads, a
+# group of three, one layer, an odd vocabulary.  D: a width and a feed-forward width that are
+# no multiples of 8 and a head size that is no multiple of 16 (the matrix-core kernels refuse
+# them and the plain 32-bit kernels take over), as many key/value heads as query heads.
+TINY_C = dict(
+    architectures=["Qwen2ForCausalLM"],
+    model_type="qwen2",
+    vocab_size=1003,
+    hidden_size=72,
+    intermediate_size=200,
+    num_hidden_layers=1,
+    num_attention_heads=6,
+    num_key_value_heads=2,
+    head_dim=48,
+    max_position_embeddings=256,
+    rms_norm_eps=3e-6,
+    rope_theta=500000.0,
+    hidden_act="silu",
+    tie_word_embeddings=True,
+)
+TINY_D = dict(
+    architectures=["Qwen2ForCausalLM"],
+    model_type="qwen2",
+    vocab_size=300,
+    hidden_size=100,
+    intermediate_size=108,
+    num_hidden_layers=2,
+    num_attention_heads=5,
+    num_key_value_heads=5,
+    max_position_embeddings=300,
+    rms_norm_eps=1e-4,
+    rope_theta=777.0,
+    hidden_act="silu",
+    tie_word_embeddings=False,
+)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+BLOCK_SIZE = {"A": 16, "B": 8, "C": 32, "D": 4}
 
 
 def make_model_dir(tmp_path: Path, which: str, seed: int = 0, storage_dtype: str = "bfloat16") -> Path:

@@ -15,7 +15,7 @@ import schedules
 from helpers import BLOCK_SIZE, TINY, StepEntry, make_model_dir, make_runner, random_tokens, read_weights
 from kernel_doubles import TorchOps
 
-LENGTHS = {"A": (5, 17, 33, 70, 41, 52), "B": (1, 9, 24, 40, 63, 37)}
+LENGTHS = {"A": (5, 17, 33, 70, 41, 52), "B": (1, 9, 24, 40, 63, 37), "C": (3, 65, 34, 97, 40, 51), "D": (2, 19, 35, 66, 45, 50)}
 
 # float32: the engine and the plain implementation (float64) differ by float32
 # rounding only.  bfloat16: activations between kernels are rounded to 8 bits of
@@ -104,7 +104,7 @@ CASES = [
 
 @pytest.mark.parametrize("backend,dtype", CASES)
 @pytest.mark.parametrize("family", list(FAMILIES))
-@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_schedule_matches_plain(tmp_path, which, family, backend, dtype):
     requests = _requests(which)
     steps = FAMILIES[family](requests)

@@ -23,7 +23,7 @@ from mini_llm_runtime_amd.engine import ModelRunner
 from mini_llm_runtime_amd.replay import PAGE_TOKENS, TraceError, replay
 
 ROOT = Path(__file__).resolve().parents[1]
-LENGTHS = {"A": (40, 75, 33, 130, 64, 90), "B": (36, 63, 100, 41, 77, 50)}
+LENGTHS = {"A": (40, 75, 33, 130, 64, 90), "B": (36, 63, 100, 41, 77, 50), "C": (35, 70, 99, 44, 65, 38), "D": (37, 66, 34, 101, 52, 40)}
 
 
 def _requests(which):
@@ -117,7 +117,7 @@ def test_replay_rejects_bad_lines(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_trace_run_program(tmp_path, gpu_device, which, dtype):
     d = make_model_dir(tmp_path, which, seed=33)
     cfg, w = read_weights(d)
