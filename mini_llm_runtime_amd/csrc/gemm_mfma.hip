@@ -25,6 +25,9 @@
 //    With more than one K slice both kernels write float32 partial sums
 //    [slice, M, N]; the consumer (the residual-adding norm kernel) sums them in a
 //    fixed order, so results do not depend on which slice finishes first.
+//  * Both also run the query/key/value product with bias, rotation and the cache write as
+//    their epilogue (QkvTarget): the streaming kernel for up to 64 tokens (in slabs of 16),
+//    the tiled one beyond.
 // K must be a multiple of 8 (16-byte rows); other shapes take the FMA kernel.
 //
 // SwiGLU epilogue: with gate and up rows interleaved in pairs
@@ -732,11 +735,11 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   return 0;
 }
 
-// The query/key/value product of up to 64 tokens with everything that follows it before
-// attention: bias, rotation of the query and key heads (cos, sin: [m, head_dim / 2] float32,
+// The query/key/value product with everything that follows it before attention: bias, rotation of the query and key heads (cos, sin: [m, head_dim / 2] float32,
 // or null for none), queries to q_out [m, heads * head_dim], keys and values into the slots
 // of their pages (`write` 0: another layer owns the pages).  w is [(heads + 2 kv_heads) *
-// head_dim, k]; head_dim a multiple of 16, k of 8.
+// head_dim, k]; head_dim a multiple of 16, k of 8.  kernel: 0 chooses (the streaming kernel up
+// to 64 tokens unless it would read x too often, else a tiled one), or 16, 11, 22, 44.
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
                             const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
