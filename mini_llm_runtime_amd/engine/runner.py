@@ -100,6 +100,7 @@ class ModelRunner:
         # time, and replayed from then on, if every part of the model allows it; a bounded number
         # of such recordings is kept, the least recently used one goes first.
         self.max_step_graphs = 16
+        self.max_decode_graphs = 64
         self.max_graph_tokens = 8192
         self._step_graphs: dict[tuple, tuple] = {}
         self._step_seen: dict[tuple, int] = {}
@@ -375,7 +376,7 @@ class ModelRunner:
         self, key: tuple[int, int], layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray
     ) -> torch.Tensor:
         padded, width = key
-        graph = self._graphs.get(key)
+        graph = self._graphs.pop(key, None)
         if graph is None:
             empty = np.zeros((0, 2), dtype=np.int32)
             arrays = self._arrays(layout, token_ids, logit_rows, empty, padded, width)
@@ -406,7 +407,13 @@ class ModelRunner:
             with torch.cuda.graph(captured):
                 out = self.model.forward(ctx, ctx.memo["logit_rows"])
             graph = (captured, static, out, spans, buf.size)
-            self._graphs[key] = graph
+            # nothing is running here (the plain run above was waited for): the graphs that
+            # were used longest ago can go
+            while len(self._graphs) >= self.max_decode_graphs:
+                oldest = next(iter(self._graphs))
+                del self._graphs[oldest]
+                self._staging.pop(oldest, None)
+        self._graphs[key] = graph  # most recently used last
         out = self._replay(key, graph, layout, token_ids, None)
         if logit_rows.size == layout.num_entries and (logit_rows == np.arange(layout.num_entries)).all():
             return out[: layout.num_entries]
@@ -455,10 +462,11 @@ class ModelRunner:
         layout = self.cache.begin_step([(rid, 1) for rid in request_ids])
         try:
             key = self._graph_key(layout)
-            graph = self._graphs.get(key) if key is not None else None
+            graph = self._graphs.pop(key, None) if key is not None else None
             if graph is None:
                 self.cache.abort_step()
                 return None
+            self._graphs[key] = graph  # most recently used last
             out = self._replay(key, graph, layout, np.zeros(count, dtype=np.int32), device_tokens)
         except BaseException:
             self.cache.abort_step()

@@ -166,6 +166,7 @@ def test_long_decoding_graph_replays_match_eager(tmp_path, dtype):
     for use_graphs in (True, False):
         config, model, cache, runner = make_runner(model_dir, ops, block_size=8, num_blocks=80, max_requests=4)
         runner.use_graphs = use_graphs
+        runner.max_decode_graphs = 2  # three batch sizes follow: the graph used longest ago has to go
         cache.poison()
         got = {}
         for rid, toks in requests.items():
@@ -188,7 +189,7 @@ def test_long_decoding_graph_replays_match_eager(tmp_path, dtype):
                     got[("x", fed_x + i)] = out.logits[i].float().cpu()
                 fed_x += n
         if use_graphs:
-            assert len(runner._graphs) >= 2, "the decode steps did not go through captured graphs"
+            assert len(runner._graphs) == 2, "the decode steps did not go through captured graphs, or too many were kept"
         results.append(got)
     graph, eager = results
     assert graph.keys() == eager.keys()
