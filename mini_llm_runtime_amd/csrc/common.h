@@ -69,16 +69,32 @@ __device__ inline float load_as_f32(const void* p, int64_t i, int is_f32) {
   return is_f32 ? static_cast<const float*>(p)[i] : to_f32(static_cast<const bf16*>(p)[i]);
 }
 
+// Reductions over a wavefront whose 64 lanes are all active; every lane gets the result.
+// Inside a row of 16 lanes the values rotate through the vector ALU's own lane crossbar
+// (DPP row_ror: every lane reads the lane 1, 2, 4, 8 places to its left, cyclically), then the
+// four rows' results meet as scalars.  A shuffle would go through LDS six times instead.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
 __device__ inline float wave_sum(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+  v += dpp_move<0x121>(v);  // row_ror:1
+  v += dpp_move<0x122>(v);  // row_ror:2
+  v += dpp_move<0x124>(v);  // row_ror:4
+  v += dpp_move<0x128>(v);  // row_ror:8
+  return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
 __device__ inline float wave_max(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-  return v;
+  v = fmaxf(v, dpp_move<0x121>(v));
+  v = fmaxf(v, dpp_move<0x122>(v));
+  v = fmaxf(v, dpp_move<0x124>(v));
+  v = fmaxf(v, dpp_move<0x128>(v));
+  return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
 // Sum over a workgroup of up to 1024 threads (a whole number of wavefronts);
