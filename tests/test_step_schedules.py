@@ -242,3 +242,36 @@ def test_recorded_prompt_steps_match_plain_steps(tmp_path, dtype):
             assert not runner._step_graphs
     for i, (want, have) in enumerate(zip(outputs[False], outputs[True])):
         assert torch.equal(want, have), f"step {i}: a replayed step differs from the plain one"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_half_billion_layer_sizes_match_plain(tmp_path, dtype):
+    """Two layers of the Qwen2.5-0.5B sizes (width 896, 14 query and 2 key/value heads of 64,
+    feed-forward 4864, vocabulary 151936): the kernels that the large tiles, the long rows of the
+    head and prompts of several query tiles select, against the plain implementation; one long
+    prompt whole and cut before its last 32 tokens, three shorter ones mixed."""
+    from mini_llm_runtime_amd.config.presets import load_preset
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+    from mini_llm_runtime_amd.models.registry import config_from_dict
+    from mini_llm_runtime_amd.weights import write_random_model
+
+    data = load_preset("qwen2.5-0.5b")
+    data["num_hidden_layers"] = 2
+    config = config_from_dict(data)
+    model_dir = write_random_model(config, tmp_path / "half", seed=21, storage_dtype="bfloat16")
+    cfg, weights = read_weights(model_dir)
+    vocab = cfg["vocab_size"]
+    long = {"w": random_tokens(1100, vocab, 700)}
+    short = {f"s{i}": random_tokens(n, vocab, 710 + i) for i, n in enumerate((150, 70, 97))}
+    _, _, cache, runner = make_runner(model_dir, HipOps(dtype, "cuda"), block_size=16, num_blocks=96, max_requests=4)
+    cache.poison()
+    for requests, steps in (
+        (long, schedules.whole(long)),
+        (long, schedules.bulk_then_tail(long)),
+        (short, schedules.mixed(short, seed=3)),
+    ):
+        got = schedules.run_schedule(runner, cache, steps)
+        _compare(got, requests, weights, cfg, dtype)
+    cache.check_invariants()
+    assert cache.request_ids == ()
