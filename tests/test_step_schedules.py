@@ -275,3 +275,29 @@ def test_half_billion_layer_sizes_match_plain(tmp_path, dtype):
         _compare(got, requests, weights, cfg, dtype)
     cache.check_invariants()
     assert cache.request_ids == ()
+
+
+@pytest.mark.gpu
+def test_seven_billion_layer_sizes_match_plain(tmp_path):
+    """One layer of the Qwen2.5-7B sizes (width 3584, 28 query and 4 key/value heads of 128,
+    feed-forward 18944; a small vocabulary keeps the plain implementation quick), bfloat16: the
+    largest tiles and the 128-wide heads inside the model."""
+    from mini_llm_runtime_amd.config.presets import load_preset
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+    from mini_llm_runtime_amd.models.registry import config_from_dict
+    from mini_llm_runtime_amd.weights import write_random_model
+
+    data = load_preset("qwen2.5-7b")
+    data["num_hidden_layers"] = 1
+    data["vocab_size"] = 4099
+    config = config_from_dict(data)
+    model_dir = write_random_model(config, tmp_path / "seven", seed=22, storage_dtype="bfloat16")
+    cfg, weights = read_weights(model_dir)
+    long = {"w": random_tokens(700, cfg["vocab_size"], 720)}
+    short = {f"s{i}": random_tokens(n, cfg["vocab_size"], 730 + i) for i, n in enumerate((90, 40))}
+    _, _, cache, runner = make_runner(model_dir, HipOps(torch.bfloat16, "cuda"), block_size=16, num_blocks=64, max_requests=4)
+    cache.poison()
+    for requests, steps in ((long, schedules.whole(long)), (short, schedules.mixed(short, seed=4))):
+        got = schedules.run_schedule(runner, cache, steps)
+        _compare(got, requests, weights, cfg, torch.bfloat16)
+    cache.check_invariants()
