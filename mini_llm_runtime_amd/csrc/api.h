@@ -103,4 +103,17 @@ int64_t mlr_sample_scratch(int rows, int vocab);
 int mlr_sample(const float* logits, const float* temperature, const float* uniform, int* tokens,
                float* scratch, int rows, int vocab, hipStream_t stream);
 
+// mlr_sample without a scratch argument and without any allocation: the segment results live
+// in an array inside the library (256 KiB per GPU, held until the process ends).  It has no
+// counterpart in the reference; it is for callers that cannot allocate device memory: code
+// under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+// kernels and same results as mlr_sample.  rows * ceil(vocab / 4096) * 3 must not exceed
+// mlr_sample_static_capacity() floats, else -1 with a message.  The stream's device must be the
+// current device.  All calls on one GPU share that GPU's array: calls that overlap there (two
+// streams, two threads) race, so order them.  The first call on a device looks up the array's
+// address (no allocation); make it outside a graph capture.
+int64_t mlr_sample_static_capacity();
+int mlr_sample_static(const float* logits, const float* temperature, const float* uniform, int* tokens,
+                      int rows, int vocab, hipStream_t stream);
+
 }  // extern "C"

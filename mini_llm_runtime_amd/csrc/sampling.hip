@@ -12,7 +12,16 @@
 #include "api.h"
 #include "common.h"
 
+#include <mutex>
+
 namespace mlr {
+
+// Scratch of mlr_sample_static: the (max, argmax, sum) triples that sample_partial leaves for
+// sample_final, held by the library itself so that the entry point never allocates.  Every GPU
+// the library runs on holds its own copy of this array, at its own address, until the process
+// ends.  In host code the name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr int kStaticScratchFloats = 65536;  // 256 KiB
+static __device__ __align__(256) float sample_scratch[kStaticScratchFloats];
 
 constexpr int kSegment = 4096;
 constexpr int kSampleThreads = 256;
@@ -202,6 +211,58 @@ int mlr_sample(const float* logits, const float* temperature, const float* unifo
                                                                              segments);
   MLR_LAUNCH_CHECK();
   sample_final_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, scratch, tokens, vocab,
+                                                           segments);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int64_t mlr_sample_static_capacity() { return kStaticScratchFloats; }
+
+int mlr_sample_static(const float* logits, const float* temperature, const float* uniform, int* tokens, int rows,
+                      int vocab, hipStream_t stream) {
+  MLR_REQUIRE(logits && tokens, "null pointer");
+  MLR_REQUIRE(rows > 0 && vocab > 0, "sizes must be > 0");
+  MLR_REQUIRE((temperature == nullptr) == (uniform == nullptr), "temperature and uniform come together");
+  const int segments = (vocab + kSegment - 1) / kSegment;
+  MLR_REQUIRE(segments <= 65535, "vocabulary too large for one launch");
+  const int64_t needed = static_cast<int64_t>(rows) * segments * 3;
+  if (needed > kStaticScratchFloats) {
+    set_error("mlr_sample_static: " + std::to_string(rows) + " rows of " + std::to_string(vocab) + " logits need " +
+              std::to_string(needed) + " floats of scratch, the library holds " + std::to_string(kStaticScratchFloats) +
+              " (rows * ceil(vocab / 4096) * 3 must not exceed that); use mlr_sample with a buffer of the caller");
+    return -1;
+  }
+  // The array's address on the current device, asked for once per device.
+  constexpr int kMaxDevices = 64;
+  static float* address[kMaxDevices] = {};
+  static std::mutex guard;
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error(std::string("mlr_sample_static: no usable current device: ") + hipGetErrorString(e));
+    return -1;
+  }
+  float* scratch_ptr = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(guard);
+    if (address[device] == nullptr) {
+      void* found = nullptr;
+      e = hipGetSymbolAddress(&found, HIP_SYMBOL(sample_scratch));
+      if (e != hipSuccess || found == nullptr) {
+        set_error(std::string("mlr_sample_static: cannot find the scratch array on device ") + std::to_string(device) +
+                  ": " + hipGetErrorString(e));
+        return -1;
+      }
+      address[device] = static_cast<float*>(found);
+    }
+    scratch_ptr = address[device];
+  }
+  // Nothing in the array has to start at zero: sample_partial writes every triple that
+  // sample_final reads, and what an earlier, larger call left behind them is never looked at.
+  sample_partial_kernel<<<dim3(rows, segments), kSampleThreads, 0, stream>>>(logits, temperature, scratch_ptr, vocab,
+                                                                             segments);
+  MLR_LAUNCH_CHECK();
+  sample_final_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, scratch_ptr, tokens, vocab,
                                                            segments);
   MLR_LAUNCH_CHECK();
   return 0;
