@@ -12,6 +12,7 @@ from .config import ConfigError, ModelConfig, Qwen2Config
 from .engine import (
     BatchingPolicy,
     ContinuousBatchEngine,
+    EngineConfig,
     EngineStepResult,
     ModelRunner,
     PagedBlockAdmissionController,
@@ -37,6 +38,7 @@ __all__ = [
     "CacheManager",
     "ConfigError",
     "ContinuousBatchEngine",
+    "EngineConfig",
     "DecoderModel",
     "EngineStepResult",
     "ModelConfig",

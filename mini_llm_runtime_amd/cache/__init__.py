@@ -1,7 +1,7 @@
 """Paged keys and values, block tables, and per-request state slots."""
 
 from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
-from .manager import CacheManager, CacheStats, KVGroup, RequestCache, StepLayout
+from .manager import CacheManager, CacheStats, KVGroup, RequestCache, StepLayout, VisibilityError
 from .spec import PagedKVSpec, SlotStateSpec
 
 __all__ = [
@@ -15,5 +15,6 @@ __all__ = [
     "SlotPool",
     "SlotStateSpec",
     "StepLayout",
+    "VisibilityError",
     "blocks_for",
 ]

@@ -197,6 +197,11 @@ class CacheStats:
     storage_bytes: int
 
 
+class VisibilityError(RuntimeError):
+    """A site read the step's pending tokens before they were written, or a step was
+    committed although a site that owns pages never wrote."""
+
+
 class CacheManager:
     def __init__(
         self,
@@ -207,6 +212,7 @@ class CacheManager:
         max_requests: int,
         dtype: torch.dtype,
         device: Union[str, torch.device] = "cuda",
+        check_visibility: bool = False,
     ) -> None:
         if block_size <= 0:
             raise ValueError("block_size must be > 0")
@@ -238,6 +244,13 @@ class CacheManager:
         self.slots = SlotPool(self.max_requests)
         self._requests: dict[str, RequestCache] = {}
         self._pending: Optional[list[_PendingEntry]] = None
+        # Debug check of what the reference's adapter enforces per layer
+        # (src/mini_llm_runtime/paged_kv_adapter.py:109-147, 168-178): pending tokens of a site
+        # may be read only after that site wrote them, and a step commits only when every
+        # site that owns pages has written.  Mixers report through `KVView.written()` /
+        # `KVView.reading()`; without the flag the reports cost nothing.
+        self.check_visibility = bool(check_visibility)
+        self._written_sites: set[int] = set()
 
     # ---- lookups ----------------------------------------------------------------
     @property
@@ -266,6 +279,30 @@ class CacheManager:
     @property
     def step_in_flight(self) -> bool:
         return self._pending is not None
+
+    # ---- visibility of pending tokens (debug) ------------------------------------------------
+    @property
+    def visibility_tracker(self) -> Optional["CacheManager"]:
+        """What a `KVView` reports to: this manager when the check is on, else None."""
+        return self if self.check_visibility else None
+
+    def note_write(self, site: int, owner: int) -> None:
+        if self._pending is None:
+            raise VisibilityError(f"site {site} wrote keys and values outside a step")
+        if site != owner:
+            raise VisibilityError(f"site {site} wrote into the pages of site {owner}, which it only reads")
+        self._written_sites.add(owner)
+
+    def note_read(self, site: int, owner: int) -> None:
+        if self._pending is None:
+            raise VisibilityError(f"site {site} read the cache outside a step")
+        if owner not in self._written_sites:
+            raise VisibilityError(
+                f"site {site} reads the step's pending tokens of site {owner} before they were written"
+            )
+
+    def _unwritten_sites(self) -> list[int]:
+        return [s for g in self.groups for s in g.sites if s not in self._written_sites]
 
     # ---- request lifetime ---------------------------------------------------------
     def create_request(self, request_id: str) -> RequestCache:
@@ -371,6 +408,7 @@ class CacheManager:
         for entry in pending:
             entry.request.pending_tokens = entry.num_new
         self._pending = pending
+        self._written_sites.clear()
         return self._layout(pending)
 
     def _rollback(self, pending: list[_PendingEntry]) -> None:
@@ -398,6 +436,10 @@ class CacheManager:
         """Make the step's tokens count; returns the window pages given back per request."""
         if self._pending is None:
             raise RuntimeError("no step in flight")
+        if self.check_visibility:
+            missing = self._unwritten_sites()
+            if missing:
+                raise VisibilityError(f"cannot commit: sites {missing} own pages and did not write this step's tokens")
         pending, self._pending = self._pending, None
         passed: dict[str, dict[int, tuple[int, ...]]] = {}
         for entry in pending:

@@ -10,8 +10,9 @@ its `experiments/continuous_batch_engine_runner.py:32-52` (`--model`, `--block-s
 `--local-files-only`, `--output-dir`) and runs the same kind of demonstration:
 requests that join and leave a running batch, with a record of every step.  The
 reference's `--prefill-attention-backend` and `--prefill-kv-write-backend` choose
-between its PyTorch code paths; this engine has one kernel path, so the options
-are accepted with their reference values and have no effect.
+between its PyTorch code paths; this engine has one kernel path and no such options.
+`--dtype` defaults to what the model folder's config.json says (`torch_dtype`); the page
+pool is `--num-blocks` pages or, without it, `--kv-memory-fraction` of the free device memory.
 
 Tokens in, tokens out: the engine has no tokenizer of its own (the reference's
 scripts borrow an external one).  `--prompt` is accepted when the model folder
@@ -31,7 +32,7 @@ from typing import Any, Optional, Sequence
 
 def _add_model_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--model", required=True, type=Path, help="folder with config.json and model.safetensors")
-    p.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    p.add_argument("--dtype", default=None, choices=("bfloat16", "float32"), help="default: config.json's torch_dtype")
     p.add_argument("--local-files-only", action="store_true", help="accepted for compatibility; models are always local")
 
 
@@ -59,13 +60,13 @@ def build_parser() -> argparse.ArgumentParser:
     e = sub.add_parser("engine", help="continuous batching over several requests")
     _add_model_options(e)
     e.add_argument("--block-size", type=int, default=16)
-    e.add_argument("--num-blocks", type=int, default=256)
+    e.add_argument("--num-blocks", type=int, default=None, help="pages of the cache pool")
+    e.add_argument("--kv-memory-fraction", type=float, default=0.8, help="share of free device memory for pages when --num-blocks is not given")
+    e.add_argument("--check-cache-visibility", action="store_true", help="debug: refuse reads of pending tokens before their write")
     e.add_argument("--max-running-requests", type=int, default=3)
     e.add_argument("--max-batch-tokens", type=int, default=64)
     e.add_argument("--max-mixed-prefill-tokens", type=int, default=None)
     e.add_argument("--batching-policy", choices=("continuous", "static"), default="continuous")
-    e.add_argument("--prefill-attention-backend", choices=("auto", "masked", "segmented_sdpa"), default="auto")
-    e.add_argument("--prefill-kv-write-backend", choices=("scalar", "vectorized"), default="vectorized")
     e.add_argument("--requests", type=Path, help='JSON list of {"id", "prompt_ids", "max_new_tokens", "arrival_step"}')
     e.add_argument("--num-requests", type=int, default=3, help="synthetic requests when --requests is not given")
     e.add_argument("--prompt-len", type=int, default=9)
@@ -94,7 +95,9 @@ def _tokenize(model_dir: Path, text: str) -> list[int]:
 
 
 def cmd_generate(args: argparse.Namespace) -> int:
-    from .engine.factory import default_ops, load_model, make_cache, parse_dtype
+    from .config.model_config import read_config_json
+    from .engine.config import EngineConfig
+    from .engine.factory import default_ops, load_model, make_cache
     from .engine.generation import generate
     from .engine.runner import ModelRunner
     from .sampling.sampler import GREEDY, SamplingParams
@@ -104,7 +107,7 @@ def cmd_generate(args: argparse.Namespace) -> int:
     if (args.prompt is None) == (args.prompt_ids is None):
         raise SystemExit("give exactly one of --prompt and --prompt-ids")
     prompt = args.prompt_ids if args.prompt_ids is not None else _tokenize(args.model, args.prompt)
-    dtype = parse_dtype(args.dtype)
+    dtype = EngineConfig(dtype=args.dtype).resolved_dtype(read_config_json(args.model))
     ops = default_ops(dtype, "cuda")
     _, model = load_model(args.model, dtype=dtype, device=ops.device)
     need = len(prompt) + args.max_new_tokens
@@ -149,19 +152,22 @@ def _record_step(result, manager) -> dict[str, Any]:
 def cmd_engine(args: argparse.Namespace) -> int:
     import torch
 
+    from .engine.config import EngineConfig
     from .engine.engine import ContinuousBatchEngine
     from .engine.scheduler import BatchingPolicy
 
-    engine = ContinuousBatchEngine.from_model_dir(
-        args.model,
+    config = EngineConfig(
         dtype=args.dtype,
         block_size=args.block_size,
         num_blocks=args.num_blocks,
+        kv_memory_fraction=args.kv_memory_fraction,
         max_running_requests=args.max_running_requests,
         max_batch_tokens=args.max_batch_tokens,
         max_mixed_prefill_tokens=args.max_mixed_prefill_tokens,
         batching_policy=BatchingPolicy(args.batching_policy),
+        check_cache_visibility=args.check_cache_visibility,
     )
+    engine = ContinuousBatchEngine.from_model_dir(args.model, config)
     vocab = engine.runner.vocab_size
     if args.requests is not None:
         requests = json.loads(args.requests.read_text())
@@ -211,8 +217,9 @@ def cmd_engine(args: argparse.Namespace) -> int:
         "schema_version": 1,
         "artifact": "continuous_batching_run",
         "model": str(args.model),
-        "dtype": args.dtype,
+        "dtype": str(engine.runner.dtype).replace("torch.", ""),
         "block_size": args.block_size,
+        "num_blocks": engine.manager.groups[0].num_blocks if engine.manager.groups else 0,
         "requests": requests,
         "steps": records,
         "generated_token_ids": tokens,
@@ -222,7 +229,7 @@ def cmd_engine(args: argparse.Namespace) -> int:
     if args.output_dir is not None:
         args.output_dir.mkdir(parents=True, exist_ok=True)
         (args.output_dir / "result.json").write_text(json.dumps(artifact, indent=2))
-        lines = ["# Continuous batching run", "", f"model: `{args.model}`, dtype {args.dtype}, block size {args.block_size}", ""]
+        lines = ["# Continuous batching run", "", f"model: `{args.model}`, dtype {artifact['dtype']}, block size {args.block_size}", ""]
         lines += ["| step | tokens | prefill | decode | finished |", "|---|---|---|---|---|"]
         lines += [f"| {r['step']} | {r['token_count']} | {r['prefill']} | {r['decode']} | {r['finished']} |" for r in records]
         lines += ["", "| request | generated |", "|---|---|"] + [f"| {rid} | {ids} |" for rid, ids in tokens.items()]

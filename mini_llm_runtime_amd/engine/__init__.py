@@ -1,6 +1,7 @@
 """Step function, scheduler, admission and the continuous-batching engine."""
 
 from .admission import BlockReservation, PagedBlockAdmissionController
+from .config import EngineConfig, GraphLimits
 from .engine import ContinuousBatchEngine, EngineStepResult
 from .factory import load_model, make_cache, parse_dtype
 from .generation import GenerationOutput, generate, greedy_generate
@@ -22,6 +23,8 @@ __all__ = [
     "BatchingPolicy",
     "BlockReservation",
     "ContinuousBatchEngine",
+    "EngineConfig",
+    "GraphLimits",
     "EngineStepResult",
     "FinishReason",
     "GenerationOutput",

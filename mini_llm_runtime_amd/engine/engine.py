@@ -26,6 +26,7 @@ those of the plain loop.
 from __future__ import annotations
 
 import time
+import warnings
 from contextlib import contextmanager
 from dataclasses import dataclass
 from pathlib import Path
@@ -35,6 +36,7 @@ import torch
 
 from ..sampling.sampler import GREEDY, Sampler, SamplingParams
 from .admission import PagedBlockAdmissionController
+from .config import EngineConfig
 from .metrics import RequestMetricsCollector
 from .runner import ModelRunner, StepEntry, StepOutput
 from .scheduler import (
@@ -142,6 +144,7 @@ class ContinuousBatchEngine:
         self.lookahead_hits = 0
         self.lookahead_misses = 0
         self.lookahead_error: Optional[Exception] = None  # what switched the lookahead off, if anything did
+        self.config: Optional[EngineConfig] = None  # set by from_model_dir
 
     @property
     def manager(self):
@@ -152,34 +155,62 @@ class ContinuousBatchEngine:
     def from_model_dir(
         cls,
         model_dir: Union[str, Path],
+        config: Optional[EngineConfig] = None,
         *,
-        dtype: Union[str, torch.dtype] = "bfloat16",
-        device: Union[str, torch.device] = "cuda",
-        block_size: int = 16,
-        num_blocks: int = 1024,
-        max_running_requests: int = 8,
-        max_batch_tokens: int = 2048,
-        max_mixed_prefill_tokens: Optional[int] = None,
-        batching_policy: BatchingPolicy = BatchingPolicy.CONTINUOUS,
         ops=None,
-        **kwargs,
+        **overrides,
     ) -> "ContinuousBatchEngine":
-        from .factory import default_ops, load_model, make_cache, parse_dtype
+        """Model folder -> engine, set up by an `EngineConfig` (keyword arguments replace
+        single fields of it).  `ops` replaces the HIP kernel library (tests on the CPU)."""
+        from ..models.registry import load_config
+        from ..config.model_config import read_config_json
+        from .factory import blocks_from_free_memory, default_ops, load_model, make_cache
 
-        dtype = parse_dtype(dtype)
-        ops = ops or default_ops(dtype, device)
+        config = (config or EngineConfig()).with_overrides(**overrides)
+        dtype = ops.dtype if ops is not None and config.dtype is None else config.resolved_dtype(read_config_json(model_dir))
+        ops = ops or default_ops(dtype, config.device, config.tuning)
+        load_config(model_dir)  # an unknown architecture fails before any weight is read
         _, model = load_model(model_dir, dtype=dtype, device=ops.device)
-        cache = make_cache(model, block_size=block_size, num_blocks=num_blocks, max_requests=max_running_requests)
-        runner = ModelRunner(model, cache, ops)
-        admission = PagedBlockAdmissionController(cache, max_step_tokens=max_batch_tokens)
-        scheduler = RequestScheduler(
-            max_running_requests=max_running_requests,
-            max_batch_tokens=max_batch_tokens,
-            max_mixed_prefill_tokens=max_mixed_prefill_tokens,
-            admission_callback=admission.try_admit,
-            batching_policy=batching_policy,
+        num_blocks = config.num_blocks
+        if num_blocks is None:
+            num_blocks = blocks_from_free_memory(
+                model, config.block_size, dtype, torch.device(ops.device), config.kv_memory_fraction
+            )
+        cache = make_cache(
+            model,
+            block_size=config.block_size,
+            num_blocks=num_blocks,
+            max_requests=config.max_running_requests,
+            check_visibility=config.check_cache_visibility,
         )
-        return cls(scheduler=scheduler, runner=runner, admission=admission, **kwargs)
+        limits = config.graphs
+        runner = ModelRunner(
+            model,
+            cache,
+            ops,
+            use_graphs=limits.enabled,
+            max_graph_batch=limits.max_decode_batch,
+            max_decode_graphs=limits.max_decode_graphs,
+            max_step_graphs=limits.max_step_graphs,
+            max_graph_tokens=limits.max_step_tokens,
+        )
+        admission = PagedBlockAdmissionController(cache, max_step_tokens=config.max_batch_tokens)
+        scheduler = RequestScheduler(
+            max_running_requests=config.max_running_requests,
+            max_batch_tokens=config.max_batch_tokens,
+            max_mixed_prefill_tokens=config.max_mixed_prefill_tokens,
+            admission_callback=admission.try_admit,
+            batching_policy=config.batching_policy,
+        )
+        engine = cls(
+            scheduler=scheduler,
+            runner=runner,
+            admission=admission,
+            enable_tracing=config.enable_tracing,
+            lookahead=config.lookahead,
+        )
+        engine.config = config
+        return engine
 
     # ---- requests ---------------------------------------------------------------------------------
     def submit(
@@ -199,6 +230,15 @@ class ContinuousBatchEngine:
             raise ValueError(f"prompt tokens outside the vocabulary of {vocab}: {bad[:5]}")
         if len(prompt_token_ids) + max_new_tokens - 1 > self.runner.max_positions:
             raise ValueError("prompt length + max_new_tokens - 1 exceeds max_position_embeddings")
+        # a request that no empty pool could hold would sit at the head of the queue for good,
+        # and everything behind it with it: it is refused here, before it is queued
+        lifetime = len(prompt_token_ids) + max_new_tokens - 1
+        if not self.manager.can_ever_hold(lifetime, self.admission.max_step_tokens):
+            need = self.manager.lifetime_blocks(lifetime, self.admission.max_step_tokens)
+            have = [g.num_blocks for g in self.manager.groups]
+            raise ValueError(
+                f"request {request_id!r} can never be admitted: it needs {need} pages per pool, the pools have {have}"
+            )
         sampling = GREEDY if temperature == 0.0 else SamplingParams(float(temperature), int(seed))
         request = self.scheduler.submit(
             request_id,
@@ -215,8 +255,12 @@ class ContinuousBatchEngine:
     def step(self) -> Optional[EngineStepResult]:
         """Schedule and run one step; None when nothing can run."""
         started_ns = self._clock_ns()
-        with _trace_range(self.enable_tracing, "scheduler.schedule_step"):
-            batch = self.scheduler.schedule_step()
+        try:
+            with _trace_range(self.enable_tracing, "scheduler.schedule_step"):
+                batch = self.scheduler.schedule_step()
+        except BaseException:
+            self._drop_ahead()  # whatever the scheduler refused, no launched step stays open
+            raise
         if batch is None:
             self._drop_ahead()
             return None
@@ -248,11 +292,11 @@ class ContinuousBatchEngine:
                 chosen = ahead.chosen
             else:
                 with _trace_range(self.enable_tracing, f"model.step:tokens={batch.token_count}"):
-                    output = self.runner.step(entries)
+                    output = self.runner.step(entries, borrow_logits=True)  # sampled from right below
                 chosen = None
                 if output.logits is not None:
                     chosen = _TokensOnTheWay(self.sampler.sample(output.logits, params, indices))
-        except Exception:
+        except BaseException:  # also an interrupt must not leave admitted requests and a batch behind
             self._drop_ahead()
             with _trace_range(self.enable_tracing, "engine.rollback"):
                 self.admission.release_admitted(batch.admitted_request_ids)
@@ -268,6 +312,12 @@ class ContinuousBatchEngine:
                 self._ahead = None
                 self.lookahead = False
                 self.lookahead_error = error
+                warnings.warn(
+                    f"decoding one step ahead was switched off after {type(error).__name__}: {error}; "
+                    "steps go on one by one, which is slower",
+                    RuntimeWarning,
+                    stacklevel=2,
+                )
         with _trace_range(self.enable_tracing, "token.d2h_sync"):
             host_tokens = chosen.wait() if chosen is not None else []
         tokens_ready_ns = self._clock_ns()

@@ -10,35 +10,20 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from ..cache.manager import CacheManager
+from ..cache.spec import PagedKVSpec
 from ..config.model_config import ModelConfig
 from ..models.registry import build_model, load_config
 from ..parts.model import DecoderModel
 from ..weights.loader import load_weights
 
-DTYPES = {
-    "bfloat16": torch.bfloat16,
-    "bf16": torch.bfloat16,
-    "float32": torch.float32,
-    "fp32": torch.float32,
-}
+from .config import blocks_for_memory, parse_dtype  # noqa: F401  (parse_dtype is part of this module's surface)
 
 
-def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
-    if isinstance(name, torch.dtype):
-        if name not in (torch.bfloat16, torch.float32):
-            raise ValueError("the engine's dtype is bfloat16 or float32")
-        return name
-    try:
-        return DTYPES[name]
-    except KeyError:
-        raise ValueError(f"unknown dtype {name!r}; use bfloat16 or float32") from None
-
-
-def default_ops(dtype: torch.dtype, device: Union[str, torch.device]) -> Any:
+def default_ops(dtype: torch.dtype, device: Union[str, torch.device], tuning: Any = None) -> Any:
     """The HIP kernel library; raises when it cannot be built or there is no GPU."""
     from ..kernels.ops import HipOps
 
-    return HipOps(dtype=dtype, device=device)
+    return HipOps(dtype=dtype, device=device, tuning=tuning)
 
 
 def load_model(
@@ -63,6 +48,7 @@ def make_cache(
     max_requests: int,
     dtype: Optional[torch.dtype] = None,
     device: Optional[Union[str, torch.device]] = None,
+    check_visibility: bool = False,
 ) -> CacheManager:
     return CacheManager(
         model.site_cache_specs(),
@@ -71,4 +57,29 @@ def make_cache(
         max_requests=max_requests,
         dtype=dtype or model.dtype,
         device=device or model.device,
+        check_visibility=check_visibility,
     )
+
+
+def page_bytes(model: DecoderModel, block_size: int, dtype: torch.dtype) -> int:
+    """Bytes one page id costs over all page pools of a model (every pool is given the same
+    number of pages): keys and values of every site that owns pages."""
+    width = torch.empty((), dtype=dtype).element_size()
+    total = 0
+    for spec in model.site_cache_specs():
+        if isinstance(spec, PagedKVSpec):
+            total += 2 * spec.num_kv_heads * spec.head_dim * block_size * width
+    return total
+
+
+def blocks_from_free_memory(
+    model: DecoderModel, block_size: int, dtype: torch.dtype, device: torch.device, fraction: float
+) -> int:
+    """Pages per pool that `fraction` of the device memory free right now holds."""
+    per_page = page_bytes(model, block_size, dtype)
+    if per_page == 0:
+        return 1  # a model without paged sites still gets a (never used) pool
+    if device.type != "cuda":
+        raise ValueError("kv_memory_fraction needs a GPU; give num_blocks instead")
+    free, _ = torch.cuda.mem_get_info(device)
+    return blocks_for_memory(per_page, free, fraction)

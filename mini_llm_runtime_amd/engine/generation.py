@@ -77,7 +77,7 @@ def generate(
     try:
         tokens = prompt
         for index in range(max_new_tokens):
-            out = runner.step([StepEntry.of(request_id, tokens, (len(tokens) - 1,))])
+            out = runner.step([StepEntry.of(request_id, tokens, (len(tokens) - 1,))], borrow_logits=True)
             if captured is not None:
                 captured.append(out.logits[0].clone())
             nxt = int(sampler.sample(out.logits, [sampling], [index]).cpu()[0])

@@ -43,12 +43,18 @@ class StepEntry:
 @dataclass
 class StepOutput:
     """logits: [K, vocab] float32 on the device (None when nothing was wanted), in the
-    order of the entries and of each entry's `want`; `rows[i]` = (request, index)."""
+    order of the entries and of each entry's `want`; `rows[i]` = (request, index).
+    They are the caller's to keep, unless the step was asked for with `borrow_logits=True`
+    (or launched with `launch_decode`): then they may be a view of a recorded step's output
+    buffer, which the next step of the same shape overwrites.
+    site_outputs: with `capture_sites=True`, [sites, K, hidden] float32: the residual stream
+    after every execution site at the wanted rows."""
 
     logits: Optional[torch.Tensor]
     rows: tuple[tuple[str, int], ...]
     layout: StepLayout
     passed_pages: dict = field(default_factory=dict)
+    site_outputs: Optional[torch.Tensor] = None
 
 
 def _pack_int32(arrays: Sequence[np.ndarray]) -> tuple[np.ndarray, list[tuple[int, tuple[int, ...]]]]:
@@ -73,6 +79,9 @@ class ModelRunner:
         *,
         use_graphs: bool = True,
         max_graph_batch: int = 256,
+        max_decode_graphs: int = 64,
+        max_step_graphs: int = 16,
+        max_graph_tokens: int = 8192,
     ) -> None:
         if model.embed_weight is None:
             raise ValueError("the model's parameters are not loaded")
@@ -92,16 +101,18 @@ class ModelRunner:
         # width) as a HIP graph and replayed: a decode step of a small model is hundreds of
         # short kernels, and launching them one by one from the host costs more than running them.
         # Only for models whose parts all say `replayable`.
-        self.use_graphs = bool(use_graphs) and self.device.type == "cuda"
+        # (a recording runs the parts' host code once, so their reports to the visibility check
+        # would be missing from every replay: the check runs unrecorded)
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and not cache.check_visibility
         self.max_graph_batch = int(max_graph_batch)
         self._graphs: dict[tuple[int, int], tuple] = {}
         self._staging: dict[tuple[int, int], list] = {}
         # Any other step (prompt portions, mixed batches) is recorded when its sizes come a second
         # time, and replayed from then on, if every part of the model allows it; a bounded number
         # of such recordings is kept, the least recently used one goes first.
-        self.max_step_graphs = 16
-        self.max_decode_graphs = 64
-        self.max_graph_tokens = 8192
+        self.max_step_graphs = int(max_step_graphs)
+        self.max_decode_graphs = int(max_decode_graphs)
+        self.max_graph_tokens = int(max_graph_tokens)
         self._step_graphs: dict[tuple, tuple] = {}
         self._step_seen: dict[tuple, int] = {}
 
@@ -204,6 +215,9 @@ class ModelRunner:
                     block_size=self.cache.block_size,
                     window=spec.window,
                     writable=source == site,
+                    site=site,
+                    owner=source,
+                    tracker=self.cache.visibility_tracker,
                 )
             elif isinstance(spec, SlotStateSpec):
                 ctx.state_views[site] = StateView(self.cache.state_banks[source].tensor, state_read, state_write)
@@ -217,7 +231,12 @@ class ModelRunner:
         return host, spans
 
     def _forward_eager(
-        self, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray, tiles: np.ndarray
+        self,
+        layout: StepLayout,
+        token_ids: np.ndarray,
+        logit_rows: np.ndarray,
+        tiles: np.ndarray,
+        site_outputs: Optional[list] = None,
     ) -> Optional[torch.Tensor]:
         single = layout.q_lens == 1
         host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, tiles))
@@ -234,7 +253,7 @@ class ModelRunner:
             num_decode_entries=int(single.sum()),
             max_decode_context=int(layout.context_lens[single].max()) if single.any() else 0,
         )
-        return self.model.forward(ctx, ctx.memo["logit_rows"] if logit_rows.size else None)
+        return self.model.forward(ctx, ctx.memo["logit_rows"] if logit_rows.size else None, site_outputs)
 
     # ---- steps of sizes seen before, as HIP graphs ----------------------------------------------------
     def _table_quantum(self) -> int:
@@ -484,7 +503,12 @@ class ModelRunner:
 
     # -------------------------------------------------------------------------------------------
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
+    def step(
+        self, entries: Sequence[StepEntry], *, borrow_logits: bool = False, capture_sites: bool = False
+    ) -> StepOutput:
+        """Run one batch.  borrow_logits: the caller uses the logits before the next step and
+        accepts a view of a recorded step's buffer (saves a copy).  capture_sites: also return
+        the residual stream after every site at the wanted rows (runs unrecorded)."""
         self._validate(entries)
         layout = self.cache.begin_step([(e.request_id, len(e.tokens)) for e in entries])
         try:
@@ -499,9 +523,15 @@ class ModelRunner:
             if self.fail_next_step is not None:
                 error, self.fail_next_step = self.fail_next_step, None
                 raise error
-            key = self._graph_key(layout)
+            captured: Optional[list] = [] if capture_sites else None
+            borrowed = False
+            key = None if capture_sites else self._graph_key(layout)
             if key is not None:
                 logits = self._forward_graph(key, layout, token_ids, logit_rows)
+                borrowed = True
+            elif capture_sites:
+                tiles = query_tiles(layout.q_lens, layout.q_starts)
+                logits = self._forward_eager(layout, token_ids, logit_rows, tiles, captured)
             else:
                 tiles = query_tiles(layout.q_lens, layout.q_starts)
                 step_key = self._step_key(layout, logit_rows, tiles)
@@ -512,10 +542,14 @@ class ModelRunner:
                         self._step_seen.clear()
                 if seen >= 2:
                     logits = self._forward_recorded(step_key, layout, token_ids, logit_rows, tiles)
+                    borrowed = True
                 else:
                     logits = self._forward_eager(layout, token_ids, logit_rows, tiles)
+            if borrowed and not borrow_logits and logits is not None:
+                logits = logits.clone()
         except BaseException:
             self.cache.abort_step()
             raise
         passed = self.cache.commit_step()
-        return StepOutput(logits=logits, rows=tuple(rows), layout=layout, passed_pages=passed)
+        sites = torch.stack(captured) if captured else None
+        return StepOutput(logits=logits, rows=tuple(rows), layout=layout, passed_pages=passed, site_outputs=sites)

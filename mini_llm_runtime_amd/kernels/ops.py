@@ -13,12 +13,12 @@ a memory fault on the GPU.
 from __future__ import annotations
 
 import ctypes
-import os
 from typing import Any, Optional, Sequence, Union
 
 import torch
 
 from . import build
+from .tuning import KernelTuning
 
 _VP = ctypes.c_void_p
 _I = ctypes.c_int
@@ -92,8 +92,14 @@ def load_library(module: build.Module = build.CORE) -> ctypes.CDLL:
 
 
 class HipOps:
-    def __init__(self, dtype: torch.dtype = torch.bfloat16, device: Union[str, torch.device] = "cuda") -> None:
+    def __init__(
+        self,
+        dtype: torch.dtype = torch.bfloat16,
+        device: Union[str, torch.device] = "cuda",
+        tuning: Optional[KernelTuning] = None,
+    ) -> None:
         self.dtype = dtype
+        self.tuning = tuning or KernelTuning()
         self.code = _dtype_code(dtype)
         device = torch.device(device)
         if device.type != "cuda":
@@ -109,9 +115,9 @@ class HipOps:
         if self.lib.mlr_version() != 1:
             raise KernelError("the built kernel library is of another version than this package")
         self._attention_libs: dict[int, ctypes.CDLL] = {}
-        self.decode_partition = int(os.environ.get("MLR_DECODE_PARTITION", "256"))
-        self.max_k_slices = int(os.environ.get("MLR_MAX_K_SLICES", "16"))
-        self.decode_max_groups = int(os.environ.get("MLR_DECODE_MAX_GROUPS", "1024"))
+        self.decode_partition = self.tuning.decode_partition
+        self.max_k_slices = self.tuning.max_k_slices
+        self.decode_max_groups = self.tuning.decode_max_groups
 
     def attention_library(self, head_dim: int) -> ctypes.CDLL:
         """The MFMA attention kernels of one head size, compiled on first use."""

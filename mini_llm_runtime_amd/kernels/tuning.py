@@ -1,0 +1,21 @@
+"""Knobs of the kernel library's launch heuristics.  Tests and measurements change them
+through `HipOps(..., tuning=...)`; the defaults are what the measurements chose."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass(frozen=True)
+class KernelTuning:
+    decode_partition: int = 256  # keys per split of the decode attention
+    decode_max_groups: int = 1024  # cap on the decode attention's workgroups
+    max_k_slices: int = 16  # most partial sums a narrow product may be cut into
+    fuse_norm: bool = True  # norm (+ residual) as the prologue of the product behind it, for few tokens
+    fuse_merge: bool = True  # merge of the decode attention's splits as the prologue of the output product
+
+    def __post_init__(self) -> None:
+        for name in ("decode_partition", "decode_max_groups", "max_k_slices"):
+            value = getattr(self, name)
+            if isinstance(value, bool) or not isinstance(value, int) or value <= 0:
+                raise ValueError(f"KernelTuning.{name} must be a positive integer")

@@ -118,6 +118,9 @@ class GQAAttention(Mixer):
             qkv = ops.qkv_rope_write(
                 h, self.qkv_weight, self.qkv_bias_vec, rotation, cache.slot_mapping, cache.key, cache.value, **pages
             )
+        if cache.writable:
+            cache.written()
+        cache.reading()
         attended = ops.paged_attention(
             qkv,
             cache.key,

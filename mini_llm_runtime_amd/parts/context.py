@@ -38,6 +38,21 @@ class KVView:
     block_size: int
     window: Optional[int]
     writable: bool  # False when the site reads another site's cache
+    site: int = -1  # the execution site this view was made for
+    owner: int = -1  # the site that owns the pages (== site when writable)
+    tracker: Any = None  # the cache manager's visibility check, when it is switched on
+
+    def written(self) -> None:
+        """The mixer reports that it has stored the step's keys and values of this site."""
+        if self.tracker is not None:
+            self.tracker.note_write(self.site, self.owner)
+
+    def reading(self) -> None:
+        """The mixer reports that it is about to read this site's pages, the step's own
+        tokens included.  With the check switched on this raises unless the owning site
+        has written them."""
+        if self.tracker is not None:
+            self.tracker.note_read(self.site, self.owner)
 
 
 @dataclass

@@ -119,13 +119,32 @@ class DecoderModel:
         return sum(seen.values())
 
     # ---- compute ----------------------------------------------------------------------
-    def forward(self, ctx: StepContext, logit_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
-        """Run the step's tokens through all sites; logits [K, vocab] float32 at `logit_rows`."""
+    def forward(
+        self,
+        ctx: StepContext,
+        logit_rows: Optional[torch.Tensor],
+        site_outputs: Optional[list] = None,
+    ) -> Optional[torch.Tensor]:
+        """Run the step's tokens through all sites; logits [K, vocab] float32 at `logit_rows`.
+
+        site_outputs: a list that receives, after every site, the float32 residual stream at
+        `logit_rows` ([K, hidden]): what the reference's `return_layer_outputs` captures
+        after each layer (src/mini_llm_runtime/qwen_model_runner.py:266-281).  A tool for
+        finding the layer at which a wrong logit first appears; it adds a few small kernels
+        per site and is never recorded into a graph."""
         ops = ctx.ops
         x = ops.embedding(self.embed_weight, ctx.token_ids)
         delta: Optional[torch.Tensor] = None
+        capture = site_outputs is not None and logit_rows is not None and logit_rows.numel() > 0
         for site, entry in enumerate(self.spec.order):
             x, delta = self.layers[entry.layer].forward(ctx, x, delta, site)
+            if capture:
+                # the site's own output is not added into the stream yet: add it here, in 32-bit
+                rows = ops.gather_rows(x, logit_rows)
+                if delta is not None:
+                    own = ops.gather_rows(delta, logit_rows)
+                    rows = rows + (own.sum(0) if own.dim() == 3 else own.float())
+                site_outputs.append(rows)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         if ctx.logits_for_all:

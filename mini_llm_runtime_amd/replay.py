@@ -4,6 +4,7 @@ cache manager and kernels, the ones generation uses; it has no forward pass,
 cache or loader of its own.
 
     bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+                  [--block-size 16] [--max-live 8] [--layers]
 
 Steps come on standard input, one JSON object a line:
 
@@ -12,7 +13,9 @@ Steps come on standard input, one JSON object a line:
 All entries of a step are one batch.  For a step in which something is wanted,
 `<out>/<step>.f32` receives the logits at the wanted places, in the order of the
 entries and of `want`, as little-endian float32 [wanted, vocab].  After every step
-a line `done <step>` is printed and flushed.
+a line `done <step>` is printed and flushed.  With `--layers`, `<out>/<step>.layers.f32`
+also receives the residual stream after every execution site at the same places, float32
+[sites, wanted, hidden]: where a wrong logit first appears.
 
 The reference's nearest tools capture per-step logits of one request
 (src/mini_llm_runtime/generation.py:84-94, `return_step_logits`) and snapshot block
@@ -28,9 +31,9 @@ from pathlib import Path
 from typing import Any, Optional, Sequence, TextIO
 
 
-PAGE_TOKENS = 16  # tokens per page of the replay pool
-ROUNDING = 64  # the caller counts every request's tokens rounded up to this
-MAX_LIVE = 8
+PAGE_TOKENS = 16  # default tokens per page of the replay pool
+ROUNDING = 64  # the caller counts every request's tokens rounded up to this (or to a larger page)
+MAX_LIVE = 8  # default number of request slots
 
 
 def parse_args(argv: Optional[Sequence[str]] = None) -> argparse.Namespace:
@@ -39,6 +42,9 @@ def parse_args(argv: Optional[Sequence[str]] = None) -> argparse.Namespace:
     p.add_argument("--dtype", required=True, choices=("bfloat16", "float32"))
     p.add_argument("--out", required=True, type=Path, help="folder for <step>.f32 files")
     p.add_argument("--max-tokens", required=True, type=int, help="most tokens live requests hold at any time")
+    p.add_argument("--block-size", type=int, default=PAGE_TOKENS, help="tokens per page of the cache pool")
+    p.add_argument("--max-live", type=int, default=MAX_LIVE, help="most requests that are live at one time")
+    p.add_argument("--layers", action="store_true", help="also write <step>.layers.f32: the stream after every site")
     return p.parse_args(argv)
 
 
@@ -66,7 +72,7 @@ def _parse_step(line: str) -> dict[str, Any]:
     return step
 
 
-def replay(runner, cache, lines: TextIO, out_dir: Path, done: TextIO) -> int:
+def replay(runner, cache, lines: TextIO, out_dir: Path, done: TextIO, layers: bool = False) -> int:
     """Run every step read from `lines`; returns the number of steps."""
     from .engine.runner import StepEntry
 
@@ -84,14 +90,23 @@ def replay(runner, cache, lines: TextIO, out_dir: Path, done: TextIO) -> int:
             for e in step["entries"]:
                 rid = str(e["id"])
                 if not cache.has_request(rid):
+                    if cache.slots.free_count == 0:
+                        raise TraceError(
+                            f"step {index}: request {rid!r} would be live request number "
+                            f"{cache.max_requests + 1}; --max-live is {cache.max_requests}"
+                        )
                     cache.create_request(rid)
                     created.append(rid)
                 entries.append(StepEntry.of(rid, e["tokens"], e["want"]))
             if entries:
-                result = runner.step(entries)
+                result = runner.step(entries, borrow_logits=True, capture_sites=layers)  # copied out right here
                 if result.logits is not None:
                     rows = result.logits.float().cpu().numpy().astype("<f4", copy=False)
                     rows.tofile(out_dir / f"{index}.f32")
+                if result.site_outputs is not None:
+                    result.site_outputs.float().cpu().numpy().astype("<f4", copy=False).tofile(
+                        out_dir / f"{index}.layers.f32"
+                    )
         except Exception:
             for rid in created:
                 cache.release_request(rid)
@@ -107,8 +122,8 @@ def replay(runner, cache, lines: TextIO, out_dir: Path, done: TextIO) -> int:
 
 def main(argv: Optional[Sequence[str]] = None) -> int:
     args = parse_args(argv)
-    if args.max_tokens <= 0:
-        print("trace_run: --max-tokens must be > 0", file=sys.stderr)
+    if args.max_tokens <= 0 or args.block_size <= 0 or args.max_live <= 0:
+        print("trace_run: --max-tokens, --block-size and --max-live must be > 0", file=sys.stderr)
         return 2
     import torch
 
@@ -120,11 +135,12 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     device = torch.device("cuda", 0)
     ops = default_ops(dtype, device)
     _, model = load_model(args.model, dtype=dtype, device=device)
-    pages = -(-args.max_tokens // PAGE_TOKENS)
-    cache = make_cache(model, block_size=PAGE_TOKENS, num_blocks=pages, max_requests=MAX_LIVE)
+    # the caller rounds every request up to max(64, page) tokens, so whole pages always suffice
+    pages = -(-args.max_tokens // args.block_size)
+    cache = make_cache(model, block_size=args.block_size, num_blocks=pages, max_requests=args.max_live)
     runner = ModelRunner(model, cache, ops)
     try:
-        replay(runner, cache, sys.stdin, args.out, sys.stdout)
+        replay(runner, cache, sys.stdin, args.out, sys.stdout, layers=args.layers)
     except Exception as e:  # a bad trace or a failed step ends the run with a message
         print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr)
         return 1

@@ -10,6 +10,7 @@ spec, 0.02).  The reference has random weights only in its tests
 
 from __future__ import annotations
 
+import json
 import zlib
 from pathlib import Path
 from typing import Iterator, Union
@@ -74,7 +75,12 @@ def write_random_model(
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     model = build_model(config)
-    config.save(folder)
+    path = config.save(folder)
+    # the stored element type, under the key checkpoints carry it in: an engine that is not told a
+    # dtype computes in this one
+    data = json.loads(path.read_text(encoding="utf-8"))
+    data["torch_dtype"] = storage_dtype
+    path.write_text(json.dumps(data, indent=2) + "\n", encoding="utf-8")
     layout, stream = random_checkpoint_tensors(model, seed, _STORAGE[storage_dtype])
     write_safetensors(
         folder / "model.safetensors",

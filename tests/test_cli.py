@@ -23,11 +23,11 @@ def test_option_names_follow_the_reference():
     g = p.parse_args(["generate", "--model", "m", "--prompt-ids", "1,2 3", "--max-new-tokens", "4", "--local-files-only"])
     assert g.prompt_ids == [1, 2, 3] and g.max_new_tokens == 4 and g.temperature == 0.0 and g.local_files_only
     assert p.parse_args(["generate", "--model", "m", "--prompt", "hi"]).max_new_tokens == 8  # the reference's default
-    e = p.parse_args(["engine", "--model", "m", "--block-size", "4", "--prefill-attention-backend", "segmented_sdpa",
-                      "--prefill-kv-write-backend", "scalar", "--output-dir", "out"])
+    e = p.parse_args(["engine", "--model", "m", "--block-size", "4", "--output-dir", "out"])
     assert e.block_size == 4 and e.output_dir == Path("out") and e.batching_policy == "continuous"
-    with pytest.raises(SystemExit):
-        p.parse_args(["engine", "--model", "m", "--prefill-attention-backend", "flash"])
+    assert e.dtype is None and e.num_blocks is None and e.kv_memory_fraction == 0.8  # the model folder and free memory decide
+    with pytest.raises(SystemExit):  # the reference's choice between its PyTorch paths has nothing to choose here
+        p.parse_args(["engine", "--model", "m", "--prefill-attention-backend", "segmented_sdpa"])
     with pytest.raises(SystemExit):
         p.parse_args(["generate", "--prompt-ids", "1"])  # --model is required
 

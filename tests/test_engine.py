@@ -180,9 +180,10 @@ def test_pages_run_out_requests_wait_then_enter(tmp_path, backend, dtype):
     enter_late = next(i for i, (p, _) in enumerate(order) if p == ("late",))
     assert enter_late == done_big + 1  # the step after the pages came back
     _check_greedy(engine.scheduler.get_request("late").generated_token_ids, p2, w, cfg, dtype)
-    engine.submit("never", random_tokens(20, cfg["vocab_size"], 3), max_new_tokens=8)  # 27 tokens -> 7 pages > 6
+    # 27 tokens -> 7 pages > 6: refused when it is submitted, so it never blocks the queue
     with pytest.raises(ValueError, match="never"):
-        engine.step()
+        engine.submit("never", random_tokens(20, cfg["vocab_size"], 3), max_new_tokens=8)
+    assert "never" not in engine.scheduler.waiting_request_ids and engine.step() is None
 
 
 @pytest.mark.parametrize("backend,dtype", CASES[:2])

@@ -137,10 +137,12 @@ def test_shift_of_all_positions_changes_nothing(tmp_path):
     torch.testing.assert_close(plain.forward(toks, w, cfg, position_offset=37), plain.forward(toks, w, cfg), atol=1e-9, rtol=0)
 
 
-def test_reference_tiny_fixture_shapes_run():
+def _reference_fixture():
     """The reference's own tiny fixture (tests/test_qwen_weights.py:9-65): vocab 5, hidden 4,
-    2 layers, 2 heads / 1 KV head, head_dim 2; weights from torch.randn with seed 7."""
-    cfg = dict(vocab_size=5, hidden_size=4, intermediate_size=6, num_hidden_layers=2, num_attention_heads=2,
+    2 layers, 2 heads / 1 KV head, head_dim 2; weights from torch.randn with seed 7, drawn in
+    the order of its `tiny_state_dict`."""
+    cfg = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2",
+               vocab_size=5, hidden_size=4, intermediate_size=6, num_hidden_layers=2, num_attention_heads=2,
                num_key_value_heads=1, max_position_embeddings=8, rms_norm_eps=1e-6, rope_theta=10000.0,
                hidden_act="silu", tie_word_embeddings=True)
     g = torch.Generator().manual_seed(7)
@@ -155,8 +157,41 @@ def test_reference_tiny_fixture_shapes_run():
                   p + "self_attn.v_proj.weight": r(2, 4), p + "self_attn.v_proj.bias": r(2),
                   p + "self_attn.o_proj.weight": r(4, 4), p + "mlp.gate_proj.weight": r(6, 4),
                   p + "mlp.up_proj.weight": r(6, 4), p + "mlp.down_proj.weight": r(4, 6)})
-    logits = plain.forward([1, 4, 2, 0], w, cfg)
-    assert logits.shape == (4, 5) and torch.isfinite(logits).all()
-    # cached-vs-recomputed equivalence is what the reference tests on this fixture
-    # (tests/test_generation.py:31-52); the plain greedy is that recompute-everything loop
-    assert len(plain.greedy([1, 4], w, cfg, 3)) == 3
+    return cfg, w
+
+
+@pytest.mark.parametrize("backend", ["double", pytest.param("hip", marks=pytest.mark.gpu)])
+def test_reference_tiny_fixture_cached_equals_recomputed(tmp_path, backend):
+    """What the reference asserts on this fixture (tests/test_generation.py:31-52): generation
+    from the cache gives the tokens AND the per-step logits (atol 1e-5) of the loop that
+    recomputes everything, with its counts (3 new tokens: 3 prompt tokens, 2 decode steps, 5
+    cached).  Here the cached side is the engine (32-bit), the other the plain implementation."""
+    import json
+
+    import mini_llm_runtime_amd as mlr
+    from kernel_doubles import TorchOps
+    from mini_llm_runtime_amd.engine import ModelRunner
+    from mini_llm_runtime_amd.weights.safetensors_io import write_safetensors
+
+    cfg, w = _reference_fixture()
+    folder = tmp_path / "fixture"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    write_safetensors(folder / "model.safetensors", [(n, t.dtype, tuple(t.shape)) for n, t in w.items()], iter(w.items()))
+    if backend == "double":
+        ops = TorchOps(torch.float32, "cpu")
+    else:
+        from mini_llm_runtime_amd.kernels.ops import HipOps
+
+        ops = HipOps(torch.float32, "cuda")
+    _, model = mlr.load_model(folder, dtype=torch.float32, device=ops.device)
+    cache = mlr.make_cache(model, block_size=2, num_blocks=4, max_requests=1)
+    out = mlr.greedy_generate(ModelRunner(model, cache, ops), [1, 2, 3], max_new_tokens=3, return_step_logits=True)
+    seq, expected = [1, 2, 3], []
+    for i in range(3):
+        logits = plain.forward(seq, w, cfg)[-1]
+        assert float((out.step_logits[i].double().cpu() - logits).abs().max()) < 1e-5, f"step {i}"
+        expected.append(int(torch.argmax(logits)))
+        seq.append(expected[-1])
+    assert list(out.generated_token_ids) == expected == plain.greedy([1, 2, 3], w, cfg, 3)
+    assert (out.prefill_tokens, out.decode_steps, out.cache_length, out.stopped_by_eos) == (3, 2, 5, False)

@@ -22,6 +22,7 @@ LENGTHS = {"A": (5, 17, 33, 70, 41, 52), "B": (1, 9, 24, 40, 63, 37), "C": (3, 6
 # mantissa (2^-9 relative per rounding); the error is judged relative to the size
 # of the logits.
 FP32_MAX_ABS = 1e-4
+BF16_ROW_REL_L2 = 5e-2  # of any single row
 BF16_REL_L2 = 2e-2
 
 
@@ -67,9 +68,10 @@ def _requests(which: str) -> dict[str, list[int]]:
     return {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[which])}
 
 
-def _compare(got, requests, weights, cfg, dtype):
+def _compare(got, requests, weights, cfg, dtype, row_bound=None):
     assert got, "no logits came back"
     worst_abs = 0.0
+    worst_row = (0.0, None)
     num = 0.0
     den = 0.0
     for rid, toks in requests.items():
@@ -79,13 +81,18 @@ def _compare(got, requests, weights, cfg, dtype):
             assert torch.isfinite(row).all(), f"{rid}:{pos} is not finite"
             diff = row - ref[pos]
             worst_abs = max(worst_abs, float(diff.abs().max()))
-            num += float((diff**2).sum())
-            den += float((ref[pos] ** 2).sum())
+            row_num, row_den = float((diff**2).sum()), float((ref[pos] ** 2).sum())
+            worst_row = max(worst_row, ((row_num / row_den) ** 0.5, (rid, pos)))
+            num += row_num
+            den += row_den
     rel = (num / den) ** 0.5
     if dtype == torch.float32:
         assert worst_abs < FP32_MAX_ABS, f"max abs error {worst_abs:.3e}, rel L2 {rel:.3e}"
     else:
+        # all rows together, and every single row: one wrong position among hundreds must not
+        # hide in the aggregate
         assert rel < BF16_REL_L2, f"rel L2 error {rel:.3e}, max abs {worst_abs:.3e}"
+        assert worst_row[0] < (row_bound or BF16_ROW_REL_L2), f"row {worst_row[1]}: rel L2 error {worst_row[0]:.3e}"
 
 
 FAMILIES = {
@@ -121,7 +128,7 @@ def test_schedule_matches_plain(tmp_path, which, family, backend, dtype):
 
 
 @pytest.mark.parametrize("backend,dtype", CASES)
-@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_peaked_attention_mixed(tmp_path, which, backend, dtype):
     """Same as the mixed family, with query/key projections scaled up so that single
     keys dominate: a key read from a wrong slot or page changes the logits visibly."""
@@ -129,21 +136,31 @@ def test_peaked_attention_mixed(tmp_path, which, backend, dtype):
     steps = schedules.mixed(requests, seed=5)
     cfg, weights, cache, runner = _setup(tmp_path, which, backend, dtype, steps, sharp=12.0)
     got = schedules.run_schedule(runner, cache, steps)
-    _compare(got, requests, weights, cfg, dtype)
+    # Scores this large carry the bfloat16 rounding of q and k (2^-9 of a score of several
+    # dozen) into the softmax, so a single row may be off by more than elsewhere; a key taken
+    # from a wrong slot changes a row by its whole size (rel L2 near 1).
+    _compare(got, requests, weights, cfg, dtype, row_bound=0.2)
 
 
-@pytest.mark.parametrize("backend,dtype", CASES[:2])
-def test_schedules_agree_with_each_other(tmp_path, backend, dtype):
-    """In 32-bit the families agree with each other far below the plain-implementation bound."""
-    requests = _requests("B")
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+def test_schedules_agree_with_each_other(tmp_path, which, backend, dtype):
+    """The families agree with each other: in 32-bit far below the plain-implementation
+    bound; in bfloat16 every single row within what the different kernels of prompt portions
+    and single tokens round differently."""
+    requests = _requests(which)
     results = []
     for family in FAMILIES.values():
         steps = family(requests)
-        _, _, cache, runner = _setup(tmp_path, "B", backend, dtype, steps)
+        _, _, cache, runner = _setup(tmp_path, which, backend, dtype, steps)
         results.append(schedules.run_schedule(runner, cache, steps))
     for other in results[1:]:
         for key, row in results[0].items():
-            assert torch.allclose(row, other[key], atol=2e-5, rtol=0), key
+            if dtype == torch.float32:
+                assert torch.allclose(row, other[key], atol=2e-5, rtol=0), key
+            else:
+                rel = float((row - other[key]).norm() / row.norm())
+                assert rel < BF16_ROW_REL_L2, (key, rel)
 
 
 @pytest.mark.gpu
@@ -269,6 +286,8 @@ def test_half_billion_layer_sizes_match_plain(tmp_path, dtype):
     for requests, steps in (
         (long, schedules.whole(long)),
         (long, schedules.bulk_then_tail(long)),
+        (short, schedules.bulk_then_tail(short)),
+        (short, schedules.portions(short)),
         (short, schedules.mixed(short, seed=3)),
     ):
         got = schedules.run_schedule(runner, cache, steps)
@@ -277,27 +296,49 @@ def test_half_billion_layer_sizes_match_plain(tmp_path, dtype):
     assert cache.request_ids == ()
 
 
-@pytest.mark.gpu
-def test_seven_billion_layer_sizes_match_plain(tmp_path):
-    """One layer of the Qwen2.5-7B sizes (width 3584, 28 query and 4 key/value heads of 128,
-    feed-forward 18944; a small vocabulary keeps the plain implementation quick), bfloat16: the
-    largest tiles and the 128-wide heads inside the model."""
+def _one_layer_of(tmp_path, preset, dtype, seed, lengths):
+    """One layer of a large configuration's sizes with a small vocabulary (which keeps the plain
+    implementation quick): a long prompt whole, shorter ones in portions down to two tokens, with
+    their last tokens one by one, and mixed."""
     from mini_llm_runtime_amd.config.presets import load_preset
     from mini_llm_runtime_amd.kernels.ops import HipOps
     from mini_llm_runtime_amd.models.registry import config_from_dict
     from mini_llm_runtime_amd.weights import write_random_model
 
-    data = load_preset("qwen2.5-7b")
+    data = load_preset(preset)
     data["num_hidden_layers"] = 1
     data["vocab_size"] = 4099
     config = config_from_dict(data)
-    model_dir = write_random_model(config, tmp_path / "seven", seed=22, storage_dtype="bfloat16")
+    model_dir = write_random_model(config, tmp_path / "large", seed=seed, storage_dtype="bfloat16")
     cfg, weights = read_weights(model_dir)
-    long = {"w": random_tokens(700, cfg["vocab_size"], 720)}
-    short = {f"s{i}": random_tokens(n, cfg["vocab_size"], 730 + i) for i, n in enumerate((90, 40))}
-    _, _, cache, runner = make_runner(model_dir, HipOps(torch.bfloat16, "cuda"), block_size=16, num_blocks=64, max_requests=4)
+    long = {"w": random_tokens(lengths[0], cfg["vocab_size"], 720)}
+    short = {f"s{i}": random_tokens(n, cfg["vocab_size"], 730 + i) for i, n in enumerate(lengths[1:])}
+    _, _, cache, runner = make_runner(model_dir, HipOps(dtype, "cuda"), block_size=16, num_blocks=64, max_requests=4)
     cache.poison()
-    for requests, steps in ((long, schedules.whole(long)), (short, schedules.mixed(short, seed=4))):
+    for requests, steps in (
+        (long, schedules.whole(long)),
+        (short, schedules.portions(short)),
+        (short, schedules.bulk_then_tail(short, tail=12)),
+        (short, schedules.mixed(short, seed=4)),
+    ):
         got = schedules.run_schedule(runner, cache, steps)
-        _compare(got, requests, weights, cfg, torch.bfloat16)
+        _compare(got, requests, weights, cfg, dtype)
     cache.check_invariants()
+    assert cache.request_ids == ()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_seven_billion_layer_sizes_match_plain(tmp_path, dtype):
+    """Qwen2.5-7B sizes (width 3584, 28 query and 4 key/value heads of 128, feed-forward 18944):
+    the largest tiles and the 128-wide heads inside the model."""
+    lengths = (700, 90, 40) if dtype == torch.bfloat16 else (300, 70, 40)
+    _one_layer_of(tmp_path, "qwen2.5-7b", dtype, 22, lengths)
+
+
+@pytest.mark.gpu
+def test_thirty_two_billion_layer_sizes_match_plain(tmp_path):
+    """Qwen2.5-32B sizes (width 5120, 40 query and 8 key/value heads of 128: groups of five;
+    feed-forward 27648), bfloat16: 256 x 256 tiles over 55,296 and 27,648 features, a K of 27,648
+    cut into slices, decode attention with a group that does not fill its tile."""
+    _one_layer_of(tmp_path, "qwen2.5-32b", torch.bfloat16, 23, (600, 90, 40))

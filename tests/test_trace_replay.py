@@ -31,13 +31,13 @@ def _requests(which):
     return {f"q{i}": random_tokens(n, vocab, 300 + i) for i, n in enumerate(LENGTHS[which])}
 
 
-def _max_tokens(steps):
+def _max_tokens(steps, rounding=64):
     """Most tokens live requests hold at any time, each request's count rounded up to 64."""
     fed, most = {}, 0
     for step in steps:
         for e in step["entries"]:
             fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
-        most = max(most, sum(-(-n // 64) * 64 for n in fed.values()))
+        most = max(most, sum(-(-n // rounding) * rounding for n in fed.values()))
         for rid in step["end"]:
             fed.pop(rid, None)
     return most
@@ -62,18 +62,20 @@ def _collect(steps, out_dir, vocab):
 
 
 def _compare(got, requests, weights, cfg, dtype):
-    num = den = worst = 0.0
+    num = den = worst = worst_row = 0.0
     for rid, toks in requests.items():
         ref = plain.forward(toks, weights, cfg)
         for pos in range(len(toks)):
             diff = got[(rid, pos)].double() - ref[pos]
             worst = max(worst, float(diff.abs().max()))
+            worst_row = max(worst_row, float(diff.norm() / ref[pos].norm()))
             num += float((diff**2).sum())
             den += float((ref[pos] ** 2).sum())
     if dtype == "float32":
         assert worst < 1e-4, worst
     else:
         assert (num / den) ** 0.5 < 2e-2, (num / den) ** 0.5
+        assert worst_row < 5e-2, worst_row  # no single position may hide in the aggregate
 
 
 FAMILIES = {
@@ -133,3 +135,88 @@ def test_trace_run_program(tmp_path, gpu_device, which, dtype):
         assert proc.returncode == 0, proc.stderr[-2000:]
         assert proc.stdout.split() == [x for s in steps for x in ("done", str(s["step"]))]
         _compare(_collect(steps, out, cfg["vocab_size"]), requests, w, cfg, dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("block_size", [8, 32, 128])
+def test_trace_run_program_at_other_page_sizes(tmp_path, gpu_device, block_size, dtype):
+    """The program itself (not only the step function) with pages of 8, 32 and 128 tokens; a
+    page larger than 64 tokens is what the caller rounds every request up to."""
+    d = make_model_dir(tmp_path, "B", seed=34)
+    cfg, w = read_weights(d)
+    requests = _requests("B")
+    for family in ("portions", "mixed"):
+        steps = FAMILIES[family](requests)
+        out = tmp_path / f"out_{family}"
+        proc = subprocess.run(
+            [str(ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", dtype, "--out", str(out),
+             "--max-tokens", str(_max_tokens(steps, max(64, block_size))), "--block-size", str(block_size)],
+            input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300,
+        )
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        _compare(_collect(steps, out, cfg["vocab_size"]), requests, w, cfg, dtype)
+
+
+def _site_reference(toks, w, cfg):
+    x = w["model.embed_tokens.weight"].double()[torch.tensor(toks)]
+    wd = {k: v.double() for k, v in w.items()}
+    out = []
+    for i in range(cfg["num_hidden_layers"]):
+        x = plain.decoder_layer(x, torch.arange(len(toks)), wd, i, cfg)
+        out.append(x)
+    return torch.stack(out)
+
+
+def test_replay_writes_the_stream_after_every_site(tmp_path):
+    """`--layers`: <step>.layers.f32 holds [sites, wanted, hidden], the plain layers' outputs."""
+    d = make_model_dir(tmp_path, "A", seed=35)
+    cfg, w = read_weights(d)
+    toks = random_tokens(21, cfg["vocab_size"], 36)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks[:13], "want": [0, 12]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks[13:20], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks[20:], "want": [0]}], "end": ["a"]},
+    ]
+    _, model = mlr.load_model(d, dtype=torch.float32, device="cpu")
+    cache = mlr.make_cache(model, block_size=PAGE_TOKENS, num_blocks=2, max_requests=1)
+    lines = io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n")
+    replay(ModelRunner(model, cache, TorchOps(torch.float32)), cache, lines, tmp_path / "o", io.StringIO(), layers=True)
+    ref = _site_reference(toks, w, cfg)
+    layers, hidden = cfg["num_hidden_layers"], cfg["hidden_size"]
+    first = torch.from_numpy(np.fromfile(tmp_path / "o" / "0.layers.f32", dtype="<f4").reshape(layers, 2, hidden).copy())
+    assert float((first.double() - ref[:, [0, 12]]).abs().max()) < 1e-5
+    assert not (tmp_path / "o" / "1.layers.f32").exists() and not (tmp_path / "o" / "1.f32").exists()
+    last = torch.from_numpy(np.fromfile(tmp_path / "o" / "2.layers.f32", dtype="<f4").reshape(layers, 1, hidden).copy())
+    assert float((last.double() - ref[:, [20]]).abs().max()) < 1e-5
+
+
+def test_replay_names_the_limit_on_live_requests(tmp_path):
+    d = make_model_dir(tmp_path, "A", seed=37)
+    _, model = mlr.load_model(d, dtype=torch.float32, device="cpu")
+    cache = mlr.make_cache(model, block_size=PAGE_TOKENS, num_blocks=8, max_requests=2)
+    runner = ModelRunner(model, cache, TorchOps(torch.float32))
+    steps = [{"step": i, "entries": [{"id": f"r{i}", "tokens": [1, 2], "want": []}], "end": []} for i in range(3)]
+    with pytest.raises(TraceError, match="--max-live is 2"):
+        replay(runner, cache, io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n"), tmp_path / "o", io.StringIO())
+    assert set(cache.request_ids) == {"r0", "r1"}  # the steps before the refused one stand
+
+
+@pytest.mark.gpu
+def test_trace_run_program_writes_layers(tmp_path, gpu_device):
+    d = make_model_dir(tmp_path, "B", seed=38)
+    cfg, w = read_weights(d)
+    toks = random_tokens(40, cfg["vocab_size"], 39)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks[:33], "want": [32]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks[33:], "want": [0, 6]}], "end": ["a"]},
+    ]
+    proc = subprocess.run(
+        [str(ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32", "--out", str(tmp_path / "o"),
+         "--max-tokens", "64", "--layers"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    ref = _site_reference(toks, w, cfg)
+    got = np.fromfile(tmp_path / "o" / "1.layers.f32", dtype="<f4").reshape(cfg["num_hidden_layers"], 2, cfg["hidden_size"])
+    assert float((torch.from_numpy(got.copy()).double() - ref[:, [33, 39]]).abs().max()) < 1e-4
