@@ -10,7 +10,18 @@ timed steps between device synchronisations.  One JSON line is printed:
 `value` is decoded tokens per second at batch 8; `points` holds batch 1 and 64;
 `prefill` is one 2,048-token prompt; `roofline` prices the decode step by the
 bytes it must read (every weight once and the live requests' cache) against
-8 TB/s.  Peaks are MI355X's published dense figures.
+8 TB/s.  Peaks are MI355X's published dense figures.  `points_7b` and `points_32b`
+(default run only; `--no-large` leaves them out) hold decode at batch 8 and the
+prefill for the two larger shapes, with the number of layers run and of the full
+model beside them.
+
+How it measures (the reference's harness rules, src/mini_llm_runtime/timing.py:49-82,
+141-160 and environment.py:37-93): untimed warm-up first; the timed steps between
+device synchronisations; the whole timed region also between two device events
+(`ms_per_step_device`); every step's host time kept as a raw sample (`samples_ms`,
+`median_ms`, `p10_ms`, `p90_ms`; with decoding one step ahead a sample is the time between
+two steps' tokens reaching the host); `env` records versions, device, commit and whether the
+tree was dirty.  Nothing that compiles or records a graph is timed.
 
 Two further workloads print a JSON line of their own (`--workload`):
 `burst`: 64 requests arrive at once, prompt lengths uniform in [128, 2048], 32/64/128/256 new
@@ -50,6 +61,8 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked"))
+    p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
+    p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
     return p.parse_args()
 
 
@@ -225,132 +238,193 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
     }
 
 
-def main() -> int:
-    args = parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
-        return 2
+def environment() -> dict:
+    """What the numbers were measured on (src/mini_llm_runtime/environment.py:37-93 of the
+    reference records the same kinds of facts)."""
+    import platform
+    import subprocess
 
     import torch
 
-    sys.path.insert(0, str(Path(__file__).resolve().parent))
-    import mini_llm_runtime_amd  # noqa: F401
-    from mini_llm_runtime_amd.config.presets import load_preset
-    from mini_llm_runtime_amd.engine.factory import default_ops, load_model, make_cache, parse_dtype
-    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
-    from mini_llm_runtime_amd.engine.runner import ModelRunner, StepEntry
-    from mini_llm_runtime_amd.models.registry import config_from_dict
-    from mini_llm_runtime_amd.sampling.sampler import Sampler
-    from mini_llm_runtime_amd.weights.random_init import write_random_model
+    root = Path(__file__).resolve().parent
 
-    data = load_preset(args.config)
-    full_layers = int(data["num_hidden_layers"])
-    if args.layers is not None:
-        data["num_hidden_layers"] = int(args.layers)
-    config = config_from_dict(data)
-    dtype = parse_dtype(args.dtype)
-    short = "bf16" if dtype == torch.bfloat16 else "fp32"
-    device = torch.device("cuda", 0)
-    ops = default_ops(dtype, device)
+    def git(*args: str) -> str:
+        try:
+            return subprocess.run(["git", *args], cwd=root, capture_output=True, text=True, timeout=10).stdout.strip()
+        except (OSError, subprocess.SubprocessError):
+            return ""
 
-    with tempfile.TemporaryDirectory(prefix="mlr_bench_") as tmp:
-        folder = write_random_model(config, tmp, seed=args.seed, storage_dtype="bfloat16")
-        _, model = load_model(folder, dtype=dtype, device=device)
+    props = torch.cuda.get_device_properties(0)
+    return {
+        "python": platform.python_version(),
+        "torch": torch.__version__,
+        "hip": torch.version.hip,
+        "device": props.name,
+        "arch": getattr(props, "gcnArchName", ""),
+        "compute_units": props.multi_processor_count,
+        "memory_gb": round(props.total_memory / 2**30, 1),
+        "commit": git("rev-parse", "--short", "HEAD") or None,
+        "dirty": bool(git("status", "--porcelain", "--untracked-files=no")) if git("rev-parse", "HEAD") else None,
+    }
 
-    if args.workload != "decode":
-        line = (burst if args.workload == "burst" else chunked)(args, config, full_layers, model, ops, device)
-        print(json.dumps(line), flush=True)
-        return 0
 
-    batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
-    steps_total = args.warmup + args.steps
-    capacity = max(CONTEXT_LEN, args.prompt_len + steps_total + max(batches) + 9)
-    pages = max(batches) * (-(-capacity // BLOCK_SIZE)) + 8
-    cache = make_cache(model, block_size=BLOCK_SIZE, num_blocks=pages, max_requests=max(batches))
-    runner = ModelRunner(model, cache, ops)
-    sampler = Sampler(ops, device)
-    vocab = config.vocab_size
-    gen = torch.Generator().manual_seed(args.seed)
+def summary(samples_ms: list, keep: bool) -> dict:
+    ordered = sorted(samples_ms)
+    n = len(ordered)
+    out = {
+        "count": n,
+        "median_ms": round(ordered[n // 2], 4),
+        "p10_ms": round(ordered[n // 10], 4),
+        "p90_ms": round(ordered[min(n - 1, (9 * n) // 10)], 4),
+        "min_ms": round(ordered[0], 4),
+        "max_ms": round(ordered[-1], 4),
+    }
+    if keep:
+        out["samples_ms"] = [round(x, 4) for x in samples_ms]
+    return out
 
-    def prompt() -> list[int]:
-        return torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
 
-    def sync() -> None:
-        torch.cuda.synchronize(device)
+class Bench:
+    """One model shape with random weights on the device, and the measurements on it."""
 
-    def decode(batch: int, warmup: int, steps: int) -> float:
-        """ms per decode step of the continuous-batching engine at this batch size, contexts
-        starting at prompt_len: scheduler, step function, sampling on the GPU, tokens to the host."""
-        admission = PagedBlockAdmissionController(cache, max_step_tokens=args.prompt_len)
+    def __init__(self, args, name: str, layers, batches: list):
+        import torch
+
+        from mini_llm_runtime_amd.config.presets import load_preset
+        from mini_llm_runtime_amd.engine.factory import default_ops, make_cache, parse_dtype
+        from mini_llm_runtime_amd.engine.runner import ModelRunner
+        from mini_llm_runtime_amd.models.registry import build_model, config_from_dict
+        from mini_llm_runtime_amd.sampling.sampler import Sampler
+        from mini_llm_runtime_amd.weights.random_init import bind_random_weights
+
+        self.args = args
+        self.name = name
+        data = load_preset(name)
+        self.full_layers = int(data["num_hidden_layers"])
+        if layers is not None:
+            data["num_hidden_layers"] = int(layers)
+        self.config = config_from_dict(data)
+        self.dtype = parse_dtype(args.dtype)
+        self.short = "bf16" if self.dtype == torch.bfloat16 else "fp32"
+        self.device = torch.device("cuda", 0)
+        self.ops = default_ops(self.dtype, self.device)
+        self.model = build_model(self.config)
+        bind_random_weights(self.model, seed=args.seed, dtype=self.dtype, device=self.device)
+        self.batches = batches
+        steps_total = args.warmup + args.steps
+        capacity = max(CONTEXT_LEN, args.prompt_len + steps_total + max(batches) + 9)
+        pages = max(batches) * (-(-capacity // BLOCK_SIZE)) + 8
+        self.cache = make_cache(self.model, block_size=BLOCK_SIZE, num_blocks=pages, max_requests=max(batches))
+        self.runner = ModelRunner(self.model, self.cache, self.ops)
+        self.sampler = Sampler(self.ops, self.device)
+        self.gen = torch.Generator().manual_seed(args.seed)
+
+    def prompt(self) -> list:
+        import torch
+
+        return torch.randint(0, self.config.vocab_size, (self.args.prompt_len,), generator=self.gen).tolist()
+
+    def sync(self) -> None:
+        import torch
+
+        torch.cuda.synchronize(self.device)
+
+    def decode(self, batch: int, warmup: int, steps: int) -> dict:
+        """Decode steps of the continuous-batching engine at this batch size, contexts starting at
+        prompt_len: scheduler, step function, sampling on the GPU, tokens to the host."""
+        import torch
+
+        from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
+
+        args = self.args
+        admission = PagedBlockAdmissionController(self.cache, max_step_tokens=args.prompt_len)
         scheduler = RequestScheduler(
             max_running_requests=batch,
             max_batch_tokens=max(args.prompt_len, batch),
             admission_callback=admission.try_admit,
         )
-        engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
+        engine = ContinuousBatchEngine(
+            scheduler=scheduler, runner=self.runner, admission=admission, sampler=self.sampler
+        )
         for i in range(batch):
-            engine.submit(f"b{batch}-{i}", prompt(), max_new_tokens=warmup + steps + batch + 8)
+            engine.submit(f"b{batch}-{i}", self.prompt(), max_new_tokens=warmup + steps + batch + 8)
         while True:  # prompts, until a step is nothing but one token for every request
             result = engine.step()
             if len(result.batch.decode_request_ids) == batch:
                 break
         for _ in range(warmup):
             engine.step()
-        sync()
-        t0 = time.perf_counter()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        samples = []
+        self.sync()
+        begin.record()
+        t0 = last = time.perf_counter()
         for _ in range(steps):
             result = engine.step()
-        sync()
+            now = time.perf_counter()
+            samples.append((now - last) * 1e3)
+            last = now
+        end.record()
+        self.sync()
         elapsed = time.perf_counter() - t0
         assert len(result.batch.decode_request_ids) == batch and len(result.update.emitted_tokens) == batch
         engine.run_until_done()
-        return elapsed * 1e3 / steps
+        return {
+            "ms": elapsed * 1e3 / steps,
+            "ms_device": begin.elapsed_time(end) / steps,
+            "samples": samples,
+        }
 
-    from mini_llm_runtime_amd.sampling.sampler import GREEDY as _GREEDY
+    def kv_bytes_per_token(self) -> int:
+        return sum(
+            2 * len(g.sites) * g.spec.num_kv_heads * g.spec.head_dim * g.key.element_size() for g in self.cache.groups
+        )
 
-    ms_main = decode(args.batch, args.warmup, args.steps)
-    value = args.batch * 1e3 / ms_main
-    points = {}
-    for b in batches[1:]:
-        ms = decode(b, max(2, args.warmup // 2), max(8, args.steps // 2))
-        points[f"decode_b{b}"] = round(b * 1e3 / ms, 1)
+    def decode_bytes(self, batch: int, mean_context: float) -> tuple:
+        """Bytes a decode step has to read: every weight it uses once, and the live requests' cache."""
+        model, config = self.model, self.config
+        weight_bytes = model.weight_bytes()
+        if not config.tie_word_embeddings:  # an untied input table is only gathered from
+            weight_bytes -= model.embed_weight.numel() * model.embed_weight.element_size()
+        return weight_bytes, weight_bytes + batch * mean_context * self.kv_bytes_per_token()
 
-    # ---- what a decode step has to read ------------------------------------------------------
-    weight_bytes = model.weight_bytes()
-    embed_bytes = model.embed_weight.numel() * model.embed_weight.element_size()
-    if not config.tie_word_embeddings:
-        weight_bytes -= embed_bytes  # an untied input table is only gathered from
-    kv_per_token = sum(
-        2 * len(g.sites) * g.spec.num_kv_heads * g.spec.head_dim * g.key.element_size() for g in cache.groups
-    )
-    mean_context = args.prompt_len + args.warmup + args.steps / 2
-    step_bytes = weight_bytes + args.batch * mean_context * kv_per_token
-    achieved = step_bytes / (ms_main * 1e-3)
-    roofline = {
-        "bound": "hbm",
-        "achieved": round(achieved / 1e9, 1),
-        "peak": HBM_BYTES_PER_S / 1e9,
-        "unit": "GB/s",
-        "frac": round(achieved / HBM_BYTES_PER_S, 4),
-    }
+    def roofline(self, batch: int, ms: float, warmup: int, steps: int) -> dict:
+        _, step_bytes = self.decode_bytes(batch, self.args.prompt_len + warmup + steps / 2)
+        achieved = step_bytes / (ms * 1e-3)
+        return {
+            "bound": "hbm",
+            "achieved": round(achieved / 1e9, 1),
+            "peak": HBM_BYTES_PER_S / 1e9,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_BYTES_PER_S, 4),
+        }
 
-    # ---- prefill of one prompt ----------------------------------------------------------------
-    prefill = None
-    if not args.no_prefill:
-        tokens = args.prompt_len
-        times = []
-        for i in range(5):
+    def prefill(self, repeats: int = 5) -> dict:
+        """One prompt of prompt_len tokens through the step function, its last logits sampled."""
+        import torch
+
+        from mini_llm_runtime_amd.engine.runner import StepEntry
+        from mini_llm_runtime_amd.sampling.sampler import GREEDY
+
+        config, tokens = self.config, self.args.prompt_len
+        host, dev = [], []
+        for i in range(repeats + 1):  # the first run is the warm-up
             rid = f"p{i}"
-            cache.create_request(rid)
-            entry = [StepEntry.of(rid, prompt(), (tokens - 1,))]
-            sync()
+            self.cache.create_request(rid)
+            entry = [StepEntry.of(rid, self.prompt(), (tokens - 1,))]
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            self.sync()
+            begin.record()
             t0 = time.perf_counter()
-            out = runner.step(entry)
-            sampler.sample(out.logits, [_GREEDY], [0]).cpu()
-            sync()
-            times.append(time.perf_counter() - t0)
-            cache.release_request(rid)
-        ms = sorted(times[1:])[len(times[1:]) // 2] * 1e3
+            out = self.runner.step(entry, borrow_logits=True)
+            self.sampler.sample(out.logits, [GREEDY], [0]).cpu()
+            end.record()
+            self.sync()
+            host.append((time.perf_counter() - t0) * 1e3)
+            dev.append(begin.elapsed_time(end))
+            self.cache.release_request(rid)
+        host, dev = host[1:], dev[1:]
+        ms = sorted(host)[len(host) // 2]
         d = config.head_dim
         per_layer = (
             config.hidden_size * (config.num_attention_heads + 2 * config.num_key_value_heads) * d
@@ -362,26 +436,96 @@ def main() -> int:
             + config.num_hidden_layers * config.num_attention_heads * 4 * d * tokens * (tokens + 1) // 2
             + 2 * config.vocab_size * config.hidden_size
         )
-        prefill = {
+        return {
             "value": round(tokens * 1e3 / ms, 1),
             "tokens": tokens,
             "ms": round(ms, 3),
-            "frac": round(flops / (ms * 1e-3) / PEAK_FLOPS[short], 4),
+            "frac": round(flops / (ms * 1e-3) / PEAK_FLOPS[self.short], 4),
+            "ms_device": round(sorted(dev)[len(dev) // 2], 3),
+            "samples_ms": [round(x, 3) for x in host],
         }
+
+    def close(self) -> None:
+        import gc
+
+        import torch
+
+        for name in ("runner", "cache", "model", "sampler"):
+            setattr(self, name, None)
+        gc.collect()
+        torch.cuda.empty_cache()
+
+
+def large_point(args, name: str, layers: int) -> dict:
+    """Decode at batch 8 and the prefill for a larger shape, `layers` of its layers."""
+    bench = Bench(args, name, layers, [8])
+    try:
+        warmup, steps = max(2, args.warmup // 2), max(8, args.steps // 2)
+        run = bench.decode(8, warmup, steps)
+        point = {
+            "layers": bench.config.num_hidden_layers,
+            "layers_full_model": bench.full_layers,
+            "decode_b8": round(8e3 / run["ms"], 1),
+            "decode_b8_ms": round(run["ms"], 4),
+            "decode_b8_ms_device": round(run["ms_device"], 4),
+            "decode_b8_hbm_frac": bench.roofline(8, run["ms"], warmup, steps)["frac"],
+        }
+        if not args.no_prefill:
+            pre = bench.prefill(repeats=3)
+            point.update(prefill=pre["value"], prefill_ms=pre["ms"], prefill_frac=pre["frac"])
+        return point
+    finally:
+        bench.close()
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
+        return 2
+
+    sys.path.insert(0, str(Path(__file__).resolve().parent))
+    import mini_llm_runtime_amd  # noqa: F401
+
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
+    bench = Bench(args, args.config, args.layers, batches)
+    config = bench.config
+
+    if args.workload != "decode":
+        work = burst if args.workload == "burst" else chunked
+        bench.runner = bench.cache = None  # these workloads size a cache of their own
+        line = work(args, config, bench.full_layers, bench.model, bench.ops, bench.device)
+        line["env"] = environment()
+        print(json.dumps(line), flush=True)
+        return 0
+
+    main_run = bench.decode(args.batch, args.warmup, args.steps)
+    ms_main = main_run["ms"]
+    points = {}
+    for b in batches[1:]:
+        run = bench.decode(b, max(2, args.warmup // 2), max(8, args.steps // 2))
+        points[f"decode_b{b}"] = round(b * 1e3 / run["ms"], 1)
+    weight_bytes, _ = bench.decode_bytes(args.batch, 0)
+    roofline = bench.roofline(args.batch, ms_main, args.warmup, args.steps)
+    prefill = None if args.no_prefill else bench.prefill()
+    kv_per_token = bench.kv_bytes_per_token()
+    full_layers = bench.full_layers
+    bench.close()
 
     line = {
         "metric": "decode tokens/s",
-        "value": round(value, 1),
+        "value": round(args.batch * 1e3 / ms_main, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_main, 4),
+        "ms_per_step_device": round(main_run["ms_device"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": short,
-        "data": "synthetic (random weights, uniform random token ids)",
+        "dtype": bench.short,
+        "data": "synthetic (random weights made on the device, uniform random token ids)",
         "config": {
             "model": f"{args.config} shape",
             "global_batch": args.batch,
@@ -404,7 +548,12 @@ def main() -> int:
         "prefill": prefill,
         "roofline": roofline,
         "points": points,
+        "step_samples": summary(main_run["samples"], args.samples),
     }
+    if not args.no_large and args.config == "qwen2.5-0.5b" and args.layers is None and args.dtype == "bfloat16":
+        line["points_7b"] = large_point(args, "qwen2.5-7b", 28)
+        line["points_32b"] = large_point(args, "qwen2.5-32b", 16)
+    line["env"] = environment()
     print(json.dumps(line), flush=True)
     return 0
 

@@ -82,6 +82,30 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
                             int write, int kernel, hipStream_t stream);
 
+// Products of up to 16 tokens that make their own activations (gemm_fused.hip).
+// Norm prologue: h = RMSNorm(x_in + delta) * norm_weight with the delta a bfloat16 [m, k]
+// tensor, or `slices_in` float32 partial sums [slices_in, m, k] added in order, or nothing;
+// x_out (another buffer than x_in; null when nothing is added) receives x_in + delta.  Then
+// y = h w^T with the epilogues of mlr_gemm_bf16 (bias, float32 output, SwiGLU), or the
+// query/key/value epilogue of mlr_qkv_rope_write_bf16.  k a multiple of 8, at most 2048.
+// row_blocks: 0 chooses how many blocks of 16 features a workgroup owns, or 1, 2.
+int mlr_gemm_norm_fused_bf16(const float* x_in, float* x_out, const void* delta, const float* partial, int slices_in,
+                             const void* norm_weight, int norm_weight_is_f32, float eps, const void* w,
+                             const void* bias, int bias_is_f32, void* y, int out_is_f32, int swiglu, int row_blocks,
+                             int m, int n, int k, hipStream_t stream);
+int mlr_qkv_norm_fused_bf16(const float* x_in, float* x_out, const void* delta, const float* partial, int slices_in,
+                            const void* norm_weight, int norm_weight_is_f32, float eps, const void* w,
+                            const void* bias, int bias_is_f32, const float* cos, const float* sin, const int* slots,
+                            void* key_pages, void* value_pages, void* q_out, int m, int k, int heads, int kv_heads,
+                            int head_dim, int block_size, int num_pages, int write, hipStream_t stream);
+// Merge prologue: the activations are the decode attention's output of m single-token entries,
+// merged here from its unmerged partitions (`attn_partial`, as mlr_attention_decode with
+// merge 0 leaves them; part, splits, window as given there).  y = attended w^T (+ bias), k =
+// heads * head_dim; with slices > 1 y is float32 [slices, m, n] partial sums.
+int mlr_gemm_merge_fused_bf16(const float* attn_partial, const int* context_lens, int heads, int head_dim, int window,
+                              int part, int splits, const void* w, const void* bias, int bias_is_f32, void* y,
+                              int out_is_f32, int slices, int m, int n, hipStream_t stream);
+
 // Attention of every token over its request's pages: token t (entry
 // token_entry[t], absolute position positions[t]) sees the keys
 // max(0, p - window + 1) .. p of its entry's block table row (window 0: all).

@@ -753,11 +753,14 @@ int64_t mlr_attention_decode_scratch(int entries, int heads, int splits) {
 // Attention of every single-token entry (entries with more tokens are skipped).
 // Keys of an entry are cut into `splits` partitions of `part` positions (a
 // multiple of 64); with more than one partition `partial` must hold
-// mlr_attention_decode_scratch floats.
+// mlr_attention_decode_scratch floats, laid out [entry, head, split, head size + 2]
+// (numerator, maximum in base 2, denominator).  `merge` 0 leaves the partitions unmerged in
+// `partial` for a consumer that merges them itself (or for mlr_attention_decode_merge).
 int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
                          const int* block_table, int table_width, const int* cu_q, const int* context_lens,
                          void* out, float* partial, int entries, int heads, int kv_heads, int block_size,
-                         int num_pages, float scale, int window, int part, int splits, hipStream_t stream) {
+                         int num_pages, float scale, int window, int part, int splits, int merge,
+                         hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
   MLR_REQUIRE(block_size > 0 && block_size % 4 == 0, "block_size must be a multiple of 4");
@@ -799,11 +802,24 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   if (!launched) MLR_DECODE(1);
 #undef MLR_DECODE
   MLR_LAUNCH_CHECK();
-  if (splits > 1) {
+  if (splits > 1 && merge) {
     attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(
         partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, part, splits);
     MLR_LAUNCH_CHECK();
   }
+  return 0;
+}
+
+// The merge that mlr_attention_decode left out: out[t] of every single-token entry from its
+// partitions in `partial`.
+int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int* context_lens, void* out, int entries,
+                               int heads, int window, int part, int splits, hipStream_t stream) {
+  MLR_REQUIRE(partial && cu_q && context_lens && out, "null pointer");
+  MLR_REQUIRE(entries > 0 && heads > 0 && heads <= 65535, "bad sizes");
+  MLR_REQUIRE(part > 0 && part % 64 == 0 && splits > 1 && window >= 0, "bad partitions");
+  attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, context_lens,
+                                                                      static_cast<bf16*>(out), heads, window, part, splits);
+  MLR_LAUNCH_CHECK();
   return 0;
 }
 

@@ -51,7 +51,7 @@ class Module:
     name: str
     sources: tuple[str, ...]
     defines: tuple[str, ...] = field(default_factory=tuple)
-    headers: tuple[str, ...] = ("api.h", "common.h", "mfma.h")  # what the sources include: part of the stamp
+    headers: tuple[str, ...] = ("api.h", "common.h", "mfma.h", "gemm_epilogue.h")  # what the sources include: part of the stamp
 
 
 CORE = Module(
@@ -60,6 +60,7 @@ CORE = Module(
         "elementwise.hip",
         "gemm_simple.hip",
         "gemm_mfma.hip",
+        "gemm_fused.hip",
         "attention_simple.hip",
         "sampling.hip",
     ),

@@ -18,6 +18,7 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from . import build
+from .pending import PendingMerge, PendingNorm
 from .tuning import KernelTuning
 
 _VP = ctypes.c_void_p
@@ -41,6 +42,15 @@ _SIGNATURES = {
         [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
         _I,
     ),
+    "mlr_gemm_norm_fused_bf16": (
+        [_VP, _VP, _VP, _VP, _I, _VP, _I, _F, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP],
+        _I,
+    ),
+    "mlr_qkv_norm_fused_bf16": (
+        [_VP, _VP, _VP, _VP, _I, _VP, _I, _F, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        _I,
+    ),
+    "mlr_gemm_merge_fused_bf16": ([_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
         _I,
@@ -51,9 +61,10 @@ _SIGNATURES = {
     "mlr_attention_key_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
     "mlr_attention_decode": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _VP],
         _I,
     ),
+    "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_attention_prefill": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
         _I,
@@ -240,6 +251,60 @@ class HipOps:
         )
         return out
 
+    # ---- activations made inside the product that uses them ------------------------------------
+    FUSED_TOKENS = 16  # the merge prologue takes up to this many tokens
+    FUSED_NORM_TOKENS = 4  # the norm prologue up to this many (a wavefront per row)
+    FUSED_NORM_WIDTH = 2048  # and rows up to this width
+    FUSED_LDS_BYTES = 140 * 1024
+
+    def defer_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor]):
+        """The norm of `rmsnorm` as a `PendingNorm` when the product behind it could compute it
+        in its own kernel (bfloat16, few tokens, a narrow model); else None."""
+        if not (self.tuning.fuse_norm and self.dtype == torch.bfloat16 and x.dim() == 2):
+            return None
+        rows, hidden = x.shape
+        if rows > self.FUSED_NORM_TOKENS or hidden > self.FUSED_NORM_WIDTH or hidden % 8:
+            return None
+        slices = delta.shape[0] if delta is not None and delta.dim() == 3 else 0
+        if (1 + slices) * rows * hidden * 4 > self.tuning.fuse_bytes:  # every workgroup reads all of it
+            return None
+        return PendingNorm(x, delta, weight, float(eps))
+
+    def settle(self, h):
+        """The tensor behind a pending activation (run by a kernel of its own); tensors pass."""
+        if isinstance(h, PendingNorm):
+            if h.value is None:
+                h.value = self.rmsnorm(h.x, h.weight, h.eps, delta=h.delta)
+                h.residual = h.x
+            return h.value
+        if isinstance(h, PendingMerge):
+            out = self._empty((h.tokens, h.heads * h.head_dim), self.dtype)
+            self._call(
+                "mlr_attention_decode_merge", self._ptr(h.partial), self._ptr(h.cu_q), self._ptr(h.context_lens),
+                self._ptr(out), h.tokens, h.heads, h.window, h.part, h.splits, self._stream(), lib=h.library,
+            )
+            return out
+        return h
+
+    def _norm_arguments(self, h: PendingNorm):
+        """(checked tensors, ctypes arguments) of a norm prologue; allocates the updated stream."""
+        x = self._check(h.x, "residual stream", torch.float32, (None, None))
+        rows, hidden = x.shape
+        self._check(h.weight, "norm weight", (torch.float32, self.dtype), (hidden,))
+        plain = partial = None
+        slices = 0
+        if h.delta is not None and h.delta.dim() == 3:
+            partial = self._check(h.delta, "partial sums", torch.float32, (None, rows, hidden))
+            slices = partial.shape[0]
+        elif h.delta is not None:
+            plain = self._check(h.delta, "residual delta", self.dtype, (rows, hidden))
+        x_out = self._empty((rows, hidden), torch.float32) if h.delta is not None else None
+        args = (
+            self._ptr(x), self._ptr(x_out), self._ptr(plain), self._ptr(partial), slices, self._ptr(h.weight),
+            int(h.weight.dtype == torch.float32), float(h.eps),
+        )
+        return x_out if x_out is not None else x, args
+
     # ---- matrix products ----------------------------------------------------------------------
     def linear(
         self,
@@ -268,6 +333,11 @@ class HipOps:
         """
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
+        if isinstance(x, (PendingNorm, PendingMerge)):
+            fused = self._linear_fused(x, weight, bias, out_dtype, kernel, swiglu, partial_sums, mfma_kernel, slices)
+            if fused is not None:
+                return fused
+            x = self.settle(x)
         self._check(x, "linear input", self.dtype, (None, None))
         m, k = x.shape
         self._check(weight, "linear weight", self.dtype, (None, k))
@@ -302,6 +372,53 @@ class HipOps:
         self._call(
             "mlr_gemm_simple", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
             int(out_dtype == torch.float32), int(swiglu), self.code, m, n, k, self._stream(),
+        )
+        return y
+
+    def _linear_fused(self, x, weight, bias, out_dtype, kernel, swiglu, partial_sums, mfma_kernel, slices):
+        """`linear` on a pending activation in one kernel, or None when that cannot be."""
+        m, k = x.shape
+        if kernel != "auto" or mfma_kernel or self.dtype != torch.bfloat16 or k % 8 or m > self.FUSED_TOKENS:
+            return None
+        self._check(weight, "linear weight", self.dtype, (None, k))
+        n = weight.shape[0]
+        if bias is not None:
+            self._check(bias, "linear bias", (torch.float32, self.dtype), (n,))
+        if swiglu and (n % 4 or bias is not None):
+            raise KernelError("a SwiGLU product needs a multiple of 4 rows and no bias")
+        out_dtype = out_dtype or self.dtype
+        bias_f32 = int(bias is not None and bias.dtype == torch.float32)
+        if isinstance(x, PendingNorm):
+            if x.value is not None or slices not in (None, 1) or m > self.FUSED_NORM_TOKENS:
+                return None
+            # no K slices here: every workgroup needs whole rows for the norm's statistics
+            residual, norm_args = self._norm_arguments(x)
+            y = self._empty((m, n // 2 if swiglu else n), out_dtype)
+            self._call(
+                "mlr_gemm_norm_fused_bf16", *norm_args, self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
+                int(out_dtype == torch.float32), int(swiglu), 0, m, n, k, self._stream(),
+            )
+            x.residual = residual
+            return y
+        if swiglu or not self.tuning.fuse_merge:
+            return None
+        if slices is None:
+            slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices) if partial_sums else 1
+        elif slices > 1 and not partial_sums:
+            raise KernelError("k slices need partial_sums")
+        per_slice = -(-(-(-k // 32)) // slices) * 32  # columns of a slice, in whole MFMA steps
+        if m * (per_slice // 8) > 256 or m * (per_slice + 8) * 2 > self.FUSED_LDS_BYTES:
+            return None  # a thread merges one chunk of 8 columns
+        if m * per_slice * x.splits * 4 > self.tuning.fuse_bytes:  # what every workgroup reads to merge
+            return None
+        if slices > 1:
+            y = self._empty((slices, m, n), torch.float32)
+        else:
+            y = self._empty((m, n), out_dtype)
+        self._call(
+            "mlr_gemm_merge_fused_bf16", self._ptr(x.partial), self._ptr(x.context_lens), x.heads, x.head_dim, x.window,
+            x.part, x.splits, self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y),
+            int(slices > 1 or out_dtype == torch.float32), slices, m, n, self._stream(),
         )
         return y
 
@@ -395,6 +512,9 @@ class HipOps:
         `rope_kv_write`.  `fused` forces one of the two ways, `mfma_kernel` the fused kernel
         (tests).
         """
+        pending = x if isinstance(x, PendingNorm) and x.value is None else None
+        if isinstance(x, PendingNorm) and pending is None:
+            x = x.value
         m, k = x.shape
         width = (num_heads + 2 * num_kv_heads) * head_dim
         can_fuse = (
@@ -408,6 +528,10 @@ class HipOps:
             fused = can_fuse
         elif fused and not can_fuse:
             raise KernelError("the fused query/key/value kernel takes bfloat16 tokens and a full rotation")
+        if pending is not None and not (
+            fused and not mfma_kernel and m <= self.FUSED_NORM_TOKENS and width * k * 2 < 1 << 32
+        ):
+            x, pending = self.settle(pending), None
         if not fused:
             qkv = self.linear(x, weight, bias)
             self.rope_kv_write(
@@ -415,7 +539,8 @@ class HipOps:
                 num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size, write=write,
             )
             return qkv
-        self._check(x, "linear input", self.dtype, (None, None))
+        if pending is None:
+            self._check(x, "linear input", self.dtype, (None, None))
         self._check(weight, "qkv weight", self.dtype, (width, k))
         if bias is not None:
             self._check(bias, "qkv bias", (torch.float32, self.dtype), (width,))
@@ -429,6 +554,17 @@ class HipOps:
             num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
             self._check(slot_mapping, "slot mapping", torch.int32, (m,))
         q = self._empty((m, num_heads * head_dim), self.dtype)
+        if pending is not None:
+            residual, norm_args = self._norm_arguments(pending)
+            self._call(
+                "mlr_qkv_norm_fused_bf16", *norm_args, self._ptr(weight), self._ptr(bias),
+                int(bias is not None and bias.dtype == torch.float32), self._ptr(cos), self._ptr(sin),
+                self._ptr(slot_mapping if write else None), self._ptr(key_pages if write else None),
+                self._ptr(value_pages if write else None), self._ptr(q), m, k, num_heads, num_kv_heads, head_dim,
+                block_size, num_pages, int(write), self._stream(),
+            )
+            pending.residual = residual
+            return q
         self._call(
             "mlr_qkv_rope_write_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias),
             int(bias is not None and bias.dtype == torch.float32), self._ptr(cos), self._ptr(sin),
@@ -453,8 +589,13 @@ class HipOps:
         scale: float,
         window: Optional[int],
         kernel: str = "auto",
-    ) -> torch.Tensor:
+        defer_merge: bool = False,
+    ):
         """Causal attention of the step's tokens over their requests' pages.
+
+        defer_merge: the caller hands the result to `linear` and nothing else; when every
+        entry has one token and their keys are cut into partitions, it may then receive a
+        `PendingMerge` (the partitions, for that product to merge) instead of a tensor.
 
         qkv: [T, >= num_heads * head_dim], queries in the leading columns (already
         position-encoded); returns [T, num_heads * head_dim].  `ctx` describes the
@@ -523,12 +664,20 @@ class HipOps:
             partial = None
             if splits > 1:
                 partial = self._empty((lib.mlr_attention_decode_scratch(entries, num_heads, splits),), torch.float32)
+            leave_unmerged = (
+                defer_merge and self.tuning.fuse_merge and not num_tiles and num_decode == entries == tokens
+                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS
+            )
             self._call(
                 "mlr_attention_decode", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.cu_q), self._ptr(ctx.context_lens), self._ptr(out),
                 self._ptr(partial), entries, num_heads, num_kv_heads, block_size, num_pages, float(scale),
-                int(window or 0), part, splits, self._stream(), lib=lib,
+                int(window or 0), part, splits, int(not leave_unmerged), self._stream(), lib=lib,
             )
+            if leave_unmerged:
+                return PendingMerge(
+                    partial, ctx.cu_q, ctx.context_lens, tokens, num_heads, head_dim, int(window or 0), part, splits, lib
+                )
         if num_tiles:
             self._check(ctx.query_tiles, "query tiles", torch.int32, (num_tiles, 2))
             self._call(

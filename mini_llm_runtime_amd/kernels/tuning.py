@@ -13,6 +13,10 @@ class KernelTuning:
     max_k_slices: int = 16  # most partial sums a narrow product may be cut into
     fuse_norm: bool = True  # norm (+ residual) as the prologue of the product behind it, for few tokens
     fuse_merge: bool = True  # merge of the decode attention's splits as the prologue of the output product
+    # A fused prologue is repeated by every workgroup of the product, and a compute unit takes in
+    # only some 15 GB/s whatever the source: beyond this many bytes of prologue input per workgroup
+    # the kernel of its own is the faster way.
+    fuse_bytes: int = 1 << 30
 
     def __post_init__(self) -> None:
         for name in ("decode_partition", "decode_max_groups", "max_k_slices"):

@@ -34,7 +34,7 @@ class GQAAttention(Mixer):
     """
 
     replayable = True
-
+    takes_pending_norm = True  # `h` goes to the query/key/value product only
 
     def __init__(
         self,
@@ -133,5 +133,6 @@ class GQAAttention(Mixer):
             block_size=cache.block_size,
             scale=self.scale,
             window=self.window,
+            defer_merge=True,  # the output product is the only reader
         )
         return ops.linear(attended, self.o_weight, self.o_bias_vec, partial_sums=True)

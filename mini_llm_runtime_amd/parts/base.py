@@ -23,6 +23,10 @@ class Part:
     # entries, tiles, block table width).  A step of such parts can be recorded as a HIP graph
     # and replayed for later steps of the same sizes.  Off by default: a part has to say so.
     replayable = False
+    # A mixer or feed-forward that hands its input `h` to `ops.linear` / `ops.qkv_rope_write`
+    # and to nothing else may say so: it then may receive a norm that has not run yet (which
+    # those operations run, fused into their own kernel where they can) instead of a tensor.
+    takes_pending_norm = False
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}
@@ -38,6 +42,10 @@ class Part:
 
 
 class Norm(Part):
+    # True when `forward` takes `defer=True` and may then return a pending norm (an object with a
+    # `residual` attribute that holds the updated stream once a consumer has run it).
+    can_defer = False
+
     def forward(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x: float32 residual stream [T, H].  When `delta` is given, first x += delta
         (in place, summed in 32-bit); returns norm(x) in the engine's dtype.  `delta` is a

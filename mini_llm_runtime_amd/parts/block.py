@@ -45,7 +45,26 @@ class PreNormBlock(Block):
     def forward(
         self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor], site: int
     ) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
-        h = self.norm_input.forward(ctx, x, delta)
+        h = _norm(self.norm_input, self.mixer, ctx, x, delta)
         mixed = self.mixer.forward(ctx, h, site)
-        h = self.norm_post_mixer.forward(ctx, x, mixed)
-        return x, self.feed_forward.forward(ctx, h)
+        x = _stream_after(h, x)
+        h = _norm(self.norm_post_mixer, self.feed_forward, ctx, x, mixed)
+        out = self.feed_forward.forward(ctx, h)
+        return _stream_after(h, x), out
+
+
+def _norm(norm: Norm, consumer: Part, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor]):
+    """norm(x + delta) for `consumer`: possibly not run yet, if both sides can deal with that."""
+    if norm.can_defer and consumer.takes_pending_norm:
+        return norm.forward(ctx, x, delta, defer=True)
+    return norm.forward(ctx, x, delta)
+
+
+def _stream_after(h, x: torch.Tensor) -> torch.Tensor:
+    """The residual stream once `h` was consumed: the tensor the norm updated in place, or the
+    new one that the consumer of a pending norm wrote."""
+    if isinstance(h, torch.Tensor):
+        return x
+    if h.residual is None:
+        raise RuntimeError("a part that takes pending norms did not hand its input to an operation that runs them")
+    return h.residual

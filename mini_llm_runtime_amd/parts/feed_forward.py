@@ -23,7 +23,7 @@ class SwiGLU(FeedForward):
     """
 
     replayable = True
-
+    takes_pending_norm = True  # `h` goes to the gate/up product only
 
     def __init__(self, hidden_size: int, intermediate_size: int) -> None:
         if hidden_size <= 0 or intermediate_size <= 0 or intermediate_size % 2:

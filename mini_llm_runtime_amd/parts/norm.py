@@ -22,7 +22,7 @@ class RMSNorm(Norm):
     """
 
     replayable = True
-
+    can_defer = True
 
     def __init__(self, size: int, eps: float) -> None:
         if size <= 0 or not eps >= 0:
@@ -34,6 +34,13 @@ class RMSNorm(Norm):
     def param_specs(self) -> dict[str, ParamSpec]:
         return {"weight": ParamSpec((self.size,), init="one_plus_normal", keep_stored_precision=True)}
 
-    def forward(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor] = None, defer: bool = False):
+        """defer: the consumer takes a norm that has not run (see `Part.takes_pending_norm`); the
+        kernel library decides whether there is something to gain."""
+        if defer:
+            make = getattr(ctx.ops, "defer_norm", None)
+            pending = make(x, self.weight, self.eps, delta) if make is not None else None
+            if pending is not None:
+                return pending
         return ctx.ops.rmsnorm(x, self.weight, self.eps, delta=delta)
 

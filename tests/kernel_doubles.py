@@ -102,7 +102,8 @@ class TorchOps:
         return qkv
 
     def paged_attention(
-        self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window
+        self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window,
+        defer_merge=False,
     ):
         self._count("paged_attention")
         tokens = qkv.shape[0]
