@@ -94,12 +94,13 @@ class KVGroup:
 
 class StateBank:
     """Two copies of a fixed-size state per request slot: a step reads one and
-    writes the other, commit swaps them, so an aborted step changes nothing."""
+    writes the other, commit swaps them, so an aborted step changes nothing.  Two spare rows
+    behind them belong to nobody: the padded entries of a recorded step read and write those."""
 
     def __init__(self, site: int, spec: SlotStateSpec, num_slots: int, device: torch.device) -> None:
         self.site = site
         self.spec = spec
-        self.tensor = torch.zeros((num_slots * 2, *spec.shape), dtype=_TORCH_DTYPES[spec.dtype], device=device)
+        self.tensor = torch.zeros((num_slots * 2 + 2, *spec.shape), dtype=_TORCH_DTYPES[spec.dtype], device=device)
 
 
 @dataclass
@@ -279,6 +280,11 @@ class CacheManager:
     @property
     def step_in_flight(self) -> bool:
         return self._pending is not None
+
+    @property
+    def state_spare_rows(self) -> tuple[int, int]:
+        """(row to read, row to write) of every state bank that no request owns."""
+        return 2 * self.max_requests, 2 * self.max_requests + 1
 
     # ---- visibility of pending tokens (debug) ------------------------------------------------
     @property

@@ -15,6 +15,7 @@ qwen_model_runner.py:371-375, 495-503), result rows in the order of the batch
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from types import SimpleNamespace
 from typing import Any, Optional, Sequence
 
 import numpy as np
@@ -22,7 +23,7 @@ import torch
 
 from ..cache.manager import CacheManager, StepLayout
 from ..cache.spec import PagedKVSpec, SlotStateSpec
-from ..parts.context import KVView, StateView, StepContext, query_tiles
+from ..parts.context import KVView, MixerPlan, PlanInput, StateView, StepContext
 from ..parts.model import DecoderModel
 
 
@@ -100,7 +101,8 @@ class ModelRunner:
         # Steps that hold single tokens only are captured once per (padded batch, table
         # width) as a HIP graph and replayed: a decode step of a small model is hundreds of
         # short kernels, and launching them one by one from the host costs more than running them.
-        # Only for models whose parts all say `replayable`.
+        # Only for models whose parts all say `replayable`; fixed-size state is no obstacle (its
+        # rows come with the step's uploaded metadata, padded entries use the banks' spare rows).
         # (a recording runs the parts' host code once, so their reports to the visibility check
         # would be missing from every replay: the check runs unrecorded)
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and not cache.check_visibility
@@ -139,23 +141,52 @@ class ModelRunner:
                 )
 
     # ---- metadata of a step ------------------------------------------------------------------
+    FIXED_ARRAYS = 9  # token ids, positions, token entries, cu_q, q_starts, context lengths, state rows (2), wanted rows
+
+    def _plans(self, shape: PlanInput) -> list[MixerPlan]:
+        """The launch plans of the model's mixers for a step of this shape, one per plan key, in
+        the order of the sites.  The step function uploads their arrays and keys its recordings
+        by their sizes; what is in them is the mixers' business."""
+        plans: dict[Any, MixerPlan] = {}
+        for entry in self.model.spec.order:
+            plan = self.model.layers[entry.layer].mixer.plan(self.ops, shape)
+            if plan is not None and plan.key not in plans:
+                plans[plan.key] = plan
+        return list(plans.values())
+
+    @staticmethod
+    def _plan_sizes(plans: Sequence[MixerPlan]) -> tuple:
+        return tuple((repr(p.key), tuple(sorted(p.sizes.items()))) for p in plans)
+
     def _arrays(
         self,
         layout: StepLayout,
         token_ids: np.ndarray,
         logit_rows: np.ndarray,
-        tiles: np.ndarray,
+        plans: Sequence[MixerPlan],
         pad_entries: Optional[int] = None,
         table_width: Optional[int] = None,
     ) -> list[np.ndarray]:
-        """The int32 arrays a step uploads, in a fixed order.  With `pad_entries` (a batch
+        """The int32 arrays a step uploads, in a fixed order: the FIXED_ARRAYS, a slot mapping
+        and a block table per page pool, then the plans' arrays.  With `pad_entries` (a batch
         of single tokens only) every array is padded to that many entries: padded entries
-        have no cached tokens, write nothing (slot -1) and own no page."""
+        have no cached tokens, write nothing (slot -1, the state banks' spare rows) and own no
+        page.  With `table_width` the block tables are that wide."""
+        planned = [np.ascontiguousarray(a, dtype=np.int32) for p in plans for a in p.arrays.values()]
+        tables = layout.block_tables
+        if table_width is not None:
+            rows = pad_entries if pad_entries is not None else layout.num_entries
+            wide_tables = []
+            for t in tables:
+                wide = np.full((rows, table_width), -1, dtype=np.int32)
+                wide[: t.shape[0], : t.shape[1]] = t
+                wide_tables.append(wide)
+            tables = wide_tables
         if pad_entries is None:
             return [
                 token_ids, layout.positions, layout.token_entry, layout.cu_q, layout.q_starts,
-                layout.context_lens, layout.state_read, layout.state_write, logit_rows, tiles,
-                *layout.slot_mappings, *layout.block_tables,
+                layout.context_lens, layout.state_read, layout.state_write, logit_rows,
+                *layout.slot_mappings, *tables, *planned,
             ]
         count, padded = layout.num_entries, pad_entries
 
@@ -164,19 +195,15 @@ class ModelRunner:
             out[:count] = a
             return out
 
-        tables = []
-        for t in layout.block_tables:
-            wide = np.full((padded, table_width), -1, dtype=np.int32)
-            wide[:count, : t.shape[1]] = t
-            tables.append(wide)
+        spare_read, spare_write = self.cache.state_spare_rows
         return [
             pad(token_ids, 0), pad(layout.positions, 0), np.arange(padded, dtype=np.int32),
             np.arange(padded + 1, dtype=np.int32), pad(layout.q_starts, 0), pad(layout.context_lens, 0),
-            pad(layout.state_read, 0), pad(layout.state_write, 0), np.arange(padded, dtype=np.int32), tiles,
-            *[pad(m, -1) for m in layout.slot_mappings], *tables,
+            pad(layout.state_read, spare_read), pad(layout.state_write, spare_write), np.arange(padded, dtype=np.int32),
+            *[pad(m, -1) for m in layout.slot_mappings], *tables, *planned,
         ]
 
-    def _context(self, dev: torch.Tensor, spans, layout: StepLayout, **plan) -> StepContext:
+    def _context(self, dev: torch.Tensor, spans, layout: Optional[StepLayout], plans: Sequence[MixerPlan], **sizes) -> StepContext:
         groups = len(self.cache.groups)
 
         def view(i: int) -> torch.Tensor:
@@ -195,13 +222,20 @@ class ModelRunner:
             q_starts=view(4),
             context_lens=view(5),
             host=layout,
-            query_tiles=view(9) if plan["num_query_tiles"] else None,
-            **plan,
+            **sizes,
         )
         state_read, state_write = view(6), view(7)
         ctx.memo["logit_rows"] = view(8)
-        slot_maps = [view(10 + g) for g in range(groups)]
-        tables = [view(10 + groups + g) for g in range(groups)]
+        first = self.FIXED_ARRAYS
+        slot_maps = [view(first + g) for g in range(groups)]
+        tables = [view(first + groups + g) for g in range(groups)]
+        at = first + 2 * groups
+        for plan in plans:
+            fields: dict[str, Any] = dict(plan.sizes)
+            for name in plan.arrays:
+                fields[name] = view(at)
+                at += 1
+            ctx.plans[plan.key] = SimpleNamespace(**fields)
         for site in range(self.model.num_sites):
             source = self.model.cache_site_of(site)
             spec = self.cache.site_specs[source]
@@ -235,23 +269,21 @@ class ModelRunner:
         layout: StepLayout,
         token_ids: np.ndarray,
         logit_rows: np.ndarray,
-        tiles: np.ndarray,
         site_outputs: Optional[list] = None,
     ) -> Optional[torch.Tensor]:
-        single = layout.q_lens == 1
-        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, tiles))
+        longest = int(layout.context_lens.max())
+        plans = self._plans(PlanInput(layout.q_lens, layout.q_starts, longest))
+        host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, plans))
         dev = host.to(self.device, non_blocking=True)
         ctx = self._context(
             dev,
             spans,
             layout,
+            plans,
             num_tokens=layout.num_tokens,
             num_entries=layout.num_entries,
             max_q_len=int(layout.q_lens.max()),
-            max_context_len=int(layout.context_lens.max()),
-            num_query_tiles=len(tiles),
-            num_decode_entries=int(single.sum()),
-            max_decode_context=int(layout.context_lens[single].max()) if single.any() else 0,
+            max_context_len=longest,
         )
         return self.model.forward(ctx, ctx.memo["logit_rows"] if logit_rows.size else None, site_outputs)
 
@@ -259,34 +291,30 @@ class ModelRunner:
     def _table_quantum(self) -> int:
         return max(1, 1024 // self.cache.block_size)  # table widths in steps of 1,024 tokens
 
-    def _step_key(self, layout: StepLayout, logit_rows: np.ndarray, tiles: np.ndarray) -> Optional[tuple]:
-        """The sizes that fix every launch of a step; None when such steps are not recorded."""
-        if (
-            not self.use_graphs
-            or self.cache.state_banks
-            or not self.model.replayable
-            or layout.num_tokens > self.max_graph_tokens
-        ):
-            return None
+    def _table_width(self, layout: StepLayout) -> int:
         pages = -(-int(layout.context_lens.max()) // self.cache.block_size)
         quantum = self._table_quantum()
-        width = -(-pages // quantum) * quantum
-        decodes = int((layout.q_lens == 1).sum())
-        return ("step", layout.num_tokens, layout.num_entries, len(tiles), decodes, width, int(logit_rows.size))
+        return -(-pages // quantum) * quantum
+
+    def _recordable(self) -> bool:
+        return self.use_graphs and self.model.replayable
+
+    def _step_key(self, layout: StepLayout, logit_rows: np.ndarray) -> Optional[tuple]:
+        """(identity of a recording, the plans it was derived from): the sizes that fix every launch
+        of a step; None when such steps are not recorded."""
+        if not self._recordable() or layout.num_tokens > self.max_graph_tokens:
+            return None
+        width = self._table_width(layout)
+        plans = self._plans(PlanInput(layout.q_lens, layout.q_starts, width * self.cache.block_size))
+        key = ("step", layout.num_tokens, layout.num_entries, width, int(logit_rows.size), self._plan_sizes(plans))
+        return key, plans
 
     def _forward_recorded(
-        self, key: tuple, layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray, tiles: np.ndarray
+        self, key: tuple, plans: Sequence[MixerPlan], layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray
     ) -> Optional[torch.Tensor]:
         """Replay (recording first, if need be) the graph of a step of these sizes."""
-        width = key[5]
-        span = width * self.cache.block_size
-        arrays = self._arrays(layout, token_ids, logit_rows, tiles)
-        groups = len(layout.block_tables)
-        for g in range(groups):  # block tables as wide as the graph was recorded with
-            table = arrays[len(arrays) - groups + g]
-            wide = np.full((table.shape[0], width), -1, dtype=np.int32)
-            wide[:, : table.shape[1]] = table
-            arrays[len(arrays) - groups + g] = wide
+        width = key[3]
+        arrays = self._arrays(layout, token_ids, logit_rows, plans, table_width=width)
         graph = self._step_graphs.pop(key, None)
         if graph is None:
             buf, spans = _pack_int32(arrays)
@@ -295,16 +323,13 @@ class ModelRunner:
             ctx = self._context(
                 static,
                 spans,
-                layout,
+                None,  # what a recording bakes in must not come from this one step's layout
+                plans,
                 num_tokens=layout.num_tokens,
                 num_entries=layout.num_entries,
                 max_q_len=layout.num_tokens,
-                max_context_len=span,
-                num_query_tiles=len(tiles),
-                num_decode_entries=key[4],
-                max_decode_context=span if key[4] else 0,
+                max_context_len=width * self.cache.block_size,
             )
-            ctx.host = None  # what a recording bakes in must not come from this one step's layout
             wanted = ctx.memo["logit_rows"] if logit_rows.size else None
             # one plain run with exactly these launch sizes first: whatever is set up at a
             # kernel's first use must exist before the recording (the run writes the same cache
@@ -336,7 +361,7 @@ class ModelRunner:
     # ---- decode steps as HIP graphs ---------------------------------------------------------------
     def _graph_key(self, layout: StepLayout) -> Optional[tuple[int, int]]:
         """(padded batch, block table width) when the step can replay a captured graph."""
-        if not self.use_graphs or self.cache.state_banks or not self.model.replayable or (layout.q_lens != 1).any():
+        if not self._recordable() or (layout.q_lens != 1).any():
             return None
         count = layout.num_entries
         if count > self.max_graph_batch:
@@ -344,12 +369,9 @@ class ModelRunner:
         padded = 1
         while padded < count:
             padded *= 2
-        bs = self.cache.block_size
-        pages = -(-int(layout.context_lens.max()) // bs)
-        quantum = self._table_quantum()
-        return padded, -(-pages // quantum) * quantum
+        return padded, self._table_width(layout)
 
-    def _graph_staging(self, key: tuple[int, int], spans, size: int):
+    def _graph_staging(self, key: tuple, spans, size: int):
         """Two pinned host buffers per graph (a step fills one while the other may still be
         read by the previous step's copy), each with int32 views in the order of `_arrays`."""
         staging = self._staging.get(key)
@@ -369,27 +391,47 @@ class ModelRunner:
             slot[2].synchronize()  # the copy that last read this buffer
         return slot
 
-    def _fill_padded(self, views, layout: StepLayout, token_ids: np.ndarray) -> None:
+    def _padded_plans(self, padded: int, width: int, q_starts: Optional[np.ndarray] = None) -> list[MixerPlan]:
+        """Plans of a batch of `padded` single tokens whose contexts fit `width` pages."""
+        starts = np.zeros(padded, dtype=np.int32)
+        if q_starts is not None:
+            starts[: len(q_starts)] = q_starts
+        return self._plans(PlanInput(np.ones(padded, dtype=np.int32), starts, width * self.cache.block_size))
+
+    def _fill_padded(self, views, layout: StepLayout, token_ids: np.ndarray, graph) -> None:
         """`_arrays(..., pad_entries, table_width)` written into the views of a staging buffer.
         The views of the constant arrays (token_entry, cu_q, logit rows) were set when the
         buffer was made."""
         count = layout.num_entries
+        spare_read, spare_write = self.cache.state_spare_rows
         for view, values, fill in (
             (views[0], token_ids, 0), (views[1], layout.positions, 0), (views[4], layout.q_starts, 0),
-            (views[5], layout.context_lens, 0), (views[6], layout.state_read, 0), (views[7], layout.state_write, 0),
+            (views[5], layout.context_lens, 0), (views[6], layout.state_read, spare_read),
+            (views[7], layout.state_write, spare_write),
         ):
             view[:count] = values
             view[count:] = fill
         groups = len(layout.slot_mappings)
+        first = self.FIXED_ARRAYS
         for g in range(groups):
-            view = views[10 + g]
+            view = views[first + g]
             view[:count] = layout.slot_mappings[g]
             view[count:] = -1
-            table = views[10 + groups + g]
+            table = views[first + groups + g]
             t = layout.block_tables[g]
             table[:count, : t.shape[1]] = t
             table[:count, t.shape[1] :] = -1
             table[count:] = -1
+        padded, width, sizes, has_plan_arrays = graph[5]
+        if has_plan_arrays:  # plans whose arrays depend on the step's data are made again
+            plans = self._padded_plans(padded, width, layout.q_starts)
+            if self._plan_sizes(plans) != sizes:
+                raise RuntimeError("a mixer's plan for a batch of single tokens changed its sizes between steps")
+            at = first + 2 * groups
+            for plan in plans:
+                for array in plan.arrays.values():
+                    views[at][...] = np.asarray(array, dtype=np.int32).reshape(views[at].shape)
+                    at += 1
 
     def _forward_graph(
         self, key: tuple[int, int], layout: StepLayout, token_ids: np.ndarray, logit_rows: np.ndarray
@@ -397,8 +439,8 @@ class ModelRunner:
         padded, width = key
         graph = self._graphs.pop(key, None)
         if graph is None:
-            empty = np.zeros((0, 2), dtype=np.int32)
-            arrays = self._arrays(layout, token_ids, logit_rows, empty, padded, width)
+            plans = self._padded_plans(padded, width, layout.q_starts)
+            arrays = self._arrays(layout, token_ids, logit_rows, plans, padded, width)
             buf, spans = _pack_int32(arrays)
             slot = self._graph_staging(key, spans, buf.size)
             for other in self._staging[key][0]:
@@ -408,14 +450,12 @@ class ModelRunner:
             ctx = self._context(
                 static,
                 spans,
-                layout,
+                None,
+                plans,
                 num_tokens=padded,
                 num_entries=padded,
                 max_q_len=1,
                 max_context_len=width * self.cache.block_size,
-                num_query_tiles=0,
-                num_decode_entries=padded,
-                max_decode_context=width * self.cache.block_size,
                 logits_for_all=True,
             )
             # one eager run first: everything that is set up lazily must exist before capture
@@ -425,7 +465,8 @@ class ModelRunner:
             captured = torch.cuda.CUDAGraph()
             with torch.cuda.graph(captured):
                 out = self.model.forward(ctx, ctx.memo["logit_rows"])
-            graph = (captured, static, out, spans, buf.size)
+            has_plan_arrays = any(np.asarray(a).size for p in plans for a in p.arrays.values())
+            graph = (captured, static, out, spans, buf.size, (padded, width, self._plan_sizes(plans), has_plan_arrays))
             # nothing is running here (the plain run above was waited for): the graphs that
             # were used longest ago can go
             while len(self._graphs) >= self.max_decode_graphs:
@@ -443,9 +484,9 @@ class ModelRunner:
     def _replay(self, key, graph, layout: StepLayout, token_ids: np.ndarray, device_tokens: Optional[torch.Tensor]):
         """Upload the step's metadata into the graph's static buffer and replay it; token ids
         come from the host array or, stream-ordered after the upload, from a device tensor."""
-        captured, static, out, spans, size = graph
+        captured, static, out, spans, size = graph[:5]
         slot = self._graph_staging(key, spans, size)
-        self._fill_padded(slot[1], layout, token_ids)
+        self._fill_padded(slot[1], layout, token_ids, graph)
         static.copy_(slot[0], non_blocking=True)
         if self._pinned:
             done = slot[2] or torch.cuda.Event()
@@ -466,12 +507,7 @@ class ModelRunner:
         writes lands in pages that later steps, ordered behind it on the stream, overwrite).
         Returns None when such a step cannot replay an already captured graph."""
         count = len(request_ids)
-        if (
-            not self.use_graphs
-            or self.cache.state_banks
-            or not self.model.replayable
-            or not 0 < count <= self.max_graph_batch
-        ):
+        if not self._recordable() or not 0 < count <= self.max_graph_batch:
             return None
         if device_tokens.shape != (count,) or device_tokens.dtype != torch.int32 or device_tokens.device != self.device:
             raise ValueError("device_tokens must be int32 [requests] on the runner's device")
@@ -530,21 +566,19 @@ class ModelRunner:
                 logits = self._forward_graph(key, layout, token_ids, logit_rows)
                 borrowed = True
             elif capture_sites:
-                tiles = query_tiles(layout.q_lens, layout.q_starts)
-                logits = self._forward_eager(layout, token_ids, logit_rows, tiles, captured)
+                logits = self._forward_eager(layout, token_ids, logit_rows, captured)
             else:
-                tiles = query_tiles(layout.q_lens, layout.q_starts)
-                step_key = self._step_key(layout, logit_rows, tiles)
+                keyed = self._step_key(layout, logit_rows)
                 seen = 0
-                if step_key is not None:
-                    seen = self._step_seen[step_key] = self._step_seen.get(step_key, 0) + 1
+                if keyed is not None:
+                    seen = self._step_seen[keyed[0]] = self._step_seen.get(keyed[0], 0) + 1
                     if len(self._step_seen) > 4096:
                         self._step_seen.clear()
                 if seen >= 2:
-                    logits = self._forward_recorded(step_key, layout, token_ids, logit_rows, tiles)
+                    logits = self._forward_recorded(keyed[0], keyed[1], layout, token_ids, logit_rows)
                     borrowed = True
                 else:
-                    logits = self._forward_eager(layout, token_ids, logit_rows, tiles)
+                    logits = self._forward_eager(layout, token_ids, logit_rows)
             if borrowed and not borrow_logits and logits is not None:
                 logits = logits.clone()
         except BaseException:

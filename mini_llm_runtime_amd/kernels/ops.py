@@ -71,7 +71,7 @@ _SIGNATURES = {
     ),
 }
 
-from ..parts.context import QUERY_TILE, query_tiles  # noqa: F401  (the plan the prefill kernel runs)
+from .plans import PAGED_ATTENTION, QUERY_TILE, attention_plan, query_tiles  # noqa: F401
 
 
 class KernelError(RuntimeError):
@@ -139,6 +139,14 @@ class HipOps:
                 raise KernelError(f"the attention library for head size {head_dim} was built for another size")
             self._attention_libs[head_dim] = lib
         return lib
+
+    # ---- plans --------------------------------------------------------------------------------
+    ATTENTION_PLAN = PAGED_ATTENTION
+
+    @staticmethod
+    def attention_plan(shape):
+        """The plan `paged_attention` wants for a step of this shape (see kernels/plans.py)."""
+        return attention_plan(shape)
 
     # ---- helpers --------------------------------------------------------------------------
     def _stream(self) -> _VP:
@@ -590,12 +598,15 @@ class HipOps:
         window: Optional[int],
         kernel: str = "auto",
         defer_merge: bool = False,
+        plan: Any = None,
     ):
         """Causal attention of the step's tokens over their requests' pages.
 
         defer_merge: the caller hands the result to `linear` and nothing else; when every
         entry has one token and their keys are cut into partitions, it may then receive a
         `PendingMerge` (the partitions, for that product to merge) instead of a tensor.
+        plan: what `attention_plan` made for this step (query tiles, single-token entries and
+        the bound on their contexts); without one the matrix-core kernels are not used.
 
         qkv: [T, >= num_heads * head_dim], queries in the leading columns (already
         position-encoded); returns [T, num_heads * head_dim].  `ctx` describes the
@@ -630,8 +641,10 @@ class HipOps:
             and block_size % 4 == 0
             and stride % 8 == 0
         )
-        num_tiles = int(getattr(ctx, "num_query_tiles", 0))
-        num_decode = int(getattr(ctx, "num_decode_entries", 0))
+        if plan is None:
+            plan = ctx  # callers that keep the plan's fields on the batch description itself
+        num_tiles = int(getattr(plan, "num_query_tiles", 0))
+        num_decode = int(getattr(plan, "num_decode_entries", 0))
         if use_mfma and num_tiles + num_decode == 0:
             use_mfma = False  # a caller that planned nothing (kernel tests of the plain path)
         lib = None
@@ -650,7 +663,7 @@ class HipOps:
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
         self._check(ctx.context_lens, "context lengths", torch.int32, (entries,))
         if num_decode:
-            span = int(ctx.max_decode_context)
+            span = int(plan.max_decode_context)
             if window:
                 span = min(span, int(window) + 15)
             group_tiles = -(-(num_heads // num_kv_heads) // 16)
@@ -679,10 +692,10 @@ class HipOps:
                     partial, ctx.cu_q, ctx.context_lens, tokens, num_heads, head_dim, int(window or 0), part, splits, lib
                 )
         if num_tiles:
-            self._check(ctx.query_tiles, "query tiles", torch.int32, (num_tiles, 2))
+            self._check(plan.query_tiles, "query tiles", torch.int32, (num_tiles, 2))
             self._call(
                 "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
-                self._ptr(block_table), width, self._ptr(ctx.query_tiles), num_tiles, self._ptr(ctx.cu_q),
+                self._ptr(block_table), width, self._ptr(plan.query_tiles), num_tiles, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
                 float(scale), int(window or 0), self._stream(), lib=lib,
             )

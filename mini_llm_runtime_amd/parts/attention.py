@@ -9,7 +9,7 @@ import torch
 
 from ..cache.spec import PagedKVSpec
 from .base import Mixer, Part, PositionEncoding
-from .context import StepContext
+from .context import MixerPlan, PlanInput, StepContext
 from .registry import build_part, register_part
 from .spec import ParamSpec, PartSpec
 
@@ -94,6 +94,10 @@ class GQAAttention(Mixer):
     def cache_spec(self) -> PagedKVSpec:
         return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    def plan(self, ops, shape: PlanInput) -> Optional[MixerPlan]:
+        make = getattr(ops, "attention_plan", None)  # the kernel library knows what its kernels want
+        return make(shape) if make is not None else None
+
     def forward(self, ctx: StepContext, h: torch.Tensor, site: int) -> torch.Tensor:
         ops = ctx.ops
         cache = ctx.kv(site)
@@ -134,5 +138,6 @@ class GQAAttention(Mixer):
             scale=self.scale,
             window=self.window,
             defer_merge=True,  # the output product is the only reader
+            plan=ctx.plan(getattr(ops, "ATTENTION_PLAN", None)),
         )
         return ops.linear(attended, self.o_weight, self.o_bias_vec, partial_sums=True)

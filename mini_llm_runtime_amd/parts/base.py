@@ -12,7 +12,7 @@ from typing import Any, Mapping, Optional
 
 import torch
 
-from .context import StepContext
+from .context import MixerPlan, PlanInput, StepContext
 from .spec import ParamSpec
 
 
@@ -69,6 +69,13 @@ class PositionEncoding(Part):
 class Mixer(Part):
     def cache_spec(self) -> Any:
         """PagedKVSpec, SlotStateSpec or None."""
+        return None
+
+    def plan(self, ops: Any, shape: PlanInput) -> Optional[MixerPlan]:
+        """What this mixer's kernels need planned on the host for a step of this shape (tiles,
+        counts, launch sizes), or None.  The step function uploads the plan's arrays with the
+        step's metadata, hands the plan to `forward` through `ctx.plan(key)`, and records a
+        step only for replay under plans of the same sizes; it knows nothing of what is in it."""
         return None
 
     def forward(self, ctx: StepContext, h: torch.Tensor, site: int) -> torch.Tensor:

@@ -11,18 +11,27 @@ from typing import Any, Optional
 import numpy as np
 import torch
 
-QUERY_TILE = 64  # queries of one request that a mixer's prompt kernel takes together
+@dataclass(frozen=True)
+class PlanInput:
+    """What a mixer may look at when it plans its kernels for a step: the new tokens and the
+    cached tokens of every entry, and a bound on the entries' contexts after the step (the
+    exact maximum, or, for a step that is being recorded, the capacity of its block tables)."""
+
+    q_lens: np.ndarray  # [R] tokens of this step
+    q_starts: np.ndarray  # [R] tokens cached before it
+    max_context: int
 
 
-def query_tiles(q_lens, q_starts=None) -> np.ndarray:
-    """[num_tiles, 2] int32 (entry, first query) covering every entry with more than one new
-    token, the tiles with the most keys before them first: a kernel that hands them to the
-    compute units in that order can start the heavy ones early and pair them with light ones."""
-    tiles = [(r, q0) for r, n in enumerate(q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
-    if q_starts is None:
-        q_starts = [0] * len(q_lens)
-    tiles.sort(key=lambda t: -(int(q_starts[t[0]]) + t[1]))
-    return np.asarray(tiles, dtype=np.int32).reshape(-1, 2)
+@dataclass
+class MixerPlan:
+    """A mixer's launch plan for one step.  `arrays` (int32) are uploaded with the step's other
+    metadata; `sizes` are what the mixer's host code needs to launch (grid sizes, counts): they
+    are part of a recorded step's identity, so a recording is only replayed for steps whose
+    plans have the same sizes.  Mixers whose plans have the same `key` share one plan."""
+
+    key: Any
+    arrays: dict  # name -> np.ndarray (int32)
+    sizes: dict  # name -> int
 
 
 @dataclass
@@ -80,17 +89,17 @@ class StepContext:
     context_lens: torch.Tensor  # [R] int32 tokens visible after this step's write
     max_q_len: int
     max_context_len: int
-    host: Any  # the StepLayout (numpy arrays) for parts that plan on the host
-    # plan for attention kernels: tiles of 64 queries over entries with several new
-    # tokens ([num_tiles, 2]: entry, first query), and the single-token entries
-    query_tiles: Optional[torch.Tensor] = None
-    num_query_tiles: int = 0
-    num_decode_entries: int = 0
-    max_decode_context: int = 0
+    host: Any  # the StepLayout (numpy arrays) for parts that work on the host; None while a step is recorded
     logits_for_all: bool = False  # the wanted rows are all tokens, in order: no gather needed
     kv_views: dict[int, KVView] = field(default_factory=dict)
     state_views: dict[int, StateView] = field(default_factory=dict)
+    plans: dict[Any, Any] = field(default_factory=dict)  # MixerPlan.key -> its sizes and device arrays, as attributes
     memo: dict[Any, Any] = field(default_factory=dict)
+
+    def plan(self, key: Any) -> Any:
+        """The plan some mixer made under `key` (None: none did): an object whose attributes are
+        the plan's sizes and, as device tensors, its arrays."""
+        return self.plans.get(key)
 
     def kv(self, site: int) -> KVView:
         return self.kv_views[site]

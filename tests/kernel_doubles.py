@@ -103,7 +103,7 @@ class TorchOps:
 
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window,
-        defer_merge=False,
+        defer_merge=False, plan=None,
     ):
         self._count("paged_attention")
         tokens = qkv.shape[0]

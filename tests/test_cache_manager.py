@@ -200,7 +200,7 @@ def test_state_slots_are_double_buffered():
     specs = [PagedKVSpec(1, 4), SlotStateSpec((3,))]
     m = make(specs=specs, max_requests=2)
     bank = m.state_banks[1].tensor
-    assert bank.shape == (4, 3)
+    assert bank.shape == (6, 3) and m.state_spare_rows == (4, 5)  # two rows per slot, two that nobody owns
     a = m.create_request("a")
     b = m.create_request("b")
     assert (a.slot, b.slot) == (0, 1)

@@ -38,9 +38,12 @@ def _rand(shape, seed, scale=1.0):
     return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
 
 
-def _context(ops, cache, entries, dtype):
-    """A StepContext for a step of `entries` [(request, new tokens)], as the step function makes it."""
-    from mini_llm_runtime_amd.kernels.ops import query_tiles
+def _context(ops, cache, entries, dtype, mixer=None):
+    """A StepContext for a step of `entries` [(request, new tokens)], as the step function makes it:
+    the mixer's own plan for the batch, uploaded and handed out under the plan's key."""
+    from types import SimpleNamespace
+
+    from mini_llm_runtime_amd.parts.context import PlanInput
 
     lay = cache.begin_step(entries)
     dev = ops.device
@@ -48,17 +51,15 @@ def _context(ops, cache, entries, dtype):
     def t(a):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
 
-    tiles = query_tiles(lay.q_lens)
-    single = lay.q_lens == 1
     ctx = StepContext(
         ops=ops, dtype=dtype, device=dev, num_tokens=lay.num_tokens, num_entries=lay.num_entries,
         token_ids=t(np.zeros(lay.num_tokens, dtype=np.int32)), positions=t(lay.positions), token_entry=t(lay.token_entry),
         cu_q=t(lay.cu_q), q_starts=t(lay.q_starts), context_lens=t(lay.context_lens),
         max_q_len=int(lay.q_lens.max()), max_context_len=int(lay.context_lens.max()), host=lay,
-        query_tiles=t(tiles) if len(tiles) else None, num_query_tiles=len(tiles),
-        num_decode_entries=int(single.sum()),
-        max_decode_context=int(lay.context_lens[single].max()) if single.any() else 0,
     )
+    plan = mixer.plan(ops, PlanInput(lay.q_lens, lay.q_starts, int(lay.context_lens.max()))) if mixer is not None else None
+    if plan is not None:
+        ctx.plans[plan.key] = SimpleNamespace(**plan.sizes, **{n: t(a) for n, a in plan.arrays.items()})
     key, value, g = cache.site_pools(0)
     ctx.kv_views[0] = KVView(key, value, t(lay.block_tables[g]), t(lay.slot_mappings[g]), cache.block_size,
                             cache.groups[g].spec.window, True)
@@ -158,7 +159,7 @@ def test_attention_part_over_the_cache(backend, dtype, heads, kv_heads, head_dim
                                 num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, theta=10000.0)
     at = 0
     for size in (19, 13, 1, 1, 5, 1, 1):  # a prefix, a portion behind it, single tokens
-        ctx = _context(ops, cache, [("r", size)], dtype)
+        ctx = _context(ops, cache, [("r", size)], dtype, att)
         out = att.forward(ctx, h[at : at + size].to(ops.device), 0)
         out = out.double().sum(0) if out.dim() == 3 else out.double()
         cache.commit_step()
@@ -195,7 +196,7 @@ def test_pre_norm_block(backend, dtype):
     ref = plain.decoder_layer(x.double(), torch.arange(n), {k: v.double() for k, v in weights.items()}, 0, cfg)
     cache = CacheManager([att.cache_spec()], block_size=8, num_blocks=6, max_requests=1, dtype=dtype, device=ops.device)
     cache.create_request("r")
-    ctx = _context(ops, cache, [("r", n)], dtype)
+    ctx = _context(ops, cache, [("r", n)], dtype, att)
     xd = x.to(ops.device).clone()
     stream, delta = block.forward(ctx, xd, None, 0)
     assert stream is xd  # the residual stream is updated in place; the last output is handed on un-added

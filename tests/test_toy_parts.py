@@ -21,6 +21,7 @@ import json
 from dataclasses import dataclass, fields
 from typing import Any, ClassVar, Mapping
 
+import numpy as np
 import pytest
 import torch
 
@@ -32,6 +33,7 @@ from mini_llm_runtime_amd.cache import PagedKVSpec, SlotStateSpec
 from mini_llm_runtime_amd.config.model_config import ModelConfig
 from mini_llm_runtime_amd.engine import ModelRunner, StepEntry
 from mini_llm_runtime_amd.models import register_architecture, unregister_architecture
+from mini_llm_runtime_amd.parts.context import MixerPlan, PlanInput
 from mini_llm_runtime_amd.parts import (
     FeedForward,
     LayerSpec,
@@ -64,7 +66,16 @@ def _ops(backend, dtype):
 
 # ---- toy parts -------------------------------------------------------------------------------------
 class RunningMeanMixer(Mixer):
-    """out_t = W_out * mean_{i <= t}(W_in h_i): state = the running sum, one vector per request."""
+    """out_t = W_out * mean_{i <= t}(W_in h_i): state = the running sum, one vector per request.
+
+    Everything that depends on the step's data happens on the device (sums over the batch's
+    tokens, the entries' first tokens from `cu_q`, the state rows from the uploaded metadata),
+    so the part says `replayable`: its steps are recorded and replayed like attention's.  It
+    also brings a launch plan of its own kind, the index of every entry's last token, which
+    the step function uploads without knowing what it is for."""
+
+    replayable = True
+    PLAN = "toy_running_mean"
 
     def __init__(self, hidden_size: int) -> None:
         self.hidden_size = hidden_size
@@ -78,21 +89,24 @@ class RunningMeanMixer(Mixer):
     def cache_spec(self):
         return SlotStateSpec((self.hidden_size,), "float32")
 
+    def plan(self, ops, shape: PlanInput):
+        last = np.cumsum(shape.q_lens, dtype=np.int64) - 1
+        return MixerPlan(self.PLAN, {"last_token": last.astype(np.int32)}, {"entries": len(shape.q_lens)})
+
     def forward(self, ctx, h, site):
         ops = ctx.ops
-        u = ops.linear(h, self.in_weight, None).float()
+        u = ops.linear(h, self.in_weight, None).double()
         state = ctx.state(site)
-        out = torch.empty_like(u)
-        lay = ctx.host
-        for r in range(lay.num_entries):
-            a, b = int(lay.cu_q[r]), int(lay.cu_q[r + 1])
-            start = int(lay.q_starts[r])
-            running = torch.cumsum(u[a:b], dim=0)
-            if start > 0:
-                running = running + state.tensor[int(lay.state_read[r])]
-            counts = torch.arange(start + 1, start + 1 + (b - a), device=u.device, dtype=torch.float32)
-            out[a:b] = running / counts[:, None]
-            state.tensor[int(lay.state_write[r])] = running[-1]
+        plan = ctx.plan(self.PLAN)
+        assert plan.entries == ctx.num_entries and plan.last_token.shape == (ctx.num_entries,)
+        sums = torch.cumsum(u, dim=0)  # over the whole batch; each entry subtracts what came before it
+        first = ctx.cu_q[:-1].long()
+        before = torch.where((first > 0)[:, None], sums[(first - 1).clamp(min=0)], torch.zeros_like(sums[:1]))
+        carried = state.tensor[state.read_rows.long()].double() * (ctx.q_starts > 0)[:, None]
+        entry = ctx.token_entry.long()
+        running = sums - before[entry] + carried[entry]
+        out = running / (ctx.positions + 1).double()[:, None]
+        state.tensor[state.write_rows.long()] = running[plan.last_token.long()].float()
         return ops.linear(out.to(ctx.dtype), self.out_weight, None)
 
 
@@ -409,6 +423,57 @@ def test_toy_model_whole_and_in_portions(tmp_path, toy_registered, name, backend
     for rid in requests:
         cache.release_request(rid)
     assert all(g.allocator.free_count == g.num_blocks for g in cache.groups)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_steps_of_a_model_with_state_are_recorded(tmp_path, toy_registered, dtype):
+    """Fixed-size state is no obstacle to recordings: a model with the running-mean mixer decodes
+    through replayed graphs (batches of 1, 2 and 3 requests, padded to 1, 2 and 4 entries, the
+    padded one on the banks' spare rows) and repeats prompt portions through recorded steps, all
+    bit for bit what plain steps give, and the requests' states stay their own."""
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    config = mlr.models.config_from_dict(_toy_config("state"))
+    folder = mlr.write_random_model(config, tmp_path / "state", seed=8)
+    with SafetensorsFile(folder / "model.safetensors") as f:
+        weights = {n: f.tensor(n) for n in f.entries}
+    requests = {"a": random_tokens(60, 97, 3), "b": random_tokens(49, 97, 4), "c": random_tokens(38, 97, 5)}
+    refs = {rid: toy_plain(toks, weights, config) for rid, toks in requests.items()}
+    outputs = {}
+    for graphs in (False, True):
+        ops = HipOps(dtype, "cuda")
+        _, model = mlr.load_model(folder, dtype=dtype, device=ops.device)
+        assert model.replayable
+        cache = mlr.make_cache(model, block_size=4, num_blocks=64, max_requests=3)
+        cache.poison()
+        runner = ModelRunner(model, cache, ops, use_graphs=graphs)
+        got = []
+        fed = {}
+        for rid, toks in requests.items():  # prompts in portions of 8: the same sizes again and again
+            cache.create_request(rid)
+            for at in range(0, 24, 8):
+                got.append(runner.step([StepEntry.of(rid, toks[at : at + 8], range(8))]).logits)
+            fed[rid] = 24
+        live = list(requests)
+        while live:  # one token each; requests end one after the other: batches of 3, 2, 1
+            entries = [StepEntry.of(rid, [requests[rid][fed[rid]]], (0,)) for rid in live]
+            out = runner.step(entries).logits
+            got.append(out)
+            for i, rid in enumerate(live):
+                ref = refs[rid][fed[rid]]
+                err = (out[i].double().cpu() - ref).abs().max() / ref.abs().max()
+                assert err < (1e-4 if dtype == torch.float32 else 4e-2), (rid, fed[rid], float(err))
+                fed[rid] += 1
+            live = [rid for rid in live if fed[rid] < len(requests[rid])]
+        outputs[graphs] = got
+        if graphs:
+            assert set(runner._graphs) == {(1, 256), (2, 256), (4, 256)}, "single-token steps were not recorded"
+            assert len(runner._step_graphs) == 1, "the repeated portions were not recorded"
+        for rid in requests:
+            cache.release_request(rid)
+    for i, (want, have) in enumerate(zip(outputs[False], outputs[True])):
+        assert torch.equal(want, have), f"step {i}: a replayed step differs from the plain one"
 
 
 ROUTED = dict(
