@@ -92,7 +92,7 @@ def burst(args, config, full_layers, model, ops, device) -> dict:
 
     import torch
 
-    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
+    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PageAdmission, Scheduler
     from mini_llm_runtime_amd.engine.factory import make_cache
     from mini_llm_runtime_amd.engine.runner import ModelRunner
     from mini_llm_runtime_amd.sampling.sampler import Sampler
@@ -104,9 +104,9 @@ def burst(args, config, full_layers, model, ops, device) -> dict:
     sampler = Sampler(ops, device)
 
     def run(seed: int):
-        admission = PagedBlockAdmissionController(cache, max_step_tokens=budget)
-        scheduler = RequestScheduler(
-            max_running_requests=requests, max_batch_tokens=budget, admission_callback=admission.try_admit
+        admission = PageAdmission(cache, max_step_tokens=budget)
+        scheduler = Scheduler(
+            max_running_requests=requests, max_batch_tokens=budget, admit=admission.admit
         )
         engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
         rng = random.Random(seed)
@@ -119,12 +119,12 @@ def burst(args, config, full_layers, model, ops, device) -> dict:
             prompt_tokens += n
             generated += new
         steps = 0
-        while engine.scheduler.has_unfinished_requests:
+        while engine.scheduler.busy:
             engine.step()
             steps += 1
         torch.cuda.synchronize(device)
         seconds = time.perf_counter() - t0
-        shots = engine.metrics.snapshots()
+        shots = engine.all_times()
         return {
             "seconds": seconds,
             "steps": steps,
@@ -163,7 +163,7 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
     """One 8,192-token prompt in portions of 2,048 tokens beside 32 decoding requests."""
     import torch
 
-    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
+    from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PageAdmission, Scheduler
     from mini_llm_runtime_amd.engine.factory import make_cache
     from mini_llm_runtime_amd.engine.runner import ModelRunner
     from mini_llm_runtime_amd.sampling.sampler import Sampler
@@ -174,12 +174,12 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
     cache = make_cache(model, block_size=BLOCK_SIZE, num_blocks=pages, max_requests=decoders + 1)
     runner = ModelRunner(model, cache, ops)
     sampler = Sampler(ops, device)
-    admission = PagedBlockAdmissionController(cache, max_step_tokens=portion + decoders)
-    scheduler = RequestScheduler(
+    admission = PageAdmission(cache, max_step_tokens=portion + decoders)
+    scheduler = Scheduler(
         max_running_requests=decoders + 1,
         max_batch_tokens=portion + decoders,
         max_mixed_prefill_tokens=portion,
-        admission_callback=admission.try_admit,
+        admit=admission.admit,
     )
     engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
     gen = torch.Generator().manual_seed(args.seed)
@@ -196,7 +196,7 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
 
     for i in range(decoders):
         engine.submit(f"d{i}", ids(context), max_new_tokens=new_tokens)
-    while len(engine.step().batch.decode_request_ids) < decoders:
+    while len(engine.step().plan.decode_ids) < decoders:
         pass
     for _ in range(8):
         engine.step()
@@ -208,12 +208,12 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
         engine.submit(f"long{r}", ids(long_prompt), max_new_tokens=1)
         for i in range(portions):
             result, ms = timed_step()
-            batch = result.batch
-            assert batch.prefill_request_ids == (f"long{r}",) and len(batch.decode_request_ids) == decoders
+            batch = result.plan
+            assert batch.prompt_ids == (f"long{r}",) and len(batch.decode_ids) == decoders
             assert batch.token_count == portion + decoders
             if r >= warmups:
                 mixed[i].append(ms)
-        assert not timed_step()[0].batch.prefill_request_ids
+        assert not timed_step()[0].plan.prompt_ids
     by_portion = [median(times) for times in mixed]
     ms = sum(by_portion) / portions
     return {
@@ -334,14 +334,14 @@ class Bench:
         prompt_len: scheduler, step function, sampling on the GPU, tokens to the host."""
         import torch
 
-        from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PagedBlockAdmissionController, RequestScheduler
+        from mini_llm_runtime_amd.engine import ContinuousBatchEngine, PageAdmission, Scheduler
 
         args = self.args
-        admission = PagedBlockAdmissionController(self.cache, max_step_tokens=args.prompt_len)
-        scheduler = RequestScheduler(
+        admission = PageAdmission(self.cache, max_step_tokens=args.prompt_len)
+        scheduler = Scheduler(
             max_running_requests=batch,
             max_batch_tokens=max(args.prompt_len, batch),
-            admission_callback=admission.try_admit,
+            admit=admission.admit,
         )
         engine = ContinuousBatchEngine(
             scheduler=scheduler, runner=self.runner, admission=admission, sampler=self.sampler
@@ -350,7 +350,7 @@ class Bench:
             engine.submit(f"b{batch}-{i}", self.prompt(), max_new_tokens=warmup + steps + batch + 8)
         while True:  # prompts, until a step is nothing but one token for every request
             result = engine.step()
-            if len(result.batch.decode_request_ids) == batch:
+            if len(result.plan.decode_ids) == batch:
                 break
         for _ in range(warmup):
             engine.step()
@@ -367,7 +367,7 @@ class Bench:
         end.record()
         self.sync()
         elapsed = time.perf_counter() - t0
-        assert len(result.batch.decode_request_ids) == batch and len(result.update.emitted_tokens) == batch
+        assert len(result.plan.decode_ids) == batch and len(result.report.emitted) == batch
         engine.run_until_done()
         return {
             "ms": elapsed * 1e3 / steps,
@@ -377,7 +377,7 @@ class Bench:
 
     def kv_bytes_per_token(self) -> int:
         return sum(
-            2 * len(g.sites) * g.spec.num_kv_heads * g.spec.head_dim * g.key.element_size() for g in self.cache.groups
+            len(g.sites) * g.spec.bytes_per_token(g.key.element_size()) for g in self.cache.groups
         )
 
     def decode_bytes(self, batch: int, mean_context: float) -> tuple:

@@ -15,9 +15,9 @@ from .engine import (
     EngineConfig,
     EngineStepResult,
     ModelRunner,
-    PagedBlockAdmissionController,
-    RequestMetricsCollector,
-    RequestScheduler,
+    PageAdmission,
+    Request,
+    Scheduler,
     StepEntry,
     generate,
     greedy_generate,
@@ -43,11 +43,11 @@ __all__ = [
     "EngineStepResult",
     "ModelConfig",
     "ModelRunner",
-    "PagedBlockAdmissionController",
+    "PageAdmission",
     "PagedKVSpec",
     "Qwen2Config",
-    "RequestMetricsCollector",
-    "RequestScheduler",
+    "Request",
+    "Scheduler",
     "Sampler",
     "SamplingParams",
     "SlotStateSpec",

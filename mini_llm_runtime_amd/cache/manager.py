@@ -64,7 +64,7 @@ class KVGroup:
         # never zeroed: stale bytes must be unreachable, not clean
         self.key = torch.empty(shape, dtype=dtype, device=device)
         self.value = torch.empty(
-            (len(self.sites), num_blocks, spec.num_kv_heads, spec.head_dim, block_size), dtype=dtype, device=device
+            (len(self.sites), num_blocks, spec.num_kv_heads, spec.value_dim, block_size), dtype=dtype, device=device
         )
 
     @property
@@ -89,7 +89,7 @@ class KVGroup:
         return min(full, bounded)
 
     def storage_bytes(self) -> int:
-        return 2 * self.key.numel() * self.key.element_size()
+        return (self.key.numel() + self.value.numel()) * self.key.element_size()
 
 
 class StateBank:

@@ -136,12 +136,12 @@ def _record_step(result, manager) -> dict[str, Any]:
         request = manager.get_request(rid)
         active[rid] = {"block_ids": [list(t) for t in request.tables], "token_count": request.num_tokens}
     return {
-        "step": result.batch.step_index,
-        "token_count": result.batch.token_count,
-        "prefill": list(result.batch.prefill_request_ids),
-        "decode": list(result.batch.decode_request_ids),
-        "emitted": [list(t) for t in result.update.emitted_tokens],
-        "finished": list(result.update.finished_request_ids),
+        "step": result.plan.index,
+        "token_count": result.plan.token_count,
+        "prefill": list(result.plan.prompt_ids),
+        "decode": list(result.plan.decode_ids),
+        "emitted": [list(t) for t in result.report.emitted],
+        "finished": list(result.report.finished),
         "released_blocks": {rid: {str(g): list(ids) for g, ids in blocks.items()} for rid, blocks in result.released_blocks},
         "active_cache_after_step": active,
         "cache_stats_after_step": [asdict(s) for s in manager.stats()],
@@ -185,7 +185,7 @@ def cmd_engine(args: argparse.Namespace) -> int:
     pending = sorted(requests, key=lambda r: r.get("arrival_step", 0))
     records = []
     step_no = 0
-    while pending or engine.scheduler.has_unfinished_requests:
+    while pending or engine.scheduler.busy:
         while pending and pending[0].get("arrival_step", 0) <= step_no:
             r = pending.pop(0)
             engine.submit(
@@ -202,13 +202,13 @@ def cmd_engine(args: argparse.Namespace) -> int:
         records.append(_record_step(result, engine.manager))
         rec = records[-1]
         print(f"step={rec['step']} prefill={rec['prefill']} decode={rec['decode']} finished={rec['finished']}")
-    tokens = {str(r["id"]): list(engine.scheduler.get_request(str(r["id"])).generated_token_ids) for r in requests}
+    tokens = {str(r["id"]): list(engine.request(str(r["id"])).output) for r in requests}
     all_released = engine.manager.request_ids == () and all(
         g.allocator.free_count == g.num_blocks for g in engine.manager.groups
     )
     metrics = {}
     for rid in tokens:
-        m = engine.metrics.snapshot(rid)
+        m = engine.times(rid)
         metrics[rid] = {"queue_wait_ms": m.queue_wait_ms, "ttft_ms": m.ttft_ms, "median_tpot_ms": m.median_tpot_ms, "e2e_ms": m.e2e_ms}
     for rid, ids in tokens.items():
         print(f"{rid}: ids={ids}")

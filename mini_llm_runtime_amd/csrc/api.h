@@ -32,6 +32,9 @@ int mlr_rmsnorm(float* x, const void* delta, const float* partial, int slices, c
 // x (float32) += delta (dtype), count elements.
 int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t stream);
 
+// x (float32, in place) = x * scale, and, when cap > 0, cap * tanh(that / cap).
+int mlr_scale_softcap(float* x, float scale, float cap, int64_t count, hipStream_t stream);
+
 // out[p, k, :] = src[p, rows[k], :] for every plane p of src [planes, src_rows, width];
 // rows are `row_bytes` wide (a multiple of 4).
 int mlr_gather_rows(const void* src, const int* rows, void* out, int count, int64_t row_bytes,

@@ -315,6 +315,24 @@ int mlr_rmsnorm(float* x, const void* delta, const float* partial, int slices, c
   return 0;
 }
 
+// x = cap * tanh(x * scale / cap) when cap > 0, else x * scale (float32, in place).
+__global__ __launch_bounds__(256) void scale_softcap_kernel(float* __restrict__ x, float scale, float cap, int64_t count) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const float v = x[i] * scale;
+  x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
+int mlr_scale_softcap(float* x, float scale, float cap, int64_t count, hipStream_t stream) {
+  MLR_REQUIRE(x != nullptr, "null pointer");
+  MLR_REQUIRE(count > 0 && cap >= 0.f, "count must be > 0 and the cap >= 0");
+  const int64_t blocks = (count + 255) / 256;
+  MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
+  scale_softcap_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, scale, cap, count);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
 int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t stream) {
   MLR_REQUIRE(x && delta, "null pointer");
   MLR_REQUIRE(count > 0, "count must be > 0");

@@ -1,50 +1,40 @@
 """Step function, scheduler, admission and the continuous-batching engine."""
 
-from .admission import BlockReservation, PagedBlockAdmissionController
+from .admission import PageAdmission, PagePromise
 from .config import EngineConfig, GraphLimits
 from .engine import ContinuousBatchEngine, EngineStepResult
 from .factory import load_model, make_cache, parse_dtype
 from .generation import GenerationOutput, generate, greedy_generate
-from .metrics import RequestMetrics, RequestMetricsCollector, TokenEvent
+from .metrics import RequestTimes, summarize
+from .request import EndReason, Phase, Request, Timeline
 from .runner import ModelRunner, StepEntry, StepOutput
-from .scheduler import (
-    BatchingPolicy,
-    FinishReason,
-    RequestScheduler,
-    RequestState,
-    RequestStatus,
-    ScheduledRequest,
-    SchedulerBatch,
-    SchedulerStepUpdate,
-    WorkKind,
-)
+from .scheduler import BatchingPolicy, Scheduler, Slice, StepPlan, StepReport
 
 __all__ = [
     "BatchingPolicy",
-    "BlockReservation",
     "ContinuousBatchEngine",
+    "EndReason",
     "EngineConfig",
-    "GraphLimits",
     "EngineStepResult",
-    "FinishReason",
     "GenerationOutput",
+    "GraphLimits",
     "ModelRunner",
-    "PagedBlockAdmissionController",
-    "RequestMetrics",
-    "RequestMetricsCollector",
-    "RequestScheduler",
-    "RequestState",
-    "RequestStatus",
-    "ScheduledRequest",
-    "SchedulerBatch",
-    "SchedulerStepUpdate",
+    "PageAdmission",
+    "PagePromise",
+    "Phase",
+    "Request",
+    "RequestTimes",
+    "Scheduler",
+    "Slice",
     "StepEntry",
     "StepOutput",
-    "TokenEvent",
-    "WorkKind",
+    "StepPlan",
+    "StepReport",
+    "Timeline",
     "generate",
     "greedy_generate",
     "load_model",
     "make_cache",
     "parse_dtype",
+    "summarize",
 ]

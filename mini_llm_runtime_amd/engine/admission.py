@@ -1,72 +1,65 @@
-"""Admission by pages: a request enters only when the pages of its whole life can
-be promised to it, so that no running request ever runs out of pages.
+"""Admission by pages: a request enters only when the pages of its whole life can be
+promised to it, so that no admitted request ever runs out of pages.
 
-Behaviour of the reference's `PagedBlockAdmissionController`
-(src/mini_llm_runtime/block_admission.py:18-93): `try_admit` either creates the
-request in the cache manager with its capacity set aside, or changes nothing and
-returns False; a request that could never fit raises; finished (or un-admitted)
-requests give everything back.  The promise here is a count per page pool, not a
-set of pinned pages.
+What the reference's admission controller decides (src/mini_llm_runtime/block_admission.py:18-93):
+either the request is created in the cache manager with its capacity set aside, or nothing
+changes and the answer is no; a request that could never fit is an error; a request that ends
+(or is un-admitted after a failed step) gives everything back.  The promise here is a count per
+page pool that the cache manager keeps, not a set of pinned pages.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Iterable
 
 from ..cache.manager import CacheManager
-from .scheduler import RequestState
+from .request import Request
 
 
 @dataclass(frozen=True)
-class BlockReservation:
+class PagePromise:
     request_id: str
-    max_cache_tokens: int
-    block_counts: tuple[int, ...]  # per page pool
+    tokens: int  # most tokens the request ever caches
+    pages: tuple[int, ...]  # promised per page pool
 
 
-class PagedBlockAdmissionController:
+class PageAdmission:
     def __init__(self, manager: CacheManager, *, max_step_tokens: int) -> None:
         if max_step_tokens <= 0:
             raise ValueError("max_step_tokens must be > 0")
         self.manager = manager
         self.max_step_tokens = int(max_step_tokens)
-        self._reservations: dict[str, BlockReservation] = {}
+        self._promises: dict[str, PagePromise] = {}
 
     @property
-    def reservations(self) -> tuple[BlockReservation, ...]:
-        return tuple(self._reservations.values())
+    def promises(self) -> tuple[PagePromise, ...]:
+        return tuple(self._promises.values())
 
-    def reservation_for(self, request_id: str) -> BlockReservation:
-        try:
-            return self._reservations[request_id]
-        except KeyError:
-            raise KeyError(f"request {request_id!r} has no reservation") from None
+    def pages_for(self, tokens: int) -> tuple[int, ...]:
+        return tuple(self.manager.lifetime_blocks(tokens, self.max_step_tokens))
 
-    def try_admit(self, request: RequestState) -> bool:
-        if request.request_id in self._reservations:
-            raise RuntimeError(f"request {request.request_id!r} is already admitted")
-        tokens = request.max_cache_tokens
-        if not self.manager.try_create_reserved(request.request_id, tokens, self.max_step_tokens):
+    def can_ever_admit(self, tokens: int) -> bool:
+        """Whether empty pools could hold a request that caches this many tokens."""
+        return self.manager.can_ever_hold(tokens, self.max_step_tokens)
+
+    def admit(self, request: Request) -> bool:
+        if request.id in self._promises:
+            raise RuntimeError(f"request {request.id!r} is already admitted")
+        if not self.manager.try_create_reserved(request.id, request.cache_tokens, self.max_step_tokens):
             return False
-        self._reservations[request.request_id] = BlockReservation(
-            request_id=request.request_id,
-            max_cache_tokens=tokens,
-            block_counts=tuple(self.manager.lifetime_blocks(tokens, self.max_step_tokens)),
-        )
+        self._promises[request.id] = PagePromise(request.id, request.cache_tokens, self.pages_for(request.cache_tokens))
         return True
 
-    def release_finished(self, request_ids: tuple[str, ...]) -> dict[str, dict[int, tuple[int, ...]]]:
-        return self.release_admitted(request_ids)
-
-    def release_admitted(self, request_ids: tuple[str, ...]) -> dict[str, dict[int, tuple[int, ...]]]:
-        """Give back the pages and promises of admitted requests (finished, or un-admitted after a failed step)."""
-        if len(set(request_ids)) != len(request_ids):
-            raise ValueError("request ids must not repeat")
-        missing = [rid for rid in request_ids if rid not in self._reservations]
-        if missing:
-            raise KeyError(f"requests without a reservation: {missing}")
-        released = {}
-        for rid in request_ids:
-            released[rid] = self.manager.release_request(rid)
-            del self._reservations[rid]
-        return released
+    def release(self, request_ids: Iterable[str]) -> dict[str, dict[int, tuple[int, ...]]]:
+        """Requests that ended, or were un-admitted, give back their pages, promises and slots;
+        returns the pages each one held, per pool."""
+        ids = tuple(request_ids)
+        unknown = [rid for rid in ids if rid not in self._promises]
+        if unknown or len(set(ids)) != len(ids):
+            raise KeyError(f"not admitted, or named twice: {unknown or ids}")
+        freed = {}
+        for rid in ids:
+            freed[rid] = self.manager.release_request(rid)
+            del self._promises[rid]
+        return freed

@@ -1,26 +1,23 @@
-"""The synchronous continuous-batching loop: scheduler -> step function -> sampler
--> scheduler, with pages given back as requests finish.
+"""The continuous-batching loop: plan a step, run it, choose tokens, apply them, give pages back.
 
-One engine step, as in the reference's `ContinuousBatchEngine.step`
-(src/mini_llm_runtime/engine.py:150-281): schedule; run the model; choose tokens on
-the GPU and bring them to the host in ONE copy (engine.py:257-261); apply the
-results; release finished requests' pages in the same step (engine.py:268-269).
-On any exception the step's newly admitted requests are released and the
-scheduler's batch is undone, so the same step can be tried again
-(engine.py:249-254).  Unlike the reference, which runs prompts and decodes as two
-forwards (engine.py:186-248), a step here is one forward over the whole batch.
+What one step does follows the reference's engine (src/mini_llm_runtime/engine.py:150-281): the
+scheduler decides; the model runs; tokens are chosen on the GPU and come to the host in ONE
+copy (engine.py:257-261); the results are applied and finished requests' pages are released in
+the same step (engine.py:268-269).  When anything fails, the requests the plan admitted are
+released and the plan is cancelled, so that the same step can be tried again
+(engine.py:249-254).  Unlike the reference, which runs prompts and decodes as two forwards
+(engine.py:186-248), a step here is one forward over the whole batch, and the plan's entries
+go to the step function as they are.
 
-Decoding one step ahead.  The host's share of a decode step (scheduling, block
-tables, the launch itself, waiting for the chosen tokens) is a good part of the
-step's time for a small model, and the GPU would idle through it.  So, before it
-waits for the tokens of step k, the engine launches step k+1 for the same requests
-with the token ids taken on the device from the sampler's output; nothing about
-that step counts yet.  When the scheduler, now knowing step k's tokens, asks for
-exactly that step, it is committed and only its tokens are waited for; when it
-asks for anything else (a request finished, another was admitted) the launch is
-abandoned: its pages go back, and what it wrote is overwritten by the steps that
-follow it on the stream.  Results, their order and the scheduler's decisions are
-those of the plain loop.
+Decoding one step ahead.  The host's share of a decode step (planning, block tables, the
+launch itself, waiting for the chosen tokens) is a good part of the step's time for a small
+model, and the GPU would idle through it.  So, before it waits for the tokens of step k, the
+engine launches step k+1 for the same requests with the token ids taken on the device from
+the sampler's output; nothing about that step counts yet.  When the scheduler, now knowing
+step k's tokens, plans exactly that step, it is committed and only its tokens are waited for;
+when it plans anything else (a request finished, another was admitted) the launch is
+abandoned: its pages go back, and what it wrote is overwritten by the steps that follow it on
+the stream.  Results, their order and the scheduler's decisions are those of the plain loop.
 """
 
 from __future__ import annotations
@@ -35,25 +32,20 @@ from typing import Callable, Collection, Iterator, Optional, Sequence, Union
 import torch
 
 from ..sampling.sampler import GREEDY, Sampler, SamplingParams
-from .admission import PagedBlockAdmissionController
+from .admission import PageAdmission
 from .config import EngineConfig
-from .metrics import RequestMetricsCollector
-from .runner import ModelRunner, StepEntry, StepOutput
-from .scheduler import (
-    BatchingPolicy,
-    RequestScheduler,
-    RequestState,
-    SchedulerBatch,
-    SchedulerStepUpdate,
-    WorkKind,
-)
+from .metrics import RequestTimes
+from .request import Request
+from .runner import ModelRunner, StepOutput
+from .scheduler import Scheduler, StepPlan, StepReport
 
 
 @contextmanager
-def _trace_range(enabled: bool, message: str) -> Iterator[None]:
-    """Optional roctx range (visible to rocprofv3); always popped, also on errors."""
+def _traced(enabled: bool, label: str) -> Iterator[None]:
+    """A named range for rocprofv3's marker trace; closed on errors too.  The names are the
+    reference's (engine.py:24-33, 170-281), so that traces of both read alike."""
     if enabled:
-        torch.cuda.nvtx.range_push(message)
+        torch.cuda.nvtx.range_push(label)
     try:
         yield
     finally:
@@ -61,53 +53,53 @@ def _trace_range(enabled: bool, message: str) -> Iterator[None]:
             torch.cuda.nvtx.range_pop()
 
 
-class _TokensOnTheWay:
-    """The chosen tokens of one step, being copied to the host.  The copy is put on the
-    stream right behind the sampling, BEFORE any later step is launched, and waited for by
-    its own event: waiting for it then does not wait for what was launched after it."""
+class _ChosenTokens:
+    """The tokens chosen in one step, on their way to the host.  The copy is put on the stream
+    right behind the sampling, BEFORE any later step is launched, and has an event of its own:
+    waiting for it does not wait for what was launched after it."""
 
-    _landing: list = []  # pinned host buffers that are not in use (allocating one costs a system call)
+    _spare: list = []  # pinned landing buffers not in use (making one costs a system call)
 
-    def __init__(self, chosen: torch.Tensor) -> None:
-        self.device_tokens = chosen
-        self._event = None
-        self._buffer = None
-        if chosen.device.type == "cuda":
-            count = chosen.numel()
-            pool = _TokensOnTheWay._landing
-            self._buffer = pool.pop() if pool and pool[-1].numel() >= count else torch.empty(
-                max(256, count), dtype=chosen.dtype, pin_memory=True
-            )
-            self._host = self._buffer[:count]
-            self._host.copy_(chosen, non_blocking=True)
-            self._event = torch.cuda.Event()
-            self._event.record(torch.cuda.current_stream(chosen.device))
-        else:
-            self._host = chosen
+    def __init__(self, on_device: torch.Tensor) -> None:
+        self.on_device = on_device
+        self._event = self._buffer = None
+        if on_device.device.type != "cuda":
+            self._host = on_device
+            return
+        count = on_device.numel()
+        spare = _ChosenTokens._spare
+        self._buffer = spare.pop() if spare and spare[-1].numel() >= count else torch.empty(
+            max(256, count), dtype=on_device.dtype, pin_memory=True
+        )
+        self._host = self._buffer[:count]
+        self._host.copy_(on_device, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record(torch.cuda.current_stream(on_device.device))
 
     def wait(self) -> list[int]:
         if self._event is not None:
             self._event.synchronize()
         tokens = self._host.tolist()
-        if self._buffer is not None:
-            if len(_TokensOnTheWay._landing) < 8:
-                _TokensOnTheWay._landing.append(self._buffer)
-            self._buffer = None
+        if self._buffer is not None and len(_ChosenTokens._spare) < 8:
+            _ChosenTokens._spare.append(self._buffer)
+        self._buffer = None
         return tokens
 
 
 @dataclass
-class _LaunchedAhead:
+class _Flight:
+    """A step that has been launched: what the step function returned and the chosen tokens."""
+
     request_ids: tuple[str, ...]
-    output: "StepOutput"
-    chosen: _TokensOnTheWay
+    output: StepOutput
+    chosen: Optional[_ChosenTokens]
 
 
 @dataclass(frozen=True)
 class EngineStepResult:
-    batch: SchedulerBatch
-    update: SchedulerStepUpdate
-    released_blocks: tuple[tuple[str, dict], ...]
+    plan: StepPlan
+    report: StepReport
+    released_blocks: tuple[tuple[str, dict], ...]  # (request, pages it held per pool) of the requests that ended
     started_ns: int
     tokens_ready_ns: int
     completed_ns: int
@@ -117,19 +109,20 @@ class ContinuousBatchEngine:
     def __init__(
         self,
         *,
-        scheduler: RequestScheduler,
+        scheduler: Scheduler,
         runner: ModelRunner,
-        admission: PagedBlockAdmissionController,
+        admission: PageAdmission,
         sampler: Optional[Sampler] = None,
         clock_ns: Callable[[], int] = time.perf_counter_ns,
-        metrics: Optional[RequestMetricsCollector] = None,
         enable_tracing: bool = False,
         lookahead: bool = True,
     ) -> None:
         if admission.manager is not runner.cache:
-            raise ValueError("the admission controller and the runner must share one cache manager")
+            raise ValueError("the admission and the runner must share one cache manager")
         if scheduler.max_running_requests > runner.cache.max_requests:
             raise ValueError("the scheduler may run more requests than the cache manager has slots")
+        if scheduler.cut_prompts and not runner.model.splittable:
+            raise ValueError("a part of this model needs whole prompts: the scheduler must not cut them (cut_prompts=False)")
         if enable_tracing and runner.device.type != "cuda":
             raise ValueError("tracing ranges need a GPU engine")
         self.scheduler = scheduler
@@ -137,10 +130,9 @@ class ContinuousBatchEngine:
         self.admission = admission
         self.sampler = sampler or Sampler(runner.ops, runner.device)
         self._clock_ns = clock_ns
-        self.metrics = metrics or RequestMetricsCollector()
         self.enable_tracing = enable_tracing
         self.lookahead = bool(lookahead)
-        self._ahead: Optional[_LaunchedAhead] = None
+        self._ahead: Optional[_Flight] = None
         self.lookahead_hits = 0
         self.lookahead_misses = 0
         self.lookahead_error: Optional[Exception] = None  # what switched the lookahead off, if anything did
@@ -150,7 +142,7 @@ class ContinuousBatchEngine:
     def manager(self):
         return self.admission.manager
 
-    # ---- construction from a model folder ------------------------------------------------------
+    # ---- from a model folder --------------------------------------------------------------------
     @classmethod
     def from_model_dir(
         cls,
@@ -162,8 +154,8 @@ class ContinuousBatchEngine:
     ) -> "ContinuousBatchEngine":
         """Model folder -> engine, set up by an `EngineConfig` (keyword arguments replace
         single fields of it).  `ops` replaces the HIP kernel library (tests on the CPU)."""
-        from ..models.registry import load_config
         from ..config.model_config import read_config_json
+        from ..models.registry import load_config
         from .factory import blocks_from_free_memory, default_ops, load_model, make_cache
 
         config = (config or EngineConfig()).with_overrides(**overrides)
@@ -194,13 +186,14 @@ class ContinuousBatchEngine:
             max_step_graphs=limits.max_step_graphs,
             max_graph_tokens=limits.max_step_tokens,
         )
-        admission = PagedBlockAdmissionController(cache, max_step_tokens=config.max_batch_tokens)
-        scheduler = RequestScheduler(
+        admission = PageAdmission(cache, max_step_tokens=config.max_batch_tokens)
+        scheduler = Scheduler(
             max_running_requests=config.max_running_requests,
             max_batch_tokens=config.max_batch_tokens,
             max_mixed_prefill_tokens=config.max_mixed_prefill_tokens,
-            admission_callback=admission.try_admit,
+            admit=admission.admit,
             batching_policy=config.batching_policy,
+            cut_prompts=model.splittable,  # a capability of the model's parts, not a choice of the caller
         )
         engine = cls(
             scheduler=scheduler,
@@ -212,7 +205,7 @@ class ContinuousBatchEngine:
         engine.config = config
         return engine
 
-    # ---- requests ---------------------------------------------------------------------------------
+    # ---- requests -------------------------------------------------------------------------------
     def submit(
         self,
         request_id: str,
@@ -222,183 +215,169 @@ class ContinuousBatchEngine:
         eos_token_ids: Union[int, Collection[int], None] = None,
         temperature: float = 0.0,
         seed: int = 0,
-    ) -> RequestState:
-        arrival_ns = self._clock_ns()
+    ) -> Request:
+        """Queue a request (names of the reference's entry point, engine.py:120-148).  Refused
+        here, before it is queued: tokens outside the vocabulary, more positions than the model
+        has, and a request that no empty page pool could hold (it would sit at the head of the
+        queue for good, and everything behind it with it)."""
+        arrived = self._clock_ns()
         vocab = self.runner.vocab_size
-        bad = [t for t in prompt_token_ids if isinstance(t, int) and t >= vocab]
-        if bad:
-            raise ValueError(f"prompt tokens outside the vocabulary of {vocab}: {bad[:5]}")
-        if len(prompt_token_ids) + max_new_tokens - 1 > self.runner.max_positions:
-            raise ValueError("prompt length + max_new_tokens - 1 exceeds max_position_embeddings")
-        # a request that no empty pool could hold would sit at the head of the queue for good,
-        # and everything behind it with it: it is refused here, before it is queued
+        outside = [t for t in prompt_token_ids if isinstance(t, int) and t >= vocab]
+        if outside:
+            raise ValueError(f"prompt tokens outside the vocabulary of {vocab}: {outside[:5]}")
         lifetime = len(prompt_token_ids) + max_new_tokens - 1
-        if not self.manager.can_ever_hold(lifetime, self.admission.max_step_tokens):
-            need = self.manager.lifetime_blocks(lifetime, self.admission.max_step_tokens)
+        if lifetime > self.runner.max_positions:
+            raise ValueError("prompt length + max_new_tokens - 1 exceeds max_position_embeddings")
+        if not self.admission.can_ever_admit(lifetime):
             have = [g.num_blocks for g in self.manager.groups]
             raise ValueError(
-                f"request {request_id!r} can never be admitted: it needs {need} pages per pool, the pools have {have}"
+                f"request {request_id!r} can never be admitted: it needs {list(self.admission.pages_for(lifetime))} "
+                f"pages per pool, the pools have {have}"
             )
         sampling = GREEDY if temperature == 0.0 else SamplingParams(float(temperature), int(seed))
-        request = self.scheduler.submit(
-            request_id,
-            prompt_token_ids,
-            max_new_tokens=max_new_tokens,
-            eos_token_ids=eos_token_ids,
-            sampling=sampling,
+        request = self.scheduler.add(
+            request_id, prompt_token_ids, max_new_tokens=max_new_tokens, stop_tokens=eos_token_ids, sampling=sampling
         )
-        self.metrics.register_request(request_id, arrival_ns)
+        request.timeline.stamp("arrived", arrived)
         return request
 
-    # ---- the loop -----------------------------------------------------------------------------------
+    def request(self, request_id: str) -> Request:
+        return self.scheduler.request(request_id)
+
+    def times(self, request_id: str) -> RequestTimes:
+        return RequestTimes.of(self.scheduler.request(request_id))
+
+    def all_times(self) -> tuple[RequestTimes, ...]:
+        return tuple(RequestTimes.of(r) for r in self.scheduler.requests)
+
+    # ---- one step -------------------------------------------------------------------------------
     @torch.inference_mode()
     def step(self) -> Optional[EngineStepResult]:
-        """Schedule and run one step; None when nothing can run."""
-        started_ns = self._clock_ns()
+        """Plan and run one step; None when nothing can run."""
+        started = self._clock_ns()
         try:
-            with _trace_range(self.enable_tracing, "scheduler.schedule_step"):
-                batch = self.scheduler.schedule_step()
+            with _traced(self.enable_tracing, "scheduler.schedule_step"):
+                plan = self.scheduler.plan()
         except BaseException:
-            self._drop_ahead()  # whatever the scheduler refused, no launched step stays open
+            self._abandon_ahead()  # whatever the scheduler refused, no launched step stays open
             raise
-        if batch is None:
-            self._drop_ahead()
+        if plan is None:
+            self._abandon_ahead()
             return None
-        label = (
-            f"engine.step:{batch.step_index}:prefill={len(batch.prefill_request_ids)}:"
-            f"decode={len(batch.decode_request_ids)}"
-        )
-        with _trace_range(self.enable_tracing, label):
-            return self._execute(batch, started_ns)
-
-    def _execute(self, batch: SchedulerBatch, started_ns: int) -> EngineStepResult:
-        try:
-            self.metrics.require_registered(tuple(i.request_id for i in batch.items))
-            entries = []
-            params: list[SamplingParams] = []
-            indices: list[int] = []
-            for item in batch.items:
-                request = self.scheduler.get_request(item.request_id)
-                if item.kind is WorkKind.PREFILL and item.start == 0:
-                    self.metrics.record_prefill_started(item.request_id, self._clock_ns())
-                want = (len(item.input_token_ids) - 1,) if item.produces_token else ()
-                entries.append(StepEntry(item.request_id, item.input_token_ids, want))
-                if item.produces_token:
-                    params.append(request.sampling)
-                    indices.append(len(request.generated_token_ids))
-            ahead = self._take_ahead(batch)
-            if ahead is not None:
-                output = self.runner.commit(ahead.output)
-                chosen = ahead.chosen
-            else:
-                with _trace_range(self.enable_tracing, f"model.step:tokens={batch.token_count}"):
-                    output = self.runner.step(entries, borrow_logits=True)  # sampled from right below
-                chosen = None
-                if output.logits is not None:
-                    chosen = _TokensOnTheWay(self.sampler.sample(output.logits, params, indices))
-        except BaseException:  # also an interrupt must not leave admitted requests and a batch behind
-            self._drop_ahead()
-            with _trace_range(self.enable_tracing, "engine.rollback"):
-                self.admission.release_admitted(batch.admitted_request_ids)
-                self.scheduler.abort_step()
-            raise
-
-        if self.lookahead and chosen is not None:
-            # step k is launched and counted; a failure to launch k+1 early must not undo it
+        label = f"engine.step:{plan.index}:prefill={len(plan.prompt_ids)}:decode={len(plan.decode_ids)}"
+        with _traced(self.enable_tracing, label):
             try:
-                with _trace_range(self.enable_tracing, "model.step:ahead"):
-                    self._ahead = self._launch_ahead(batch, output, chosen.device_tokens, params, indices)
-            except Exception as error:  # noqa: BLE001 - decoding goes on without the lookahead
-                self._ahead = None
-                self.lookahead = False
-                self.lookahead_error = error
-                warnings.warn(
-                    f"decoding one step ahead was switched off after {type(error).__name__}: {error}; "
-                    "steps go on one by one, which is slower",
-                    RuntimeWarning,
-                    stacklevel=2,
-                )
-        with _trace_range(self.enable_tracing, "token.d2h_sync"):
-            host_tokens = chosen.wait() if chosen is not None else []
-        tokens_ready_ns = self._clock_ns()
-        generated = {rid: int(tok) for (rid, _), tok in zip(output.rows, host_tokens)}
-        with _trace_range(self.enable_tracing, "scheduler.apply_and_release"):
-            update = self.scheduler.apply_step_results(generated)
-            if self._ahead is not None and set(update.finished_request_ids) & set(self._ahead.request_ids):
-                self._drop_ahead()  # it holds pages of a request that is about to be released
-            released = self.admission.release_finished(update.finished_request_ids)
-        completed_ns = self._clock_ns()
-        self.metrics.record_tokens(update.emitted_tokens, tokens_ready_ns)
-        self.metrics.record_completed(update.finished_request_ids, completed_ns)
-        return EngineStepResult(
-            batch=batch,
-            update=update,
-            released_blocks=tuple(released.items()),
-            started_ns=started_ns,
-            tokens_ready_ns=tokens_ready_ns,
-            completed_ns=completed_ns,
-        )
+                flight = self._fly(plan)
+            except BaseException:  # an interrupt, too, must not leave admitted requests and a plan behind
+                self._abandon_ahead()
+                with _traced(self.enable_tracing, "engine.rollback"):
+                    self.admission.release(plan.admitted)
+                    self.scheduler.cancel()
+                raise
+            if self.lookahead and flight.chosen is not None:
+                self._look_ahead(plan, flight)
+            with _traced(self.enable_tracing, "token.d2h_sync"):
+                tokens = flight.chosen.wait() if flight.chosen is not None else []
+            ready = self._clock_ns()
+            with _traced(self.enable_tracing, "scheduler.apply_and_release"):
+                report = self.scheduler.complete({rid: int(t) for (rid, _), t in zip(flight.output.rows, tokens)})
+                if self._ahead is not None and set(report.finished) & set(self._ahead.request_ids):
+                    self._abandon_ahead()  # it holds pages of a request that is about to be released
+                released = self.admission.release(report.finished)
+            completed = self._clock_ns()
+        for rid, _ in report.emitted:
+            self.scheduler.request(rid).timeline.stamp("token", ready)
+        for rid in report.finished:
+            self.scheduler.request(rid).timeline.stamp("done", completed)
+        return EngineStepResult(plan, report, tuple(released.items()), started, ready, completed)
 
-    # ---- the step launched ahead ----------------------------------------------------------------------
-    def _launch_ahead(self, batch, output: StepOutput, chosen, params, indices) -> Optional[_LaunchedAhead]:
-        """Launch the next step now if it is bound to be one token for each request of this
-        batch that goes on: all running requests produced a token here, nobody waits who could
-        be admitted, and those that end by length with this token are left out.  (A request may
-        still end on an end-of-sequence token; then the launch is abandoned.)"""
+    def _sampling_of(self, plan: StepPlan) -> tuple[list[SamplingParams], list[int]]:
+        """Sampling parameters and index of the token to come, for every slice that emits one."""
+        emitting = [s.request for s in plan.slices if s.emits]
+        return [r.sampling for r in emitting], [len(r.output) for r in emitting]
+
+    def _fly(self, plan: StepPlan) -> _Flight:
+        """Launch the plan's step: the one launched ahead if it is that step, else a new one."""
+        for part in plan.slices:
+            if part.from_prompt and part.offset == 0:
+                part.request.timeline.stamp("scheduled", self._clock_ns())
+        ahead = self._ahead
+        if ahead is not None:
+            same = not plan.admitted and not plan.prompt_ids and plan.decode_ids == ahead.request_ids
+            if same:
+                self._ahead = None
+                self.lookahead_hits += 1
+                ahead.output = self.runner.commit(ahead.output)
+                return ahead
+            self._abandon_ahead()
+        with _traced(self.enable_tracing, f"model.step:tokens={plan.token_count}"):
+            output = self.runner.step(plan.entries, borrow_logits=True)  # sampled from right below
+        chosen = None
+        if output.logits is not None:
+            chosen = _ChosenTokens(self.sampler.sample(output.logits, *self._sampling_of(plan)))
+        return _Flight(tuple(rid for rid, _ in output.rows), output, chosen)
+
+    # ---- the step launched ahead ------------------------------------------------------------------
+    def _look_ahead(self, plan: StepPlan, flight: _Flight) -> None:
+        """Launch the next step now if it is bound to be one token for each request of this step
+        that goes on: every active request emits a token here, nobody waits who could be let in,
+        and those that end by length with this token are left out.  (A request may still end on a
+        stop token; then the launch is abandoned.)  A failure here must not undo the step that is
+        already launched and counted: decoding goes on without looking ahead."""
+        try:
+            with _traced(self.enable_tracing, "model.step:ahead"):
+                self._ahead = self._launch_ahead(plan, flight)
+        except Exception as error:  # noqa: BLE001
+            self._ahead = None
+            self.lookahead = False
+            self.lookahead_error = error
+            warnings.warn(
+                f"decoding one step ahead was switched off after {type(error).__name__}: {error}; "
+                "steps go on one by one, which is slower",
+                RuntimeWarning,
+                stacklevel=2,
+            )
+
+    def _launch_ahead(self, plan: StepPlan, flight: _Flight) -> Optional[_Flight]:
         scheduler = self.scheduler
-        running = scheduler.running_request_ids
-        produced = [rid for rid, _ in output.rows]
-        if not running or sorted(running) != sorted(produced):
+        active = scheduler.active_ids
+        emitting = plan.emitting_ids
+        if not active or sorted(active) != sorted(emitting):
             return None
-        if scheduler.waiting_request_ids and len(running) < scheduler.max_running_requests:
+        if scheduler.queued_ids and len(active) < scheduler.max_running_requests:
             return None
-        by_id = {rid: i for i, rid in enumerate(produced)}
-        going_on = [rid for rid in running if indices[by_id[rid]] + 1 < scheduler.get_request(rid).max_new_tokens]
+        place = {rid: i for i, rid in enumerate(emitting)}
+        going_on = [rid for rid in active if len(scheduler.request(rid).output) + 1 < scheduler.request(rid).max_new_tokens]
         if not going_on:
             return None
-        order = [by_id[rid] for rid in going_on]
-        tokens = chosen
-        if order != list(range(len(produced))):
-            tokens = chosen[torch.tensor(order, dtype=torch.int64, device=chosen.device)]
+        picks = [place[rid] for rid in going_on]
+        tokens = flight.chosen.on_device
+        if picks != list(range(len(emitting))):
+            tokens = tokens[torch.tensor(picks, dtype=torch.int64, device=tokens.device)]
         launched = self.runner.launch_decode(going_on, tokens)
         if launched is None:
             return None
         try:
-            ahead = _TokensOnTheWay(
-                self.sampler.sample(launched.logits, [params[i] for i in order], [indices[i] + 1 for i in order])
+            requests = [scheduler.request(rid) for rid in going_on]
+            chosen = _ChosenTokens(
+                self.sampler.sample(launched.logits, [r.sampling for r in requests], [len(r.output) + 1 for r in requests])
             )
         except BaseException:
             self.runner.abort(launched)
             raise
-        return _LaunchedAhead(tuple(going_on), launched, ahead)
+        return _Flight(tuple(going_on), launched, chosen)
 
-    def _take_ahead(self, batch: SchedulerBatch) -> Optional[_LaunchedAhead]:
-        """The step launched ahead if `batch` is that step; otherwise it is abandoned."""
-        ahead = self._ahead
-        if ahead is None:
-            return None
-        same = (
-            not batch.admitted_request_ids
-            and all(i.kind is WorkKind.DECODE for i in batch.items)
-            and tuple(i.request_id for i in batch.items) == ahead.request_ids
-        )
-        if not same:
-            self._drop_ahead()
-            return None
-        self._ahead = None
-        self.lookahead_hits += 1
-        return ahead
-
-    def _drop_ahead(self) -> None:
+    def _abandon_ahead(self) -> None:
         if self._ahead is not None:
             ahead, self._ahead = self._ahead, None
             self.lookahead_misses += 1
             self.runner.abort(ahead.output)
 
+    # ---- to the end -----------------------------------------------------------------------------------
     def run_until_done(self) -> list[EngineStepResult]:
         """Step until every submitted request has finished."""
         results = []
-        while self.scheduler.has_unfinished_requests:
+        while self.scheduler.busy:
             result = self.step()
             if result is None:
                 raise RuntimeError("requests are unfinished but nothing can run: the page budget admits no progress")
@@ -415,16 +394,12 @@ class ContinuousBatchEngine:
         seed: int = 0,
     ) -> list[list[int]]:
         """Submit all prompts, run to completion, return each prompt's generated tokens."""
-        base = len(self.metrics.request_ids)
+        base = len(self.scheduler.requests)
         ids = [f"generate-{base + i}" for i in range(len(prompts))]
         for i, (rid, prompt) in enumerate(zip(ids, prompts)):
             self.submit(
-                rid,
-                list(prompt),
-                max_new_tokens=max_new_tokens,
-                eos_token_ids=eos_token_ids,
-                temperature=temperature,
-                seed=seed + i,
+                rid, list(prompt), max_new_tokens=max_new_tokens, eos_token_ids=eos_token_ids,
+                temperature=temperature, seed=seed + i,
             )
         self.run_until_done()
-        return [list(self.scheduler.get_request(rid).generated_token_ids) for rid in ids]
+        return [list(self.scheduler.request(rid).output) for rid in ids]

@@ -68,7 +68,7 @@ def page_bytes(model: DecoderModel, block_size: int, dtype: torch.dtype) -> int:
     total = 0
     for spec in model.site_cache_specs():
         if isinstance(spec, PagedKVSpec):
-            total += 2 * spec.num_kv_heads * spec.head_dim * block_size * width
+            total += spec.bytes_per_token(width) * block_size
     return total
 
 

@@ -1,21 +1,19 @@
-"""Single-request generation over the step function: one whole-prompt step, then
-one token per step.
+"""One request through the step function by itself: its prompt in one step, then a token per step.
 
-Same control loop and counts as the reference's `greedy_generate`
-(src/mini_llm_runtime/generation.py:29-117): N new tokens cost one prompt step and
-at most N-1 decode steps; the last generated token is never fed back, so the cache
-ends at prompt + N - 1 tokens (generation.py:41-42); capacity is checked before
-anything is written (generation.py:53-57, 74-80); EOS stops without a further step.
+The entry point and what it reports have the reference's names
+(src/mini_llm_runtime/generation.py:29-117): N new tokens cost one prompt step and at most
+N - 1 decode steps; the last generated token is never fed back, so the cache ends at
+prompt + N - 1 tokens (generation.py:41-42); room in the cache is checked before anything is
+written (generation.py:53-57, 74-80); a stop token ends the run without a further step.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Collection, Optional, Sequence, Union
+from typing import Collection, Iterator, Optional, Sequence, Union
 
 import torch
 
-from ..cache.block_pool import blocks_for
 from ..sampling.sampler import GREEDY, Sampler, SamplingParams
 from .runner import ModelRunner, StepEntry
 
@@ -30,14 +28,27 @@ class GenerationOutput:
     step_logits: Optional[tuple[torch.Tensor, ...]] = None
 
 
-def _normalize_eos(eos_token_ids: Union[int, Collection[int], None], vocab_size: int) -> frozenset[int]:
+def _stop_set(eos_token_ids: Union[int, Collection[int], None], vocab_size: int) -> frozenset[int]:
     if eos_token_ids is None:
         return frozenset()
-    values = {eos_token_ids} if isinstance(eos_token_ids, int) else {int(t) for t in eos_token_ids}
-    invalid = sorted(t for t in values if not 0 <= t < vocab_size)
-    if invalid:
-        raise ValueError(f"EOS token ids outside the vocabulary: {invalid}")
-    return frozenset(values)
+    stops = frozenset([eos_token_ids] if isinstance(eos_token_ids, int) else (int(t) for t in eos_token_ids))
+    outside = sorted(t for t in stops if not 0 <= t < vocab_size)
+    if outside:
+        raise ValueError(f"EOS token ids outside the vocabulary: {outside}")
+    return stops
+
+
+def _token_stream(
+    runner: ModelRunner, sampler: Sampler, request_id: str, prompt: Sequence[int], sampling: SamplingParams, limit: int
+) -> Iterator[tuple[int, torch.Tensor]]:
+    """(token, the logits it was chosen from) for up to `limit` tokens; every `next` runs one
+    step: the prompt first, then the token chosen last."""
+    feed = list(prompt)
+    for index in range(limit):
+        out = runner.step([StepEntry.of(request_id, feed, (len(feed) - 1,))], borrow_logits=True)
+        token = int(sampler.sample(out.logits, [sampling], [index]).cpu()[0])
+        yield token, out.logits[0]
+        feed = [token]
 
 
 @torch.inference_mode()
@@ -56,48 +67,41 @@ def generate(
         raise ValueError("the prompt must not be empty")
     if max_new_tokens <= 0:
         raise ValueError("max_new_tokens must be > 0")
-    required = len(prompt) + max_new_tokens - 1
-    if required > runner.max_positions:
+    most_cached = len(prompt) + max_new_tokens - 1
+    if most_cached > runner.max_positions:
         raise ValueError("prompt length + max_new_tokens - 1 exceeds max_position_embeddings")
-    eos = _normalize_eos(eos_token_ids, runner.vocab_size)
+    stops = _stop_set(eos_token_ids, runner.vocab_size)
     cache = runner.cache
     for group in cache.groups:
-        need = group.lifetime_blocks(required, len(prompt))
+        need = group.lifetime_blocks(most_cached, len(prompt))
         if need > group.allocator.available_count:
             raise RuntimeError(
                 f"the cache has {group.allocator.available_count} free pages in group {group.index}, "
                 f"generation needs {need}"
             )
-    sampler = Sampler(runner.ops, runner.device)
-    cache.create_request(request_id)
-    generated: list[int] = []
-    captured: Optional[list[torch.Tensor]] = [] if return_step_logits else None
+    tokens: list[int] = []
+    kept: list[torch.Tensor] = []
     stopped = False
-    decode_steps = 0
+    cache.create_request(request_id)
     try:
-        tokens = prompt
-        for index in range(max_new_tokens):
-            out = runner.step([StepEntry.of(request_id, tokens, (len(tokens) - 1,))], borrow_logits=True)
-            if captured is not None:
-                captured.append(out.logits[0].clone())
-            nxt = int(sampler.sample(out.logits, [sampling], [index]).cpu()[0])
-            generated.append(nxt)
-            if index > 0:
-                decode_steps += 1
-            stopped = nxt in eos
-            if stopped or index == max_new_tokens - 1:
-                break
-            tokens = [nxt]
-        cache_length = cache.get_request(request_id).num_tokens
+        stream = _token_stream(runner, Sampler(runner.ops, runner.device), request_id, prompt, sampling, max_new_tokens)
+        for token, logits in stream:
+            tokens.append(token)
+            if return_step_logits:
+                kept.append(logits.clone())  # the step's buffer may be a recording's own
+            if token in stops:
+                stopped = True
+                break  # before the stream feeds it back: no step is spent on a stop token
+        cached = cache.get_request(request_id).num_tokens
     finally:
         cache.release_request(request_id)
     return GenerationOutput(
-        generated_token_ids=tuple(generated),
+        generated_token_ids=tuple(tokens),
         stopped_by_eos=stopped,
         prefill_tokens=len(prompt),
-        decode_steps=decode_steps,
-        cache_length=cache_length,
-        step_logits=tuple(captured) if captured is not None else None,
+        decode_steps=len(tokens) - 1,
+        cache_length=cached,
+        step_logits=tuple(kept) if return_step_logits else None,
     )
 
 
@@ -120,4 +124,4 @@ def greedy_generate(
     )
 
 
-__all__ = ["GenerationOutput", "generate", "greedy_generate", "blocks_for"]
+__all__ = ["GenerationOutput", "generate", "greedy_generate"]

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "mlr_embedding": ([_VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
+    "mlr_scale_softcap": ([_VP, _F, _F, _I64, _VP], _I),
     "mlr_gather_rows": ([_VP, _VP, _VP, _I, _I64, _I, _I, _VP], _I),
     "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
@@ -236,9 +237,17 @@ class HipOps:
         return out
 
     def add_(self, x: torch.Tensor, delta: torch.Tensor) -> None:
+        """x (float32) += delta (the engine's dtype, or float32), in place."""
         self._check(x, "residual stream", torch.float32)
-        self._check(delta, "residual delta", self.dtype, tuple(x.shape))
-        self._call("mlr_add", self._ptr(x), self._ptr(delta), self.code, x.numel(), self._stream())
+        self._check(delta, "residual delta", (self.dtype, torch.float32), tuple(x.shape))
+        self._call("mlr_add", self._ptr(x), self._ptr(delta), _dtype_code(delta.dtype), x.numel(), self._stream())
+
+    def scale_softcap_(self, x: torch.Tensor, scale: float = 1.0, cap: Optional[float] = None) -> None:
+        """x (float32) = x * scale, then, with a cap, cap * tanh(x / cap); in place."""
+        self._check(x, "values", torch.float32)
+        if cap is not None and not cap > 0:
+            raise KernelError("a soft cap must be > 0")
+        self._call("mlr_scale_softcap", self._ptr(x), float(scale), float(cap or 0.0), x.numel(), self._stream())
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
         """x[rows] for x [T, H], or x[:, rows] for a stack [S, T, H]."""
@@ -453,6 +462,7 @@ class HipOps:
         return cos, sin
 
     def _check_pages(self, key_pages, value_pages, num_kv_heads, head_dim, block_size) -> int:
+        """Pages as the attention kernels read them: values as wide as keys."""
         self._check(key_pages, "key pages", self.dtype, (None, num_kv_heads, block_size, head_dim))
         self._check(value_pages, "value pages", self.dtype, (key_pages.shape[0], num_kv_heads, head_dim, block_size))
         return key_pages.shape[0]

@@ -27,6 +27,9 @@ class Part:
     # and to nothing else may say so: it then may receive a norm that has not run yet (which
     # those operations run, fused into their own kernel where they can) instead of a tensor.
     takes_pending_norm = False
+    # False for a part that needs a request's whole prompt in one step (it cannot go on from a
+    # cached prefix): the scheduler then never cuts prompts of a model that holds it.
+    splittable = True
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}
@@ -63,6 +66,11 @@ class PositionEncoding(Part):
 
     def apply(self, ctx: StepContext, q: torch.Tensor, k: torch.Tensor) -> None:
         """Encode positions into q [T, Hq, d] and k [T, Hkv, d] in place."""
+        raise NotImplementedError
+
+    def embed(self, ctx: StepContext) -> torch.Tensor:
+        """[T, hidden] (float32 or the engine's dtype) to be added to the embedded tokens, for an
+        encoding that a model names as its `position_embedding`."""
         raise NotImplementedError
 
 

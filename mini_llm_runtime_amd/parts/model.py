@@ -36,8 +36,12 @@ class DecoderModel:
         self.spec = spec
         self.layers: list[Block] = [_build_layer(s) for s in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm)
+        self.position_embedding = (
+            build_part("position", spec.position_embedding) if spec.position_embedding is not None else None
+        )
         self.embed_weight: Optional[torch.Tensor] = None
         self.head_weight: Optional[torch.Tensor] = None
+        self.head_bias: Optional[torch.Tensor] = None
         self.dtype: Optional[torch.dtype] = None
         self.device: Optional[torch.device] = None
         if not spec.order:
@@ -77,10 +81,17 @@ class DecoderModel:
         """Every part says that its steps can be recorded and replayed (`Part.replayable`)."""
         return all(part.replayable for _, part in self.named_parts())
 
+    @property
+    def splittable(self) -> bool:
+        """Every part can go on from a cached prefix, so prompts may be cut into portions."""
+        return all(part.splittable for _, part in self.named_parts())
+
     def named_parts(self) -> Iterator[tuple[str, Part]]:
         for i, layer in enumerate(self.layers):
             yield from _walk(f"layers.{i}", layer)
         yield from _walk("final_norm", self.final_norm)
+        if self.position_embedding is not None:
+            yield from _walk("position_embedding", self.position_embedding)
 
     def param_specs(self) -> dict[str, ParamSpec]:
         specs: dict[str, ParamSpec] = {
@@ -88,6 +99,8 @@ class DecoderModel:
         }
         if not self.spec.tie_word_embeddings:
             specs["head.weight"] = ParamSpec((self.spec.vocab_size, self.spec.hidden_size))
+        if self.spec.head_bias:
+            specs["head.bias"] = ParamSpec((self.spec.vocab_size,), keep_stored_precision=True)
         for path, part in self.named_parts():
             for name, p in part.param_specs().items():
                 specs[f"{path}.{name}"] = p
@@ -104,13 +117,14 @@ class DecoderModel:
         self.device = torch.device(device)
         self.embed_weight = params["embed.weight"]
         self.head_weight = params["embed.weight"] if self.spec.tie_word_embeddings else params["head.weight"]
+        self.head_bias = params.get("head.bias")
         for path, part in self.named_parts():
             own = {name: params[f"{path}.{name}"] for name in part.param_specs()}
             part.bind(own, dtype=dtype, device=self.device)
 
     def weight_bytes(self) -> int:
         seen: dict[int, int] = {}
-        tensors = [self.embed_weight, self.head_weight]
+        tensors = [self.embed_weight, self.head_weight, self.head_bias]
         for _, part in self.named_parts():
             tensors.extend(getattr(part, name) for name in part.param_specs())
         for t in tensors:
@@ -133,7 +147,12 @@ class DecoderModel:
         finding the layer at which a wrong logit first appears; it adds a few small kernels
         per site and is never recorded into a graph."""
         ops = ctx.ops
+        spec = self.spec
         x = ops.embedding(self.embed_weight, ctx.token_ids)
+        if spec.embedding_scale != 1.0:
+            ops.scale_softcap_(x, spec.embedding_scale)
+        if self.position_embedding is not None:
+            ops.add_(x, self.position_embedding.embed(ctx))
         delta: Optional[torch.Tensor] = None
         capture = site_outputs is not None and logit_rows is not None and logit_rows.numel() > 0
         for site, entry in enumerate(self.spec.order):
@@ -153,7 +172,10 @@ class DecoderModel:
             rows = ops.gather_rows(x, logit_rows)
             delta_rows = ops.gather_rows(delta, logit_rows) if delta is not None else None
         h = self.final_norm.forward(ctx, rows, delta_rows)
-        return ops.linear(h, self.head_weight, None, out_dtype=torch.float32)
+        logits = ops.linear(h, self.head_weight, self.head_bias, out_dtype=torch.float32)
+        if spec.logit_scale != 1.0 or spec.logit_softcap is not None:
+            ops.scale_softcap_(logits, spec.logit_scale, spec.logit_softcap)
+        return logits
 
 
 def site_spec_kinds(model: DecoderModel) -> tuple[int, int]:

@@ -60,7 +60,14 @@ class WeightRule:
     interleaved instead: source row i goes to row_start + (i // block) * period +
     i % block (two matrices woven together in groups of `block` rows).  `optional`
     tensors may be absent; when `must_equal` names another parameter, a present
-    tensor has to equal it (a tied head stored a second time)."""
+    tensor has to equal it (a tied head stored a second time).
+
+    A rule may take only a part of the stored tensor, and several rules may read the same
+    tensor (a checkpoint that stores q, k and v as one matrix, or all experts stacked):
+    `source_index` picks [index] of the leading dimension, `transpose` swaps a matrix that is
+    stored [in, out], `source_rows` = (first, count) then takes rows of what is left, in that
+    order.  `source_shape` is the stored tensor's whole shape; it is needed whenever the part
+    taken is not the whole tensor."""
 
     name: str
     dest: str
@@ -70,6 +77,39 @@ class WeightRule:
     must_equal: Optional[str] = None
     block: int = 0
     period: int = 0
+    source_shape: Optional[tuple[int, ...]] = None
+    source_index: Optional[int] = None
+    source_rows: Optional[tuple[int, int]] = None
+    transpose: bool = False
+
+    def part_shape(self, stored: tuple[int, ...]) -> tuple[int, ...]:
+        """Shape of what this rule takes of a stored tensor of shape `stored`."""
+        shape = tuple(stored)
+        if self.source_index is not None:
+            if not shape or not 0 <= self.source_index < shape[0]:
+                raise ValueError(f"weight rule {self.name!r}: source_index {self.source_index} is outside {shape}")
+            shape = shape[1:]
+        if self.transpose:
+            if len(shape) != 2:
+                raise ValueError(f"weight rule {self.name!r}: only matrices can be transposed, found {shape}")
+            shape = shape[::-1]
+        if self.source_rows is not None:
+            first, count = self.source_rows
+            if not shape or first < 0 or count <= 0 or first + count > shape[0]:
+                raise ValueError(f"weight rule {self.name!r}: source_rows {self.source_rows} are outside {shape}")
+            shape = (count, *shape[1:])
+        return shape
+
+    def take(self, tensor):
+        """The part of the stored tensor this rule feeds its destination with."""
+        if self.source_index is not None:
+            tensor = tensor[self.source_index]
+        if self.transpose:
+            tensor = tensor.t()
+        if self.source_rows is not None:
+            first, count = self.source_rows
+            tensor = tensor[first : first + count]
+        return tensor
 
     def dest_rows(self, count: int) -> "list[int]":
         """Destination row of each of `count` source rows."""
@@ -92,3 +132,9 @@ class ModelSpec:
     tie_word_embeddings: bool
     weight_rules: tuple[WeightRule, ...]
     init_std: float = 0.02
+    # What some decoders do around the layers; the defaults do nothing.
+    embedding_scale: float = 1.0  # the embedded tokens times this
+    position_embedding: Optional[PartSpec] = None  # a position part whose `embed` is added to the embedded tokens
+    head_bias: bool = False  # logits += parameter `head.bias`
+    logit_scale: float = 1.0  # logits times this ...
+    logit_softcap: Optional[float] = None  # ... then cap * tanh(logits / cap)

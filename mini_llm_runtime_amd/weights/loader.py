@@ -82,25 +82,55 @@ def checkpoint_files(model_dir: Union[str, Path]) -> dict[str, SafetensorsFile]:
     raise FileNotFoundError(f"no model.safetensors in {model_dir}")
 
 
-def expected_tensors(model: DecoderModel) -> dict[str, tuple[WeightRule, tuple[int, ...], ParamSpec]]:
-    """Checkpoint tensor name -> (rule, shape it must have, the parameter it feeds)."""
+def _stored_shape(rule: WeightRule, p: ParamSpec) -> tuple[int, ...]:
+    """Shape the checkpoint tensor of a rule must have; the part the rule takes of it must be
+    what the destination rows want."""
+    part = p.shape if rule.rows is None else (rule.rows, *p.shape[1:])
+    if rule.source_shape is not None:
+        stored = tuple(rule.source_shape)
+    elif rule.source_index is not None or rule.source_rows is not None:
+        raise ValueError(f"weight rule {rule.name!r} takes a part of its tensor and must give source_shape")
+    else:
+        stored = tuple(part[::-1]) if rule.transpose else tuple(part)
+    if rule.part_shape(stored) != tuple(part):
+        raise ValueError(
+            f"weight rule {rule.name!r}: it takes {rule.part_shape(stored)} of the stored {stored}, "
+            f"{rule.dest} wants {tuple(part)}"
+        )
+    return stored
+
+
+def rules_by_tensor(model: DecoderModel) -> dict[str, list[tuple[WeightRule, tuple[int, ...], ParamSpec]]]:
+    """Checkpoint tensor name -> the rules that read it, each with the shape the stored tensor
+    must have and the parameter it feeds.  Rules that share a tensor must agree on its shape."""
     specs = model.param_specs()
-    out = {}
+    out: dict[str, list] = {}
     for rule in model.spec.weight_rules:
         if rule.dest not in specs:
             raise KeyError(f"weight rule {rule.name!r} feeds {rule.dest!r}, which the model does not have")
         p = specs[rule.dest]
-        shape = p.shape if rule.rows is None else (rule.rows, *p.shape[1:])
-        if rule.name in out:
-            raise KeyError(f"two weight rules read {rule.name!r}")
-        out[rule.name] = (rule, tuple(shape), p)
+        shape = _stored_shape(rule, p)
+        readers = out.setdefault(rule.name, [])
+        if readers:
+            if readers[0][1] != shape:
+                raise ValueError(f"the rules that read {rule.name!r} expect different shapes: {readers[0][1]} and {shape}")
+            if rule.must_equal is not None or readers[0][0].must_equal is not None:
+                raise KeyError(f"{rule.name!r}: a tensor that only repeats a parameter cannot feed another")
+            if rule.optional != readers[0][0].optional:
+                raise KeyError(f"the rules that read {rule.name!r} disagree on whether it may be absent")
+        readers.append((rule, shape, p))
     return out
+
+
+def expected_tensors(model: DecoderModel) -> dict[str, tuple[WeightRule, tuple[int, ...], ParamSpec]]:
+    """Checkpoint tensor name -> (its first rule, shape it must have, the parameter that rule feeds)."""
+    return {name: readers[0] for name, readers in rules_by_tensor(model).items()}
 
 
 def _check_coverage(model: DecoderModel) -> None:
     """Every row of every parameter must be fed by exactly one rule."""
     specs = model.param_specs()
-    covered: dict[str, list[tuple[int, int]]] = {name: [] for name in specs}
+    covered: dict[str, list[int]] = {name: [] for name in specs}
     for rule in model.spec.weight_rules:
         if rule.must_equal is not None:
             continue
@@ -124,6 +154,7 @@ def load_weights(
         raise ValueError("the engine's dtype is bfloat16 or float32")
     device = torch.device(device)
     _check_coverage(model)
+    readers = rules_by_tensor(model)  # rules that do not fit their parameters fail here, before a file is opened
     files = checkpoint_files(model_dir)
     try:
         found: dict[str, TensorEntry] = {}
@@ -133,7 +164,7 @@ def load_weights(
                 if name in found:
                     duplicates.append(f"{name} is stored in two files")
                 found[name] = entry
-        expected = expected_tensors(model)
+        expected = {name: rules[0] for name, rules in readers.items()}
         missing = [n for n, (rule, _, _) in expected.items() if n not in found and not rule.optional]
         unexpected = [n for n in found if n not in expected]
         wrong = [
@@ -144,9 +175,10 @@ def load_weights(
 
         specs = model.param_specs()
         sources: dict[str, list[TensorEntry]] = {name: [] for name in specs}
-        for n, (rule, _, _) in expected.items():
-            if n in found and rule.must_equal is None:
-                sources[rule.dest].append(found[n])
+        for n, rules in readers.items():
+            for rule, _, _ in rules:
+                if n in found and rule.must_equal is None:
+                    sources[rule.dest].append(found[n])
         params: dict[str, torch.Tensor] = {}
         for name, p in specs.items():
             stored = sources[name]
@@ -160,21 +192,23 @@ def load_weights(
 
         by_file = {f.path: f for f in files.values()}
         checks = []
-        for n, (rule, shape, _) in expected.items():
+        for n, rules in readers.items():
             if n not in found:
                 continue
             entry = found[n]
-            tensor = by_file[entry.file].tensor(n)
-            if rule.must_equal is not None:
-                checks.append((n, rule.must_equal, tensor))
-                continue
-            dest = params[rule.dest]
-            rows = dest.shape[0] if rule.rows is None else rule.rows
-            if rule.block:
-                index = torch.tensor(rule.dest_rows(rows), dtype=torch.long, device=dest.device)
-                dest.index_copy_(0, index, tensor.to(dest.dtype).to(dest.device))
-            else:
-                dest[rule.row_start : rule.row_start + rows].copy_(tensor.to(dest.dtype))
+            stored = by_file[entry.file].tensor(n)
+            for rule, _, _ in rules:
+                if rule.must_equal is not None:
+                    checks.append((n, rule.must_equal, stored))
+                    continue
+                tensor = rule.take(stored)
+                dest = params[rule.dest]
+                rows = dest.shape[0] if rule.rows is None else rule.rows
+                if rule.block:
+                    index = torch.tensor(rule.dest_rows(rows), dtype=torch.long, device=dest.device)
+                    dest.index_copy_(0, index, tensor.to(dest.dtype).to(dest.device))
+                else:
+                    dest[rule.row_start : rule.row_start + rows].copy_(tensor.to(dest.dtype))
         for n, other, tensor in checks:
             ref = params[other]
             if not torch.equal(tensor.to(ref.dtype).to(ref.device), ref):

@@ -42,6 +42,11 @@ class TorchOps:
     def add_(self, x, delta):
         x += delta.float()
 
+    def scale_softcap_(self, x, scale=1.0, cap=None):
+        x *= scale
+        if cap is not None:
+            x.copy_(cap * torch.tanh(x / cap))
+
     def gather_rows(self, x, rows):
         return (x[:, rows.long()] if x.dim() == 3 else x[rows.long()]).contiguous()
 

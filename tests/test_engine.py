@@ -16,8 +16,8 @@ from mini_llm_runtime_amd.engine import (
     BatchingPolicy,
     ContinuousBatchEngine,
     ModelRunner,
-    PagedBlockAdmissionController,
-    RequestScheduler,
+    PageAdmission,
+    Scheduler,
 )
 
 CASES = [
@@ -109,15 +109,15 @@ def test_continuous_batching_with_late_arrivals(tmp_path, backend, dtype):
         for rid, at in arrivals.items():
             if at == step:
                 engine.submit(rid, prompts[rid], max_new_tokens=12)
-        if not engine.scheduler.has_unfinished_requests and step > max(arrivals.values()):
+        if not engine.scheduler.busy and step > max(arrivals.values()):
             break
         result = engine.step()
         step += 1
         if result is None:
             continue
-        b = result.batch
-        saw_mixed |= bool(b.decode_request_ids) and bool(b.prefill_request_ids)
-        saw_portion |= any(not i.produces_token for i in b.items)
+        b = result.plan
+        saw_mixed |= bool(b.decode_ids) and bool(b.prompt_ids)
+        saw_portion |= any(not p.emits for p in b.slices)
         held = {p for rid in engine.manager.request_ids for p in engine.manager.get_request(rid).live_blocks(0)}
         reused |= held & freed
         for _, blocks in result.released_blocks:
@@ -125,13 +125,16 @@ def test_continuous_batching_with_late_arrivals(tmp_path, backend, dtype):
         engine.manager.check_invariants()
     assert saw_mixed and saw_portion and reused, "the workload must mix, cut prompts and use pages again"
     for rid, prompt in prompts.items():
-        tokens = engine.scheduler.get_request(rid).generated_token_ids
+        tokens = engine.request(rid).generated
         assert len(tokens) == 12
         _check_greedy(tokens, prompt, w, cfg, dtype)
-    assert engine.manager.request_ids == () and engine.admission.reservations == ()
+    assert engine.manager.request_ids == () and engine.admission.promises == ()
     assert engine.manager.groups[0].allocator.free_count == 40
-    m = engine.metrics.snapshot("r4")
-    assert m.ttft_ns > 0 and len(m.inter_token_ns) == 11 and m.e2e_ns >= m.ttft_ns
+    line = engine.request("r4").timeline
+    assert line.ttft_ns > 0 and len(line.gaps_ns) == 11 and line.e2e_ns >= line.ttft_ns and line.cleanup_ns >= 0
+    m = engine.times("r4")
+    assert m.tokens == 12 and m.ttft_ms == line.ttft_ns / 1e6 and m.queue_wait_ms >= 0
+    assert len(engine.all_times()) == 5
 
 
 @pytest.mark.parametrize("backend,dtype", CASES[:2])
@@ -146,7 +149,7 @@ def test_temperature_sampling_is_reproducible_and_independent_of_the_batch(tmp_p
         for i in which:
             engine.submit(f"s{i}", prompts[i], max_new_tokens=10, temperature=0.8, seed=1000 + i)
         engine.run_until_done()
-        return {i: engine.scheduler.get_request(f"s{i}").generated_token_ids for i in which}
+        return {i: engine.request(f"s{i}").generated for i in which}
 
     together = run([0, 1, 2], 3)
     again = run([0, 1, 2], 3)
@@ -170,20 +173,20 @@ def test_pages_run_out_requests_wait_then_enter(tmp_path, backend, dtype):
     engine.submit("big", p1, max_new_tokens=4)  # 13 tokens -> 4 pages
     engine.submit("late", p2, max_new_tokens=3)  # 11 tokens -> 3 pages: does not fit beside "big"
     first = engine.step()
-    assert first.batch.prefill_request_ids == ("big",) and engine.scheduler.waiting_request_ids == ("late",)
+    assert first.plan.prompt_ids == ("big",) and engine.scheduler.queued_ids == ("late",)
     order = []
-    while engine.scheduler.has_unfinished_requests:
+    while engine.scheduler.busy:
         r = engine.step()
-        order.append((r.batch.prefill_request_ids, r.update.finished_request_ids))
+        order.append((r.plan.prompt_ids, r.report.finished))
     assert any(p == ("late",) for p, _ in order)
     done_big = next(i for i, (_, f) in enumerate(order) if "big" in f)
     enter_late = next(i for i, (p, _) in enumerate(order) if p == ("late",))
     assert enter_late == done_big + 1  # the step after the pages came back
-    _check_greedy(engine.scheduler.get_request("late").generated_token_ids, p2, w, cfg, dtype)
+    _check_greedy(engine.request("late").generated, p2, w, cfg, dtype)
     # 27 tokens -> 7 pages > 6: refused when it is submitted, so it never blocks the queue
     with pytest.raises(ValueError, match="never"):
         engine.submit("never", random_tokens(20, cfg["vocab_size"], 3), max_new_tokens=8)
-    assert "never" not in engine.scheduler.waiting_request_ids and engine.step() is None
+    assert "never" not in engine.scheduler.queued_ids and engine.step() is None
 
 
 @pytest.mark.parametrize("backend,dtype", CASES[:2])
@@ -202,16 +205,16 @@ def test_failed_step_rolls_back_and_can_be_retried(tmp_path, backend, dtype):
     engine.runner.fail_next_step = RuntimeError("injected")
     with pytest.raises(RuntimeError, match="injected"):
         engine.step()
-    assert engine.scheduler.waiting_request_ids == ("C",) and engine.scheduler.running_request_ids == ("A",)
-    assert not engine.manager.has_request("C") and engine.admission.reservations[0].request_id == "A"
+    assert engine.scheduler.queued_ids == ("C",) and engine.scheduler.active_ids == ("A",)
+    assert not engine.manager.has_request("C") and engine.admission.promises[0].request_id == "A"
     assert (engine.manager.get_request("A").num_tokens, engine.manager.groups[0].allocator.free_count) == before
     engine.manager.check_invariants()
     retry = engine.step()
-    assert retry.batch.step_index == 1
-    assert retry.batch.decode_request_ids == ("A",) and retry.batch.prefill_request_ids == ("C",)
+    assert retry.plan.index == 1
+    assert retry.plan.decode_ids == ("A",) and retry.plan.prompt_ids == ("C",)
     engine.run_until_done()
-    _check_greedy(engine.scheduler.get_request("A").generated_token_ids, pa, w, cfg, dtype)
-    _check_greedy(engine.scheduler.get_request("C").generated_token_ids, pc, w, cfg, dtype)
+    _check_greedy(engine.request("A").generated, pa, w, cfg, dtype)
+    _check_greedy(engine.request("C").generated, pc, w, cfg, dtype)
 
 
 @pytest.mark.gpu
@@ -239,19 +242,19 @@ def test_decoding_one_step_ahead_changes_nothing_but_the_waiting(tmp_path, dtype
                 if at == step:
                     engine.submit(rid, prompts[rid], max_new_tokens=24, temperature=0.7 if rid == "r1" else 0.0,
                                   seed=5, eos_token_ids=eos)
-            if not engine.scheduler.has_unfinished_requests and step > max(arrivals.values()):
+            if not engine.scheduler.busy and step > max(arrivals.values()):
                 break
             result = engine.step()
             step += 1
             if result is not None:
-                trace.append((tuple((i.request_id, i.kind.value, i.input_token_ids) for i in result.batch.items),
-                              result.update.emitted_tokens, result.update.finished_request_ids, result.released_blocks))
+                trace.append((tuple((p.request_id, p.from_prompt, p.tokens) for p in result.plan.slices),
+                              result.report.emitted, result.report.finished, result.released_blocks))
         assert engine.lookahead_error is None
-        assert engine.manager.request_ids == () and engine.admission.reservations == ()
+        assert engine.manager.request_ids == () and engine.admission.promises == ()
         assert not engine.manager.step_in_flight
         engine.manager.check_invariants()
         assert engine.manager.groups[0].allocator.free_count == 30
-        tokens = {rid: engine.scheduler.get_request(rid).generated_token_ids for rid in prompts}
+        tokens = {rid: engine.request(rid).generated for rid in prompts}
         return tokens, trace, engine
 
     plain_tokens, _, _ = run(False, None)
@@ -275,7 +278,7 @@ def test_static_policy_does_not_refill(tmp_path):
     engine.step()
     engine.submit("B", [4, 5], max_new_tokens=2)
     r = engine.step()
-    assert r.batch.prefill_request_ids == () and r.batch.decode_request_ids == ("A",)
+    assert r.plan.prompt_ids == () and r.plan.decode_ids == ("A",)
 
 
 def test_engine_checks_its_wiring(tmp_path):
@@ -285,13 +288,13 @@ def test_engine_checks_its_wiring(tmp_path):
     cache = mlr.make_cache(model, block_size=4, num_blocks=8, max_requests=2)
     other = mlr.make_cache(model, block_size=4, num_blocks=8, max_requests=2)
     runner = ModelRunner(model, cache, ops)
-    sched = RequestScheduler(max_running_requests=2, max_batch_tokens=8)
+    sched = Scheduler(max_running_requests=2, max_batch_tokens=8)
     with pytest.raises(ValueError, match="share one cache"):
-        ContinuousBatchEngine(scheduler=sched, runner=runner, admission=PagedBlockAdmissionController(other, max_step_tokens=8))
-    big = RequestScheduler(max_running_requests=3, max_batch_tokens=8)
+        ContinuousBatchEngine(scheduler=sched, runner=runner, admission=PageAdmission(other, max_step_tokens=8))
+    big = Scheduler(max_running_requests=3, max_batch_tokens=8)
     with pytest.raises(ValueError, match="slots"):
-        ContinuousBatchEngine(scheduler=big, runner=runner, admission=PagedBlockAdmissionController(cache, max_step_tokens=8))
-    engine = ContinuousBatchEngine(scheduler=sched, runner=runner, admission=PagedBlockAdmissionController(cache, max_step_tokens=8))
+        ContinuousBatchEngine(scheduler=big, runner=runner, admission=PageAdmission(cache, max_step_tokens=8))
+    engine = ContinuousBatchEngine(scheduler=sched, runner=runner, admission=PageAdmission(cache, max_step_tokens=8))
     with pytest.raises(ValueError, match="vocabulary"):
         engine.submit("x", [TINY["A"]["vocab_size"]], max_new_tokens=1)
     with pytest.raises(ValueError, match="max_position"):
