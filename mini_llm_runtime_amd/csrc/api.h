@@ -70,8 +70,9 @@ int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_
 // mlr_gemm_bf16_slices returned for this shape) y is float32 [slices, m, n]: partial
 // sums over slices of k, the bias in slice 0, for the consumer to add up in order.
 int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
-// `kernel` 0 lets the shape choose; 16 (streaming, up to 16 tokens), 11, 22, 44 (LDS-tiled with
-// 64 x 64, 128 x 128, 256 x 256 tiles) force one, for tests and tuning.  Any `slices` within
+// `kernel` 0 lets the shape choose; 16 (streaming, up to 16 tokens), 14 (LDS-tiled, tiles of 32
+// tokens x 64 features), 11, 22, 44 (LDS-tiled with 64 x 64, 128 x 128, 256 x 256 tiles) force
+// one, for tests and tuning.  Any `slices` within
 // 1..64 is accepted with a float32 [slices, m, n] output.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
                   int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k, hipStream_t stream);

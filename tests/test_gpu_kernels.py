@@ -209,7 +209,7 @@ def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     assert torch.equal(picked, got.cpu()[..., [m - 1, 0], :])
 
 
-@pytest.mark.parametrize("kernel", [16, 11, 22, 44])
+@pytest.mark.parametrize("kernel", [16, 14, 11, 22, 44])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
