@@ -80,7 +80,8 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
 // The query/key/value product fused with bias, rotation (cos, sin: [m, head_dim / 2] float32,
 // or null), the queries' store to q_out [m, heads * head_dim] and the keys' and values' store
 // into their cache slots (`write` 0: no cache write).  kernel: 0 chooses; 16 the row-splitting
-// kernel (up to 64 tokens); 11, 22, 44 the tiled kernels as in mlr_gemm_bf16.
+// kernel (up to 64 tokens); 8 its variant with 8 weight rows a workgroup (up to 8 tokens); 11,
+// 22, 44 the tiled kernels as in mlr_gemm_bf16.
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
                             const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,

@@ -132,10 +132,12 @@ __device__ __forceinline__ void qkv_store4(const QkvTarget& qkv, int row0, int t
 }
 
 // Rotation and stores of the fused query/key/value product for one token: the lane holds the
-// sums of four consecutive dims d0..d0+3 of `head`; lanes q and q ^ 2 of a token hold the two
-// halves of the same rotation pairs.  Called by all lanes (it shuffles); `live` guards the stores.
-__device__ __forceinline__ void qkv_finish(const GemmEpilogue& ep, const QkvTarget& qkv, int head, int block_in_head,
-                                           bool rotated, int d0, int q, int token, bool live, float (&v)[4]) {
+// sums of four consecutive dims d0..d0+3 of `head`, which are the low halves (`low`) or the high
+// halves of the rotation pairs j0..j0+3; the lane `partner_mask` away holds the other halves.
+// Called by all lanes (it shuffles); `live` guards the stores.
+__device__ __forceinline__ void qkv_finish_pairs(const GemmEpilogue& ep, const QkvTarget& qkv, int head, bool rotated,
+                                                 int d0, int j0, bool low, int partner_mask, int token, bool live,
+                                                 float (&v)[4]) {
   const int D = qkv.head_dim;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -144,13 +146,12 @@ __device__ __forceinline__ void qkv_finish(const GemmEpilogue& ep, const QkvTarg
   }
   if (rotated) {
     const int half = D / 2;
-    const int j0 = block_in_head * 8 + (q & 1) * 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float partner = __shfl_xor(v[i], 32, kWave);
+      const float partner = __shfl_xor(v[i], partner_mask, kWave);
       const float c = qkv.cos[static_cast<int64_t>(token) * half + j0 + i];
       const float sn = qkv.sin[static_cast<int64_t>(token) * half + j0 + i];
-      v[i] = q < 2 ? v[i] * c - partner * sn : v[i] * c + partner * sn;
+      v[i] = low ? v[i] * c - partner * sn : v[i] * c + partner * sn;
     }
   }
   if (!live) return;
@@ -158,6 +159,13 @@ __device__ __forceinline__ void qkv_finish(const GemmEpilogue& ep, const QkvTarg
 #pragma unroll
   for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16(v[i]).bits;
   qkv_store4(qkv, head * D + d0, token, packed);
+}
+
+// The same for a block of 16 weight rows (8 pairs) spread over the lane quads q = 0..3 of a
+// token: quads q and q ^ 2 hold the two halves of the same pairs.
+__device__ __forceinline__ void qkv_finish(const GemmEpilogue& ep, const QkvTarget& qkv, int head, int block_in_head,
+                                           bool rotated, int d0, int q, int token, bool live, float (&v)[4]) {
+  qkv_finish_pairs(ep, qkv, head, rotated, d0, block_in_head * 8 + (q & 1) * 4, q < 2, 32, token, live, v);
 }
 
 }  // namespace mlr

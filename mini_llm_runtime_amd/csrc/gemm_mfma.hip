@@ -129,6 +129,78 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   }
 }
 
+// ---- skinny fused query/key/value product, up to 8 tokens: 8 weight rows a workgroup ----------
+// The 16 x 16 matrix-core block is filled with two halves of K instead of 16 weight rows: lane
+// rows 0..7 multiply the 8 weight rows with the tokens over the first half of K, rows 8..15 the
+// same weight rows over the second half; tokens 0..7 stand in columns 0..7 and again in 8..15.
+// The two diagonal quadrants of the result are the two partial sums, the others are not used.
+// Every lane still streams weights, and there are twice as many workgroups as with 16 rows each,
+// which counts where those leave compute units without work or give a few of them two.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_qkv8_kernel(const bf16* __restrict__ x,
+                                                                      const bf16* __restrict__ w, GemmEpilogue ep,
+                                                                      QkvTarget qkv, int M, int N, int K) {
+  constexpr int U = 8;  // k-steps in flight per wavefront
+  __shared__ float red[WAVES][kWave][4];
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int r = lane % 16;
+  const int q = lane / 16;
+  const int r8 = r % 8;
+  const int n0 = blockIdx.x * 8;
+  const int chunks = K / 8;
+  const int ksteps = (chunks + 3) / 4;
+  const int half_steps = (ksteps + 1) / 2;
+  const int shift = (r / 8) * half_steps;  // the k-step this lane's half of K starts at
+  const int per_head = qkv.head_dim / 8;
+  const int head = blockIdx.x / per_head;
+  const int block_in_head = blockIdx.x - head * per_head;
+  const bool rotated = qkv.cos != nullptr && head < qkv.heads + qkv.kv_heads;
+  // the weight row behind slot 0..7: four low halves of rotation pairs, then their high halves
+  auto row_of = [&](int slot) {
+    if (!rotated) return n0 + slot;
+    return head * qkv.head_dim + block_in_head * 4 + (slot < 4 ? slot : qkv.head_dim / 2 + slot - 4);
+  };
+  const bf16x8_t* wp = reinterpret_cast<const bf16x8_t*>(w + static_cast<int64_t>(min(row_of(r8), N - 1)) * K);
+  const bf16x8_t* xp = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(r8, M - 1)) * K);
+  const bool xok = r8 < M;
+  f32x4_t acc{0.f, 0.f, 0.f, 0.f};
+
+  for (int s0 = wave; s0 < half_steps; s0 += WAVES * U) {
+    bf16x8_t a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * WAVES;
+      const int c = (s + shift) * 4 + q;
+      a[u] = (s < half_steps && s + shift < ksteps && c < chunks) ? __builtin_nontemporal_load(wp + c) : zero_bf16x8();
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * WAVES;
+      const int c = (s + shift) * 4 + q;
+      b[u] = (xok && s < half_steps && s + shift < ksteps && c < chunks) ? xp[c] : zero_bf16x8();
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc = mfma_16x16x32(a[u], b[u], acc);
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+  __syncthreads();
+  if (wave != 0) return;
+  // lane (r < 8, q < 2) owns weight slots 4q..4q+3 of token r: its own quadrant over the first
+  // half of K plus the quadrant of lane (r + 8, q + 2) over the second half
+  const bool owner = r < 8 && q < 2;
+  const int other = owner ? lane + 8 + 32 : lane;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int ww = 0; ww < WAVES; ++ww)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] += red[ww][lane][i] + red[ww][other][i];
+  const int qq = q & 1;
+  qkv_finish_pairs(ep, qkv, head, rotated, row_of(qq * 4) - head * qkv.head_dim, block_in_head * 4, qq == 0, 16,
+                   min(r8, M - 1), owner && r8 < M, v);
+}
+
 // ---- tiled: more than 16 tokens, and wide products of fewer ---------------------------------
 // Four wavefronts in a 2 x 2 arrangement; each owns WM x WN blocks of 32 x 32 (tokens x
 // features), so the workgroup tile is (64 WM) tokens x (64 WN) features.  K in slices of 64
@@ -484,6 +556,12 @@ static int tiles_256(int m, int n) { return ((n + 255) / 256) * ((m + 255) / 256
 // eighths of the compute units, the 16-feature streaming kernel below that.
 static bool few_tokens_tiled(int n, int slices) { return ((n + 63) / 64) * slices >= 224; }
 
+// Up to 8 tokens of the fused query/key/value product: workgroups of 8 weight rows instead of
+// 16 when that shortens the longest queue of workgroups on a compute unit (256 of them).
+static bool half_rows_fill_better(int blocks16) {
+  return (2 * blocks16 + 255) / 256 < 2 * ((blocks16 + 255) / 256);
+}
+
 // Kernel and number of K slices for more than 64 tokens, when the consumer takes up to
 // `max_slices` partial sums.  A larger tile needs less L2 traffic per flop and wins once there
 // are enough of them to keep the compute units busy; the largest one wants K long enough to pay
@@ -621,10 +699,18 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
     kernel = m <= 64 ? 16 : choose_kernel(m, static_cast<int>(n), k, 1);
     if (kernel == 16 && m > 16 && (n / 16) * m * k * 2 > (32ll << 20)) kernel = 11;  // too many passes over x
   }
+  if (kernel == 8) {
+    MLR_REQUIRE(m <= 8, "the 8-row kernel takes 1..8 tokens");
+    gemm_skinny_qkv8_kernel<4><<<dim3(static_cast<unsigned>(n / 8)), 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
   if (kernel == 16) {
     MLR_REQUIRE(m <= 64, "the row-splitting kernel takes 1..64 tokens");
     const dim3 grid(static_cast<unsigned>(n / 16));
-    if (m <= 16)
+    if (m <= 8 && half_rows_fill_better(static_cast<int>(n / 16)))
+      gemm_skinny_qkv8_kernel<4><<<dim3(static_cast<unsigned>(n / 8)), 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+    else if (m <= 16)
       gemm_skinny_split_kernel<4, true, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
     else if (m <= 32)
       gemm_skinny_split_kernel<4, true, 2><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);

@@ -296,6 +296,9 @@ _QKV_CASES = [
     (14, 2, 64, 896, 300, True, True, 44), (3, 1, 48, 104, 70, True, True, 11), (3, 1, 48, 104, 70, True, True, 22),
     (5, 3, 16, 40, 200, True, True, 44), (7, 1, 80, 72, 99, True, True, 22), (2, 2, 96, 136, 65, True, False, 11),
     (4, 4, 80, 72, 77, False, True, 22), (5, 1, 256, 136, 40, True, True, 11), (3, 3, 128, 264, 150, True, True, 44),
+    (14, 2, 64, 896, 8, True, True, 8), (3, 1, 16, 40, 1, True, True, 8), (4, 4, 80, 72, 5, False, True, 8),
+    (5, 1, 128, 136, 7, True, False, 8), (6, 3, 48, 1208, 3, True, True, 8), (14, 2, 64, 896, 8, True, True, 16),
+    (6, 3, 48, 104, 5, True, True, 16), (28, 4, 128, 3584, 8, True, True, 0), (28, 4, 128, 3584, 8, True, True, 16),
 ]
 
 
@@ -303,8 +306,8 @@ _QKV_CASES = [
     "heads,kv_heads,head_dim,hidden,tokens,rotate,write,kernel", [c if len(c) == 8 else c + (0,) for c in _QKV_CASES]
 )
 def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write, kernel):
-    """Product, bias, rotation and cache write run as one kernel (a row-splitting one for few
-    tokens, the tiled ones, each forced here, for many); it has to leave the queries and the
+    """Product, bias, rotation and cache write run as one kernel (row-splitting ones for few
+    tokens, with 16 or 8 weight rows a workgroup, the tiled ones for many; each forced here); it has to leave the queries and the
     pages as the product followed by the rotation kernel does, and must not touch any slot but
     the tokens' own (a token without a slot writes nothing)."""
     ops = ops_for(torch.bfloat16)
@@ -334,8 +337,9 @@ def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads,
         out[fused] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
     for name, a, c in zip(("queries", "key pages", "value pages"), out[False], out[True]):
         assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
-        if tokens <= 16 and kernel == 0:
-            # both ways sum the product in the same order; the rotation's two products may be
+        if tokens <= 16 and (kernel == 16 or (kernel == 0 and tokens > 8)):
+            # both ways sum the product in the same order (up to 8 tokens the shape may choose the
+            # kernel that sums two halves of k); the rotation's two products may be
             # contracted differently: a last-place difference at most
             tol = dict(atol=0, rtol=2 ** -7)
         else:
