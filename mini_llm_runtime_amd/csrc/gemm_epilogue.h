@@ -76,14 +76,21 @@ __device__ __forceinline__ void finish4(const GemmEpilogue& ep, int slice, int s
     store4(ep, m, n, N, v[0], v[1], v[2], v[3]);
     return;
   }
-  float* dst = static_cast<float*>(ep.y) + (static_cast<int64_t>(slice) * M + m) * N + n;
+  const int64_t at = (static_cast<int64_t>(slice) * M + m) * N + n;
+  float* dst = static_cast<float*>(ep.y) + at;
+  float out[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    if (n + i >= N) continue;
-    float out = v[i];
-    if (slice == 0 && ep.bias != nullptr) out += load_as_f32(ep.bias, n + i, ep.bias_is_f32);
-    dst[i] = out;
+    out[i] = v[i];
+    if (slice == 0 && ep.bias != nullptr && n + i < N) out[i] += load_as_f32(ep.bias, n + i, ep.bias_is_f32);
   }
+  if (n + 3 < N && (at & 3) == 0) {
+    *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{out[0], out[1], out[2], out[3]};
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (n + i < N) dst[i] = out[i];
 }
 
 // What the fused query/key/value product needs beside the product itself: the rotation

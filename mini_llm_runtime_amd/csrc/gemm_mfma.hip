@@ -573,6 +573,9 @@ struct GemmPlan {
 };
 static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
   const int big = tiles_256(m, n), mid = tiles_128(m, n);
+  // 129..170 of the largest tiles leave a third of the compute units idle in one pass; three
+  // slices of a very long K fill two passes (2048 x 5120 x 27648: 536 us against 693 us whole)
+  if (max_slices >= 3 && big > 128 && big * 3 <= 512 && k >= 3 * 4096) return {44, 3};
   if (big >= 144 && (big >= 512 || k >= 2048)) return {44, 1};
   if (max_slices >= 2 && big * 2 >= 192 && k >= 8192) return {44, 2};
   if (mid >= 256) return {22, 1};
