@@ -399,11 +399,28 @@ constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounde
 constexpr int kKeyGroups = D <= 64 ? 2 : 1;
 constexpr int kSubTiles = kTileK / 16;
 constexpr int kPairs = kSubTiles / 2;      // the value product takes 32 key positions per MFMA
-constexpr int kKLd = D + 8;                // padded key row in LDS (elements)
-constexpr int kVLd = kTileK + 8;
+// LDS rows are read 16 bytes a lane, 16 rows x 4 consecutive pieces per wavefront instruction.
+// Measured on gfx950: that pattern is free of bank conflicts when the row stride is 32 bytes
+// modulo 64, two-way conflicted at 16 or 48 modulo 64 and worse at multiples of 64; an 8-byte
+// read costs as much as a 16-byte one.  So rows are padded to 32 modulo 64 bytes and every
+// operand is one 16-byte read.
+constexpr int kKLd = (D % 32 == 0) ? D + 16 : D;  // key row in LDS (elements)
+constexpr int kVLd = kTileK + 16;                  // value row (one head dim, the tile's key positions)
 constexpr int kPieces = (kTileK * (D / 8) + 255) / 256;  // 16-byte pieces per thread, of the key and of the value tile
 constexpr int kNoPiece = 0x3fffffff;                      // position of a piece that a thread does not have
-constexpr int kPrefillLds = 2 * kKeyGroups * (kTileK * kKLd + D * kVLd) * 2 + 16;  // bytes: two buffers per group, a flag
+// The workgroup's flag lives in the padding of a key row where rows are padded (two
+// workgroups of the small head sizes then fill a compute unit's 160 KB exactly), else behind the buffers.
+constexpr int kFlagInPadding = kKLd > D;
+constexpr int kPrefillLds = 2 * kKeyGroups * (kTileK * kKLd + D * kVLd) * 2 + (kFlagInPadding ? 0 : 16);  // bytes: two buffers per group
+
+// Where key `k` of a tile lies in LDS.  The 16 rows that a score product reads for sub-tile
+// 2 * pair + half hold the keys pair * 32 + 8 * (m / 4) + 4 * half + m % 4 (m = 0..15), so that a
+// lane's accumulator elements of the pair's two sub-tiles (4 keys each) are 8 consecutive keys:
+// exactly one 16-byte piece of a value row for the second product.
+__host__ __device__ constexpr int key_row_in_lds(int k) {
+  const int pair = k / 32, w = k % 32;
+  return (2 * pair + (w % 8) / 4) * 16 + (w / 8) * 4 + w % 4;
+}
 
 // One key/value tile on its way from the pages to LDS.
 struct TileInFlight {
@@ -426,7 +443,10 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   bf16* const lds = reinterpret_cast<bf16*>(prefill_lds);
   constexpr int kBuffer = kTileK * kKLd + D * kVLd;  // elements
-  int& sm_bad = *reinterpret_cast<int*>(prefill_lds + 2 * kKeyGroups * kBuffer * 2);
+  // the flag: in the padding of the last buffer's last key row (the groups' handover at the end
+  // overlays the front of the buffers), or behind the buffers
+  constexpr int kFlagAt = kFlagInPadding ? ((2 * kKeyGroups - 1) * kBuffer + (kTileK - 1) * kKLd + D) * 2 : 2 * kKeyGroups * kBuffer * 2;
+  int& sm_bad = *reinterpret_cast<int*>(prefill_lds + kFlagAt);
 
   const int block_size = 1 << bs_shift;
   // Workgroup -> (tile, head).  The tile list comes heaviest first (a tile late in a long
@@ -502,7 +522,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     k_row[i] = c < kTileK * (D / 8) ? row : kNoPiece;
     k_page[i] = row >> bs_shift;
     k_in_page[i] = (kvh * block_size + (row & bs_mask)) * D + ch * 8;
-    k_lds[i] = row * kKLd + ch * 8;
+    k_lds[i] = key_row_in_lds(row % kTileK) * kKLd + ch * 8;
   }
   int v_pos[kPieces], v_page[kPieces], v_in_page[kPieces], v_lds[kPieces];
   const int per_page = D * (block_size / 8);  // 16-byte pieces of a value page (one kv head)
@@ -612,12 +632,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       // The value operands of the tile's first 32 keys leave LDS now: the softmax below hides
       // their way, which would otherwise be waited for once per product.
       typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-      auto value_operand = [&](int dt, int pr) {
-        const bf16* vrow = vs + (dt * 16 + col) * kVLd + pr * 32 + quarter * 4;
-        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vrow);
-        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vrow + 16);
-        return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+      auto value_operand = [&](int dt, int pr) {  // dim dt * 16 + col, keys pr * 32 + quarter * 8 .. + 7
+        return *reinterpret_cast<const u32x4_t*>(vs + (dt * 16 + col) * kVLd + pr * 32 + quarter * 8);
       };
       constexpr bool kValuesAhead = kDimTiles <= 8;  // registers allow it
       u32x4_t ahead[kValuesAhead ? kDimTiles : 1];
@@ -633,7 +649,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
         for (int sub = 0; sub < kSubTiles; ++sub)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int key = kt0 + sub * 16 + quarter * 4 + i;
+            const int key = kt0 + (sub / 2) * 32 + quarter * 8 + (sub % 2) * 4 + i;  // see key_row_in_lds
             if (!(q_ok && key <= pq && key >= pq_first)) s[sub][i] = -INFINITY;
           }
       }
@@ -669,7 +685,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
           for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
       }
       // O^T += V^T P^T, 32 key positions per MFMA: k-slots 0..3 of a lane are its 4 keys of the
-      // pair's first sub-tile, slots 4..7 those of the second; the value operand follows the same map
+      // pair's first sub-tile, slots 4..7 those of the second: 8 consecutive keys, by the order of the
+      // key rows in LDS
 #pragma unroll
       for (int pr = 0; pr < kPairs; ++pr) {
         const u32x4_t pb = {pw[2 * pr][0], pw[2 * pr][1], pw[2 * pr + 1][0], pw[2 * pr + 1][1]};
@@ -690,7 +707,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   // merge the key groups: the second hands its state over through LDS (the tiles are done with)
   float* const handover = reinterpret_cast<float*>(prefill_lds);  // [group - 1][component][thread of the group]
   constexpr int kHandover = (2 + kDimTiles * 4) * 256;
-  static_assert((kKeyGroups - 1) * kHandover * 4 <= 2 * kKeyGroups * kBuffer * 2, "the handover fits the tile buffers");
+  static_assert((kKeyGroups - 1) * kHandover * 4 <= kFlagAt, "the handover fits the tile buffers in front of the flag");
   if (kKeyGroups > 1 && group > 0) {
     float* mine = handover + (group - 1) * kHandover;
     mine[tid] = m_run;
