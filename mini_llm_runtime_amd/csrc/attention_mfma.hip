@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 }
 
 // ---- prefill ----------------------------------------------------------------------------------
-constexpr int kTileQ = 64;                 // queries per workgroup (16 per wavefront)
+constexpr int kTileQ = 64;                 // queries per workgroup (16 per wavefront), times QB (see the kernel)
 constexpr int kTileK = D > 192 ? 32 : 64;  // key positions per LDS tile (bounded by LDS)
 // Wavefront groups of a workgroup that take the key tiles in turn and merge at the end: a
 // query tile's keys are a chain of dependent steps, and a second group halves it.  Measured:
@@ -428,6 +428,11 @@ struct TileInFlight {
   bf16x8_t v[kPieces];
 };
 
+// QB: blocks of 16 queries per wavefront (1 or 2).  With 2 a workgroup takes 128 queries and every
+// key and value operand read from LDS serves two matrix-core products, which halves the LDS
+// traffic per flop (LDS bandwidth, not the matrix cores, bounds the kernel with 1); it needs
+// twice the accumulators and is offered up to head size 128.
+template <int QB>
 __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
@@ -462,6 +467,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   const int entry = tiles[2 * tile];
   const int q0 = tiles[2 * tile + 1];
   const int kvh = head / (heads / kv_heads);
+  constexpr int kWaveQ = 16 * QB;  // queries of a wavefront
+  constexpr int kWgQ = kTileQ * QB;  // queries of the workgroup
   // uniform in a wavefront, and said so: everything derived from them (tile positions, the
   // conditions on them) then lives in scalar registers and scalar branches
   const int group = __builtin_amdgcn_readfirstlane(threadIdx.x / 256);  // key group
@@ -478,35 +485,45 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   const int* table = block_table + static_cast<int64_t>(entry) * table_width;
   if (threadIdx.x == 0) sm_bad = 0;
 
-  // this lane's query (a column of S^T)
-  const int qi = q0 + wave * 16 + col;
-  const bool q_ok = qi < q_len;
-  const int pq = pos0 + qi;  // its absolute position
-  const int pq_first = window > 0 ? max(0, pq - window + 1) : 0;
-  const RowOperand qo = load_row(
-      q + static_cast<int64_t>(t_first + (q_ok ? qi : 0)) * q_stride + static_cast<int64_t>(head) * D, q_ok, quarter);
+  // this lane's queries (columns of S^T), one per block
+  int qi[QB], pq[QB], pq_first[QB];
+  bool q_ok[QB];
+  RowOperand qo[QB];
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    qi[b] = q0 + wave * kWaveQ + b * 16 + col;
+    q_ok[b] = qi[b] < q_len;
+    pq[b] = pos0 + qi[b];  // its absolute position
+    pq_first[b] = window > 0 ? max(0, pq[b] - window + 1) : 0;
+    qo[b] = load_row(q + static_cast<int64_t>(t_first + (q_ok[b] ? qi[b] : 0)) * q_stride + static_cast<int64_t>(head) * D,
+                     q_ok[b], quarter);
+  }
 
   // key range of the workgroup: from the first query's window start to the last query's position
-  const int last_q = min(q0 + kTileQ, q_len) - 1;
+  const int last_q = min(q0 + kWgQ, q_len) - 1;
   const int k_end = pos0 + last_q + 1;
   const int k_begin_raw = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
   const int k_begin = (k_begin_raw / kTileK) * kTileK;
   // the wavefront's own range (uniform within the wavefront)
-  const int w_last = pos0 + min(q0 + wave * 16 + 15, q_len - 1);
-  const int w_first = window > 0 ? max(0, pos0 + q0 + wave * 16 - window + 1) : 0;
-  const bool wave_has_queries = q0 + wave * 16 < q_len;
+  const int w_last = pos0 + min(q0 + wave * kWaveQ + kWaveQ - 1, q_len - 1);
+  const int w_first = window > 0 ? max(0, pos0 + q0 + wave * kWaveQ - window + 1) : 0;
+  const bool wave_has_queries = q0 + wave * kWaveQ < q_len;
   // a tile is fully visible to the wavefront when it ends at or before its first query's position
   // and starts at or after its last query's window start (queries beyond q_len are never stored)
-  const int w_min_pos = pos0 + q0 + wave * 16;
-  const int w_max_first = window > 0 ? max(0, pos0 + q0 + wave * 16 + 15 - window + 1) : 0;
+  const int w_min_pos = pos0 + q0 + wave * kWaveQ;
+  const int w_max_first = window > 0 ? max(0, pos0 + q0 + wave * kWaveQ + kWaveQ - 1 - window + 1) : 0;
   // softmax in base 2: exp(x) = exp2(x * log2(e))
   const float scale2 = scale * 1.44269504088896340736f;
 
-  float m_run = -INFINITY;
-  float l_run = 0.f;  // this lane's share of the sum
-  f32x4_t acc[kDimTiles];
+  float m_run[QB], l_run[QB];  // l: this lane's share of the sum
+  f32x4_t acc[QB][kDimTiles];
 #pragma unroll
-  for (int dt = 0; dt < kDimTiles; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < QB; ++b) {
+    m_run[b] = -INFINITY;
+    l_run[b] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt) acc[b][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
   bool bad = false;
 
   // Which pieces of a tile each thread moves does not change from tile to tile: work out once
@@ -595,7 +612,9 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   // The query has to be there before the loop: a load still pending at the loop's head makes
   // the compiler wait, in every turn, for everything in flight, the next tile's loads included.
 #pragma unroll
-  for (int st = 0; st < kSteps; ++st) asm volatile("" ::"v"(qo.step[st]));
+  for (int b = 0; b < QB; ++b)
+#pragma unroll
+    for (int st = 0; st < kSteps; ++st) asm volatile("" ::"v"(qo[b].step[st]));
 
   TileInFlight flight;
   constexpr int kStep = kKeyGroups * kTileK;  // keys per turn of the loop, all groups together
@@ -624,18 +643,21 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
       // cycles, an exponential sixteen), so every per-score operation counts: the scale is
       // folded into the exponent's multiply-add, hidden scores are -inf and become 0 in the
       // exponential by themselves, and only tiles that cross a query's limits build masks.
-      f32x4_t s[kSubTiles];
+      f32x4_t s[QB][kSubTiles];
       const bool full = kt0 + kTileK - 1 <= w_min_pos && kt0 >= w_max_first;  // uniform in the wavefront
 #pragma unroll
-      for (int sub = 0; sub < kSubTiles; ++sub)
-        s[sub] = score_tile(load_row(ks + (sub * 16 + col) * kKLd, true, quarter), qo);
+      for (int sub = 0; sub < kSubTiles; ++sub) {
+        const RowOperand keys = load_row(ks + (sub * 16 + col) * kKLd, true, quarter);
+#pragma unroll
+        for (int b = 0; b < QB; ++b) s[b][sub] = score_tile(keys, qo[b]);
+      }
       // The value operands of the tile's first 32 keys leave LDS now: the softmax below hides
       // their way, which would otherwise be waited for once per product.
       typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
       auto value_operand = [&](int dt, int pr) {  // dim dt * 16 + col, keys pr * 32 + quarter * 8 .. + 7
         return *reinterpret_cast<const u32x4_t*>(vs + (dt * 16 + col) * kVLd + pr * 32 + quarter * 8);
       };
-      constexpr bool kValuesAhead = kDimTiles <= 8;  // registers allow it
+      constexpr bool kValuesAhead = kDimTiles * QB <= 8;  // registers allow it
       u32x4_t ahead[kValuesAhead ? kDimTiles : 1];
       if constexpr (kValuesAhead) {
 #pragma unroll
@@ -646,55 +668,65 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
         // a branch of its own: folded into selects, these comparisons would run for every tile
         asm volatile("" ::: "memory");
 #pragma unroll
+        for (int b = 0; b < QB; ++b)
+#pragma unroll
+          for (int sub = 0; sub < kSubTiles; ++sub)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = kt0 + (sub / 2) * 32 + quarter * 8 + (sub % 2) * 4 + i;  // see key_row_in_lds
+              if (!(q_ok[b] && key <= pq[b] && key >= pq_first[b])) s[b][sub][i] = -INFINITY;
+            }
+      }
+      uint32_t pw[QB][kSubTiles][2];
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        float tmax = -INFINITY;
+#pragma unroll
         for (int sub = 0; sub < kSubTiles; ++sub)
 #pragma unroll
+          for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[b][sub][i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float m_new = fmaxf(m_run[b], tmax * scale2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
+        const float alpha = fast_exp2(m_run[b] - m_use);          // 2^-inf = 0 for the first tile
+        float sum = 0.f;
+#pragma unroll
+        for (int sub = 0; sub < kSubTiles; ++sub) {
+          float p[4];
+#pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int key = kt0 + (sub / 2) * 32 + quarter * 8 + (sub % 2) * 4 + i;  // see key_row_in_lds
-            if (!(q_ok && key <= pq && key >= pq_first)) s[sub][i] = -INFINITY;
+            p[i] = fast_exp2(fmaf(s[b][sub][i], scale2, -m_use));
+            sum += p[i];
           }
-      }
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int sub = 0; sub < kSubTiles; ++sub)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[sub][i]);
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-      const float m_new = fmaxf(m_run, tmax * scale2);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
-      const float alpha = fast_exp2(m_run - m_use);            // 2^-inf = 0 for the first tile
-      float sum = 0.f;
-      uint32_t pw[kSubTiles][2];
-#pragma unroll
-      for (int sub = 0; sub < kSubTiles; ++sub) {
-        float p[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          p[i] = fast_exp2(fmaf(s[sub][i], scale2, -m_use));
-          sum += p[i];
+          pw[b][sub][0] = pack_bf16x2(p[0], p[1]);
+          pw[b][sub][1] = pack_bf16x2(p[2], p[3]);
         }
-        pw[sub][0] = pack_bf16x2(p[0], p[1]);
-        pw[sub][1] = pack_bf16x2(p[2], p[3]);
-      }
-      l_run = l_run * alpha + sum;
-      m_run = m_new;
-      if (__any(alpha != 1.0f)) {
+        l_run[b] = l_run[b] * alpha + sum;
+        m_run[b] = m_new;
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
-        for (int dt = 0; dt < kDimTiles; ++dt)
+          for (int dt = 0; dt < kDimTiles; ++dt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+            for (int i = 0; i < 4; ++i) acc[b][dt][i] *= alpha;
+        }
       }
       // O^T += V^T P^T, 32 key positions per MFMA: k-slots 0..3 of a lane are its 4 keys of the
       // pair's first sub-tile, slots 4..7 those of the second: 8 consecutive keys, by the order of the
       // key rows in LDS
 #pragma unroll
       for (int pr = 0; pr < kPairs; ++pr) {
-        const u32x4_t pb = {pw[2 * pr][0], pw[2 * pr][1], pw[2 * pr + 1][0], pw[2 * pr + 1][1]};
-        const bf16x8_t pop = __builtin_bit_cast(bf16x8_t, pb);
+        bf16x8_t pop[QB];
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+          const u32x4_t pb = {pw[b][2 * pr][0], pw[b][2 * pr][1], pw[b][2 * pr + 1][0], pw[b][2 * pr + 1][1]};
+          pop[b] = __builtin_bit_cast(bf16x8_t, pb);
+        }
 #pragma unroll
         for (int dt = 0; dt < kDimTiles; ++dt) {
           const u32x4_t va = (kValuesAhead && pr == 0) ? ahead[dt] : value_operand(dt, pr);
-          acc[dt] = mfma_16x16x32(__builtin_bit_cast(bf16x8_t, va), pop, acc[dt]);
+#pragma unroll
+          for (int b = 0; b < QB; ++b) acc[b][dt] = mfma_16x16x32(__builtin_bit_cast(bf16x8_t, va), pop[b], acc[b][dt]);
         }
       }
     }
@@ -705,48 +737,57 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   }
 
   // merge the key groups: the second hands its state over through LDS (the tiles are done with)
-  float* const handover = reinterpret_cast<float*>(prefill_lds);  // [group - 1][component][thread of the group]
-  constexpr int kHandover = (2 + kDimTiles * 4) * 256;
+  float* const handover = reinterpret_cast<float*>(prefill_lds);  // [group - 1][block][component][thread of the group]
+  constexpr int kPerBlock = (2 + kDimTiles * 4) * 256;
+  constexpr int kHandover = QB * kPerBlock;
   static_assert((kKeyGroups - 1) * kHandover * 4 <= kFlagAt, "the handover fits the tile buffers in front of the flag");
   if (kKeyGroups > 1 && group > 0) {
-    float* mine = handover + (group - 1) * kHandover;
-    mine[tid] = m_run;
-    mine[256 + tid] = l_run;
 #pragma unroll
-    for (int dt = 0; dt < kDimTiles; ++dt)
+    for (int b = 0; b < QB; ++b) {
+      float* mine = handover + (group - 1) * kHandover + b * kPerBlock;
+      mine[tid] = m_run[b];
+      mine[256 + tid] = l_run[b];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) mine[(2 + dt * 4 + i) * 256 + tid] = acc[dt][i];
+      for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mine[(2 + dt * 4 + i) * 256 + tid] = acc[b][dt][i];
+    }
   }
   if (bad) atomicOr(&sm_bad, 1);
   __syncthreads();
   if (group != 0) return;
-#pragma unroll
-  for (int g = 1; g < kKeyGroups; ++g) {  // in the groups' order, whichever finished first
-    const float* other = handover + (g - 1) * kHandover;
-    const float m_other = other[tid];
-    const float m_new = fmaxf(m_run, m_other);
-    const float w_mine = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);
-    const float w_other = (m_other == -INFINITY) ? 0.f : fast_exp2(m_other - m_new);
-    l_run = l_run * w_mine + other[256 + tid] * w_other;
-#pragma unroll
-    for (int dt = 0; dt < kDimTiles; ++dt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[dt][i] = acc[dt][i] * w_mine + other[(2 + dt * 4 + i) * 256 + tid] * w_other;
-    m_run = m_new;
-  }
   const bool poisoned = sm_bad != 0;
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
-  if (q_ok) {
-    const float inv = 1.0f / l_run;
-    bf16* orow = out + (static_cast<int64_t>(t_first + qi) * heads + head) * D;
 #pragma unroll
-    for (int dt = 0; dt < kDimTiles; ++dt) {
-      u16x4_t packed;
+  for (int b = 0; b < QB; ++b) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        packed[i] = f32_to_bf16(poisoned ? __builtin_nanf("") : acc[dt][i] * inv).bits;
-      *reinterpret_cast<u16x4_t*>(orow + dt * 16 + quarter * 4) = packed;
+    for (int g = 1; g < kKeyGroups; ++g) {  // in the groups' order, whichever finished first
+      const float* other = handover + (g - 1) * kHandover + b * kPerBlock;
+      const float m_other = other[tid];
+      const float m_new = fmaxf(m_run[b], m_other);
+      const float w_mine = (m_run[b] == -INFINITY) ? 0.f : fast_exp2(m_run[b] - m_new);
+      const float w_other = (m_other == -INFINITY) ? 0.f : fast_exp2(m_other - m_new);
+      l_run[b] = l_run[b] * w_mine + other[256 + tid] * w_other;
+#pragma unroll
+      for (int dt = 0; dt < kDimTiles; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[b][dt][i] = acc[b][dt][i] * w_mine + other[(2 + dt * 4 + i) * 256 + tid] * w_other;
+      m_run[b] = m_new;
+    }
+    float l = l_run[b];
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (q_ok[b]) {
+      const float inv = 1.0f / l;
+      bf16* orow = out + (static_cast<int64_t>(t_first + qi[b]) * heads + head) * D;
+#pragma unroll
+      for (int dt = 0; dt < kDimTiles; ++dt) {
+        u16x4_t packed;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          packed[i] = f32_to_bf16(poisoned ? __builtin_nanf("") : acc[b][dt][i] * inv).bits;
+        *reinterpret_cast<u16x4_t*>(orow + dt * 16 + quarter * 4) = packed;
+      }
     }
   }
 }
@@ -840,10 +881,15 @@ int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int*
   return 0;
 }
 
+// Queries per tile of the wide variant of mlr_attention_prefill (`wide` = 1); 0 if this head
+// size has none.
+int mlr_attention_wide_tile() { return D <= 128 ? 2 * kTileQ : 0; }
+
 // Attention of the query tiles listed in `tiles` ([num_tiles][2]: entry, first
-// query of the tile within the entry's new tokens; 64 queries per tile).
+// query of the tile within the entry's new tokens; 64 queries per tile, or
+// mlr_attention_wide_tile() with `wide`).
 int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
-                          const int* block_table, int table_width, const int* tiles, int num_tiles,
+                          const int* block_table, int table_width, const int* tiles, int num_tiles, int wide,
                           const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
                           int block_size, int num_pages, float scale, int window, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
@@ -851,6 +897,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   MLR_REQUIRE(kv_heads <= 65535, "too many key/value heads");  // a page's elements fit 32 bits
   MLR_REQUIRE(block_size >= 8 && (block_size & (block_size - 1)) == 0 && block_size <= kTileK,
               "block_size must be a power of two within 8 and the key tile");
+  MLR_REQUIRE(!wide || mlr_attention_wide_tile() > 0, "this head size has no wide query tiles");
   int bs_shift = 0;
   while ((1 << bs_shift) < block_size) ++bs_shift;
   MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
@@ -862,18 +909,34 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   MLR_REQUIRE(static_cast<int64_t>(num_tiles) * heads < (1ll << 31), "too many tiles for one launch");
   static bool configured = false;
   if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<1>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
+    if constexpr (D <= 128) {
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<2>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
+    }
     if (e != hipSuccess) {
       set_error(std::string("mlr_attention_prefill: cannot raise the LDS limit: ") + hipGetErrorString(e));
       return -1;
     }
     configured = true;
   }
-  attn_prefill_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256 * kKeyGroups, kPrefillLds, stream>>>(
-      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
-      static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,
-      static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);
+  const dim3 grid(static_cast<unsigned>(num_tiles) * heads);
+#define MLR_PREFILL(qb)                                                                                       \
+  attn_prefill_kernel<qb><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                                   \
+      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                             \
+      static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,             \
+      static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window)
+  if constexpr (D <= 128) {
+    if (wide)
+      MLR_PREFILL(2);
+    else
+      MLR_PREFILL(1);
+  } else {
+    MLR_PREFILL(1);
+  }
+#undef MLR_PREFILL
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -60,6 +60,7 @@ _SIGNATURES = {
     "mlr_sample_scratch": ([_I, _I], _I64),
     "mlr_attention_head_dim": ([], _I),
     "mlr_attention_key_tile": ([], _I),
+    "mlr_attention_wide_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
     "mlr_attention_decode": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _VP],
@@ -67,12 +68,12 @@ _SIGNATURES = {
     ),
     "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_attention_prefill": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
         _I,
     ),
 }
 
-from .plans import PAGED_ATTENTION, QUERY_TILE, attention_plan, query_tiles  # noqa: F401
+from .plans import PAGED_ATTENTION, QUERY_TILE, WIDE_QUERY_TILE, attention_plan, query_tiles  # noqa: F401
 
 
 class KernelError(RuntimeError):
@@ -702,10 +703,20 @@ class HipOps:
                     partial, ctx.cu_q, ctx.context_lens, tokens, num_heads, head_dim, int(window or 0), part, splits, lib
                 )
         if num_tiles:
-            self._check(plan.query_tiles, "query tiles", torch.int32, (num_tiles, 2))
+            # long prompts: tiles of 128 queries, whose key and value tiles in LDS serve twice the
+            # products, once there are enough of them to keep every compute unit busy all the same
+            tiles, wide = plan.query_tiles, 0
+            num_wide = int(getattr(plan, "num_wide_query_tiles", 0))
+            if (
+                num_wide * num_heads >= self.tuning.wide_attention_groups
+                and getattr(plan, "wide_query_tiles", None) is not None
+                and lib.mlr_attention_wide_tile() == WIDE_QUERY_TILE
+            ):
+                tiles, num_tiles, wide = plan.wide_query_tiles, num_wide, 1
+            self._check(tiles, "query tiles", torch.int32, (num_tiles, 2))
             self._call(
                 "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
-                self._ptr(block_table), width, self._ptr(plan.query_tiles), num_tiles, self._ptr(ctx.cu_q),
+                self._ptr(block_table), width, self._ptr(tiles), num_tiles, wide, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
                 float(scale), int(window or 0), self._stream(), lib=lib,
             )

@@ -10,14 +10,16 @@ import numpy as np
 from ..parts.context import MixerPlan, PlanInput
 
 QUERY_TILE = 64  # queries of one request that the prompt kernel takes together
+WIDE_QUERY_TILE = 128  # and in its variant for long prompts (two blocks of queries per wavefront)
 PAGED_ATTENTION = "paged_attention"  # the plan's key: every mixer on these kernels shares one plan per step
 
 
-def query_tiles(q_lens, q_starts=None) -> np.ndarray:
+def query_tiles(q_lens, q_starts=None, tile: int = QUERY_TILE) -> np.ndarray:
     """[num_tiles, 2] int32 (entry, first query) covering every entry with more than one new
-    token, the tiles with the most keys before them first: a kernel that hands them to the
-    compute units in that order can start the heavy ones early and pair them with light ones."""
-    tiles = [(r, q0) for r, n in enumerate(q_lens) if n > 1 for q0 in range(0, int(n), QUERY_TILE)]
+    token in tiles of `tile` queries, the tiles with the most keys before them first: a kernel
+    that hands them to the compute units in that order can start the heavy ones early and pair
+    them with light ones."""
+    tiles = [(r, q0) for r, n in enumerate(q_lens) if n > 1 for q0 in range(0, int(n), tile)]
     if q_starts is None:
         q_starts = [0] * len(q_lens)
     tiles.sort(key=lambda t: -(int(q_starts[t[0]]) + t[1]))
@@ -25,18 +27,21 @@ def query_tiles(q_lens, q_starts=None) -> np.ndarray:
 
 
 def attention_plan(shape: PlanInput) -> MixerPlan:
-    """Tiles of 64 queries over the entries with several new tokens (for the prompt kernel), and
+    """Tiles of 64 and of 128 queries over the entries with several new tokens (for the prompt
+    kernel and its wide variant; the launch picks one by how many there are), and
     how many entries have a single token and how long their contexts may be (for the split-KV
     decode kernel).  `shape.max_context` bounds the contexts; a recording is made with the
     capacity of its block tables there, so that it holds for every later step of its sizes."""
     single = shape.q_lens == 1
     decodes = int(single.sum())
     tiles = query_tiles(shape.q_lens, shape.q_starts)
+    wide = query_tiles(shape.q_lens, shape.q_starts, WIDE_QUERY_TILE)
     return MixerPlan(
         key=PAGED_ATTENTION,
-        arrays={"query_tiles": tiles},
+        arrays={"query_tiles": tiles, "wide_query_tiles": wide},
         sizes={
             "num_query_tiles": len(tiles),
+            "num_wide_query_tiles": len(wide),
             "num_decode_entries": decodes,
             "max_decode_context": int(shape.max_context) if decodes else 0,
         },

@@ -17,9 +17,12 @@ class KernelTuning:
     # only some 15 GB/s whatever the source: beyond this many bytes of prologue input per workgroup
     # the kernel of its own is the faster way.
     fuse_bytes: int = 1 << 30
+    # Prompt attention takes tiles of 128 queries instead of 64 once tiles x heads reach this many
+    # workgroups (fewer leave compute units idle behind the heaviest tiles).
+    wide_attention_groups: int = 512
 
     def __post_init__(self) -> None:
-        for name in ("decode_partition", "decode_max_groups", "max_k_slices"):
+        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups"):
             value = getattr(self, name)
             if isinstance(value, bool) or not isinstance(value, int) or value <= 0:
                 raise ValueError(f"KernelTuning.{name} must be a positive integer")

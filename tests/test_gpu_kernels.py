@@ -399,6 +399,7 @@ def _plan(entries, token_entry, positions):
     for n in q_lens:
         cu.append(cu[-1] + n)
     tiles = query_tiles(q_lens)
+    wide = query_tiles(q_lens, tile=128)
     singles = [c for c, ql in entries if ql == 1]
     return SimpleNamespace(
         num_entries=len(entries),
@@ -410,6 +411,8 @@ def _plan(entries, token_entry, positions):
         max_q_len=max(q_lens),
         query_tiles=torch.from_numpy(tiles).cuda() if len(tiles) else None,
         num_query_tiles=len(tiles),
+        wide_query_tiles=torch.from_numpy(wide).cuda() if len(wide) else None,
+        num_wide_query_tiles=len(wide),
         num_decode_entries=len(singles),
         max_decode_context=max(singles, default=0),
     )
@@ -456,6 +459,26 @@ def test_paged_attention_window(ops_for, dtype, window):
     ops = ops_for(dtype)
     heads, kv_heads, head_dim, bs = 4, 2, 32, 8
     entries = [(1, 1), (16, 16), (60, 3), (75, 1)]
+    _check_window(ops, dtype, window, heads, kv_heads, head_dim, bs, entries)
+
+
+@pytest.mark.parametrize("window", [1, 50, 128, 200])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,bs", [(4, 2, 32, 8), (6, 2, 128, 16), (7, 1, 64, 16)])
+def test_wide_prefill_attention_window(window, heads, kv_heads, head_dim, bs):
+    """Tiles of 128 queries under a window: whole prompts longer than two tiles, a portion behind a
+    cached prefix whose early pages the window has passed, and decoded tokens beside them."""
+    entries = [(1, 1), (300, 300), (260, 129), (75, 1), (131, 131)]
+    _check_window(_wide_ops(), torch.bfloat16, window, heads, kv_heads, head_dim, bs, entries)
+
+
+def _wide_ops():
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+    from mini_llm_runtime_amd.kernels.tuning import KernelTuning
+
+    return HipOps(torch.bfloat16, "cuda", tuning=KernelTuning(wide_attention_groups=1))
+
+
+def _check_window(ops, dtype, window, heads, kv_heads, head_dim, bs, entries):
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 22)
     got = ops.paged_attention(
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
@@ -562,10 +585,12 @@ def test_decode_attention_partitions(ops_for, heads, kv_heads, head_dim, partiti
 @pytest.mark.parametrize("heads,kv_heads,head_dim,bs,long", [
     (14, 2, 64, 16, 2048), (8, 2, 128, 16, 1100), (3, 1, 96, 8, 700), (2, 1, 256, 32, 600), (5, 5, 16, 64, 900),
 ])
-def test_prefill_attention_long_prompt_and_portion(ops_for, heads, kv_heads, head_dim, bs, long):
+@pytest.mark.parametrize("wide", [False, True])
+def test_prefill_attention_long_prompt_and_portion(ops_for, heads, kv_heads, head_dim, bs, long, wide):
     """The tiled prefill kernel on a long prompt (many key tiles, both key groups, tiles handed out
-    heavy first) and on a 300-token portion behind cached tokens, at several head and page sizes."""
-    ops = ops_for(torch.bfloat16)
+    heavy first) and on a 300-token portion behind cached tokens, at several head and page sizes;
+    with tiles of 64 queries and (forced: few tiles would not choose it) of 128."""
+    ops = ops_for(torch.bfloat16) if not wide else _wide_ops()
     entries = [(long, long), (long - 250, 300), (77, 77)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 27, spike=True)
     scale = head_dim**-0.5
