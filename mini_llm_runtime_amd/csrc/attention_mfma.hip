@@ -432,7 +432,11 @@ struct TileInFlight {
 // key and value operand read from LDS serves two matrix-core products, which halves the LDS
 // traffic per flop (LDS bandwidth, not the matrix cores, bounds the kernel with 1); it needs
 // twice the accumulators and is offered up to head size 128.
-template <int QB>
+// UNIFORM: the head size is a power of two and head size x page size at least 512 elements, so
+// that the 64 pieces a wavefront moves with one instruction lie in one page: the page ids are then looked up with scalar loads
+// and the addresses of the pieces are a scalar base plus a lane offset, which takes the
+// address arithmetic (a third of the vector instructions of a tile) off the vector unit.
+template <int QB, bool UNIFORM>
 __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ key_pages,
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
@@ -570,8 +574,10 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const int page0 = kt0 >> bs_shift;
 #pragma unroll
     for (int i = 0; i < kPieces; ++i) {
-      k_ids[i] = table[min(page0 + k_page[i], last_page)];
-      v_ids[i] = table[min(page0 + v_page[i], last_page)];
+      const int kp = UNIFORM ? __builtin_amdgcn_readfirstlane(k_page[i]) : k_page[i];
+      const int vp = UNIFORM ? __builtin_amdgcn_readfirstlane(v_page[i]) : v_page[i];
+      k_ids[i] = table[min(page0 + kp, last_page)];
+      v_ids[i] = table[min(page0 + vp, last_page)];
     }
   };
   auto fetch = [&](int kt0, TileInFlight& t) {  // with the ids that lookup(kt0) left
@@ -909,13 +915,13 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   MLR_REQUIRE(static_cast<int64_t>(num_tiles) * heads < (1ll << 31), "too many tiles for one launch");
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
-    if constexpr (D <= 128) {
-      if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<2>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
-    }
+    hipError_t e = hipSuccess;
+    const void* kernels[] = {reinterpret_cast<const void*>(attn_prefill_kernel<1, false>),
+                             reinterpret_cast<const void*>(attn_prefill_kernel<1, true>),
+                             reinterpret_cast<const void*>(attn_prefill_kernel<D <= 128 ? 2 : 1, false>),
+                             reinterpret_cast<const void*>(attn_prefill_kernel<D <= 128 ? 2 : 1, true>)};
+    for (const void* kernel : kernels)
+      if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLds);
     if (e != hipSuccess) {
       set_error(std::string("mlr_attention_prefill: cannot raise the LDS limit: ") + hipGetErrorString(e));
       return -1;
@@ -923,11 +929,22 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
     configured = true;
   }
   const dim3 grid(static_cast<unsigned>(num_tiles) * heads);
+  // a wavefront's 64 pieces of a tile lie in one page: whole key rows (D / 8 pieces each, a power
+  // of two) that fit a page, and as many pieces of a value page
+  const bool uniform = (D & (D - 1)) == 0 && D * block_size >= 512;
 #define MLR_PREFILL(qb)                                                                                       \
-  attn_prefill_kernel<qb><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                                   \
-      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                             \
-      static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,             \
-      static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window)
+  do {                                                                                                        \
+    if (uniform)                                                                                              \
+      attn_prefill_kernel<qb, true><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                         \
+          static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
+          static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);           \
+    else                                                                                                      \
+      attn_prefill_kernel<qb, false><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                        \
+          static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
+          static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);           \
+  } while (0)
   if constexpr (D <= 128) {
     if (wide)
       MLR_PREFILL(2);
