@@ -117,19 +117,37 @@ class ModelRunner:
         self.max_graph_tokens = int(max_graph_tokens)
         self._step_graphs: dict[tuple, tuple] = {}
         self._step_seen: dict[tuple, int] = {}
+        # One mixer per plan key makes the step's plan under that key (mixers that share a key
+        # make the same plan from the same shape), found once with a probe shape.
+        probe = PlanInput(np.ones(1, dtype=np.int32), np.zeros(1, dtype=np.int32), cache.block_size)
+        self._planners: dict[Any, Any] = {}
+        for entry in model.spec.order:
+            mixer = model.layers[entry.layer].mixer
+            plan = mixer.plan(ops, probe)
+            if plan is not None and plan.key not in self._planners:
+                self._planners[plan.key] = mixer
+        self._replayable = bool(model.replayable)  # the parts are fixed from here on
 
     # -------------------------------------------------------------------------------------------
-    def _validate(self, entries: Sequence[StepEntry]) -> None:
+    def _validate(self, entries: Sequence[StepEntry]) -> np.ndarray:
+        """Checks the entries and returns their token ids as one int32 array."""
         if not entries:
             raise ValueError("a step needs at least one entry")
+        ids = []
         for e in entries:
             if not e.tokens:
                 raise ValueError(f"request {e.request_id!r}: no tokens in this step")
-            for t in e.tokens:
-                if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < self.vocab_size:
-                    raise ValueError(
-                        f"request {e.request_id!r}: token {t!r} is outside the vocabulary of {self.vocab_size}"
-                    )
+            # prompts come in thousands of tokens: types and bounds are checked without a Python
+            # loop over them, which runs only to name the offender
+            tokens = np.asarray(e.tokens, dtype=np.int64) if set(map(type, e.tokens)) == {int} else None
+            if tokens is None or tokens.min() < 0 or tokens.max() >= self.vocab_size:
+                for t in e.tokens:
+                    if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < self.vocab_size:
+                        raise ValueError(
+                            f"request {e.request_id!r}: token {t!r} is outside the vocabulary of {self.vocab_size}"
+                        )
+                raise ValueError(f"request {e.request_id!r}: bad tokens")
+            ids.append(tokens)
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
                     raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
@@ -139,6 +157,7 @@ class ModelRunner:
                     f"request {e.request_id!r}: {cached + len(e.tokens)} tokens exceed "
                     f"max_position_embeddings={self.max_positions}"
                 )
+        return np.concatenate(ids).astype(np.int32)
 
     # ---- metadata of a step ------------------------------------------------------------------
     FIXED_ARRAYS = 9  # token ids, positions, token entries, cu_q, q_starts, context lengths, state rows (2), wanted rows
@@ -147,12 +166,13 @@ class ModelRunner:
         """The launch plans of the model's mixers for a step of this shape, one per plan key, in
         the order of the sites.  The step function uploads their arrays and keys its recordings
         by their sizes; what is in them is the mixers' business."""
-        plans: dict[Any, MixerPlan] = {}
-        for entry in self.model.spec.order:
-            plan = self.model.layers[entry.layer].mixer.plan(self.ops, shape)
-            if plan is not None and plan.key not in plans:
-                plans[plan.key] = plan
-        return list(plans.values())
+        plans = []
+        for key, mixer in self._planners.items():
+            plan = mixer.plan(self.ops, shape)
+            if plan is None or plan.key != key:
+                raise RuntimeError(f"the mixer that plans {key!r} made no plan under that key for a step's shape")
+            plans.append(plan)
+        return plans
 
     @staticmethod
     def _plan_sizes(plans: Sequence[MixerPlan]) -> tuple:
@@ -297,7 +317,7 @@ class ModelRunner:
         return -(-pages // quantum) * quantum
 
     def _recordable(self) -> bool:
-        return self.use_graphs and self.model.replayable
+        return self.use_graphs and self._replayable
 
     def _step_key(self, layout: StepLayout, logit_rows: np.ndarray) -> Optional[tuple]:
         """(identity of a recording, the plans it was derived from): the sizes that fix every launch
@@ -545,10 +565,9 @@ class ModelRunner:
         """Run one batch.  borrow_logits: the caller uses the logits before the next step and
         accepts a view of a recorded step's buffer (saves a copy).  capture_sites: also return
         the residual stream after every site at the wanted rows (runs unrecorded)."""
-        self._validate(entries)
+        token_ids = self._validate(entries)
         layout = self.cache.begin_step([(e.request_id, len(e.tokens)) for e in entries])
         try:
-            token_ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=layout.num_tokens)
             rows: list[tuple[str, int]] = []
             flat: list[int] = []
             for r, e in enumerate(entries):

@@ -83,7 +83,9 @@ class Mixer(Part):
         """What this mixer's kernels need planned on the host for a step of this shape (tiles,
         counts, launch sizes), or None.  The step function uploads the plan's arrays with the
         step's metadata, hands the plan to `forward` through `ctx.plan(key)`, and records a
-        step only for replay under plans of the same sizes; it knows nothing of what is in it."""
+        step only for replay under plans of the same sizes; it knows nothing of what is in it.
+        A mixer that plans does so for every shape, always under the same key; of several mixers
+        with the same key the first one's plan is used (they make the same plan from a shape)."""
         return None
 
     def forward(self, ctx: StepContext, h: torch.Tensor, site: int) -> torch.Tensor:
