@@ -581,7 +581,7 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
   if (mid >= 256) return {22, 1};
   if (mid >= 64) {
     int slices = 1;
-    while (slices < max_slices && slices < 4 && mid * slices < 256 && k / (2 * slices) >= 4096) slices *= 2;
+    while (slices < max_slices && slices < 4 && mid * slices < 256 && k / (2 * slices) >= 1024) slices *= 2;
     if (slices > 1) return {22, slices};
   }
   return {11, choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 4))};
