@@ -699,7 +699,10 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
   const bf16* xb = static_cast<const bf16*>(x);
   const bf16* wb = static_cast<const bf16*>(w);
   if (kernel == 0) {
-    kernel = m <= 64 ? 16 : choose_kernel(m, static_cast<int>(n), k, 1);
+    // Beyond 64 tokens the 64 x 64 tiles: with this epilogue (rotation, scattered cache stores) the
+    // larger tiles are slower than they are for the plain product, and where those would pay the
+    // caller does better with the plain product and the rotation kernel behind it.
+    kernel = m <= 64 ? 16 : 11;
     if (kernel == 16 && m > 16 && (n / 16) * m * k * 2 > (32ll << 20)) kernel = 11;  // too many passes over x
   }
   if (kernel == 8) {
