@@ -259,3 +259,29 @@ def test_safetensors_files_agree_with_the_safetensors_library(tmp_path):
             back = f.tensor(name)
             want = t.to(torch.int32) if t.dtype == torch.int64 and back.dtype == torch.int32 else t
             assert back.shape == t.shape and torch.equal(back.to(want.dtype), want), name
+
+
+# ---- the attention kernels' plan ------------------------------------------------------------------------
+def test_attention_plan_covers_every_query_once_in_both_tile_sizes():
+    """Both tile lists of the plan (64 and 128 queries) cover every token of every entry with more
+    than one new token exactly once, heaviest tiles first; single-token entries are only counted."""
+    import numpy as np
+
+    from mini_llm_runtime_amd.kernels.plans import QUERY_TILE, WIDE_QUERY_TILE, attention_plan
+    from mini_llm_runtime_amd.parts.context import PlanInput
+
+    q_lens = np.array([1, 300, 64, 1, 129, 2], dtype=np.int32)
+    q_starts = np.array([77, 0, 500, 9, 130, 4000], dtype=np.int32)
+    plan = attention_plan(PlanInput(q_lens, q_starts, 4096))
+    assert plan.sizes["num_decode_entries"] == 2 and plan.sizes["max_decode_context"] == 4096
+    for name, count, tile in (("query_tiles", "num_query_tiles", QUERY_TILE), ("wide_query_tiles", "num_wide_query_tiles", WIDE_QUERY_TILE)):
+        tiles = plan.arrays[name]
+        assert plan.sizes[count] == len(tiles)
+        covered = {r: np.zeros(n, dtype=int) for r, n in enumerate(q_lens) if n > 1}
+        for entry, q0 in tiles:
+            covered[int(entry)][q0 : q0 + tile] += 1
+        assert all((c == 1).all() for c in covered.values()), name
+        weights = [int(q_starts[e]) + int(q0) for e, q0 in tiles]
+        assert weights == sorted(weights, reverse=True), "tiles with the most keys before them come first"
+    no_prompts = attention_plan(PlanInput(np.ones(3, dtype=np.int32), np.zeros(3, dtype=np.int32), 64))
+    assert no_prompts.sizes["num_query_tiles"] == 0 and no_prompts.arrays["wide_query_tiles"].shape == (0, 2)
