@@ -142,6 +142,30 @@ def test_peaked_attention_mixed(tmp_path, which, backend, dtype):
     _compare(got, requests, weights, cfg, dtype, row_bound=0.2)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("family", ["whole", "portions", "mixed"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_wide_attention_tiles_through_the_step_function(tmp_path, which, family):
+    """Prompts of several hundred tokens with the prompt kernel's 128-query tiles forced (these
+    few tiles would not choose them): whole, in portions of changing size behind a cached prefix,
+    and mixed with decoded tokens of other requests, against the plain implementation."""
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+    from mini_llm_runtime_amd.kernels.tuning import KernelTuning
+
+    vocab = TINY[which]["vocab_size"]
+    requests = {f"w{i}": random_tokens(n, vocab, 300 + i) for i, n in enumerate((150, 290, 133, 260))}
+    steps = FAMILIES[family](requests)
+    model_dir = make_model_dir(tmp_path, which, seed=13)
+    cfg, weights = read_weights(model_dir)
+    bs = BLOCK_SIZE[which]
+    ops = HipOps(torch.bfloat16, "cuda", tuning=KernelTuning(wide_attention_groups=1))
+    _, _, cache, runner = make_runner(model_dir, ops, block_size=bs, num_blocks=schedules.pages_needed(steps, bs), max_requests=4)
+    cache.poison()
+    got = schedules.run_schedule(runner, cache, steps)
+    _compare(got, requests, weights, cfg, torch.bfloat16)
+    cache.check_invariants()
+
+
 @pytest.mark.parametrize("backend,dtype", CASES)
 @pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_schedules_agree_with_each_other(tmp_path, which, backend, dtype):
