@@ -216,7 +216,10 @@ struct TiledShape {
   static constexpr int BN = 32 * WN * GN;
   static constexpr int kPieces = (BM + BN) * (kBK / 8) / kThreads;  // 16-byte pieces per thread and slice
   static constexpr int kLds = 2 * (BM + BN) * kLd * 2;              // bytes, two buffers
-  static constexpr bool kDeep = WM * WN < 4 && GM * GN <= 4;        // loads two slices ahead for the small tiles
+  // slices of K in flight ahead of the one in LDS: one for the large tiles, two for the small ones
+  // (a slice of their work is shorter than a trip to memory; four were no faster, also for the
+  // tile of few tokens, which only streams weights)
+  static constexpr int kDepth = WM * WN >= 4 || GM * GN > 4 ? 1 : 2;
 };
 
 // Workgroup -> (slice, token tile, feature tile).  Consecutive workgroups go to the eight
@@ -249,7 +252,7 @@ __device__ __forceinline__ void place_workgroup(const TileOrder& order, int id, 
 // the rotated part (query and key heads) come in pairs: an even block holds 32 dims j of the
 // first half of their heads, the odd block after it their partners j + head_dim/2; tiles of the
 // value heads (and all tiles, without rotation) hold consecutive rows.
-template <int WM, int WN, bool DEEP, int GM = 2, int GN = 2, bool QKV = false>
+template <int WM, int WN, int DEPTH, int GM = 2, int GN = 2, bool QKV = false>
 __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                                   GemmEpilogue ep, QkvTarget qkv, TileOrder order, int M,
                                                                   int N, int K) {
@@ -338,11 +341,11 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // The LDS buffers run one slice ahead of the matrix cores.  DEEP: two register sets, so
-  // that loads run two slices ahead (with a small tile one slice of work is shorter than a
-  // trip to memory); otherwise one.  A slice past the end reads zeros through the range
-  // check, so the loop bodies need no conditions on it.
-  bf16x8_t reg_a[PIECES], reg_b[DEEP ? PIECES : 1];
+  // The LDS buffers run one slice ahead of the matrix cores, and DEPTH register sets hold the
+  // slices behind it on their way from memory (with a small tile one slice of work is shorter
+  // than a trip to memory).  A slice past the end reads zeros through the range check, so the
+  // loop bodies need no conditions on it.
+  bf16x8_t regs[DEPTH][PIECES];
   auto fetch = [&](int slice, auto& reg) {
     const int left = slice < s_end ? chunks - slice * (kBK / 8) : 0;  // chunks of K from this slice on
 #pragma unroll
@@ -375,28 +378,20 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
     }
   };
 
-  fetch(s_begin, reg_a);
-  if constexpr (DEEP) fetch(s_begin + 1, reg_b);
-  stash(0, reg_a);
+  // set j holds slice s + 1 + j while slice s is multiplied; the set that was stashed is loaded
+  // again at once, DEPTH slices further on
+#pragma unroll
+  for (int j = 0; j < DEPTH; ++j) fetch(s_begin + j, regs[j]);
+  stash(0, regs[0]);
   __syncthreads();
-  if constexpr (DEEP) {
-    for (int s = s_begin; s < s_end; s += 2) {
-      fetch(s + 2, reg_a);
-      multiply(0);
-      stash(1, reg_b);  // slice s + 1
-      __syncthreads();
-      if (s + 1 >= s_end) break;
-      fetch(s + 3, reg_b);
-      multiply(1);
-      stash(0, reg_a);  // slice s + 2
-      __syncthreads();
-    }
-  } else {
-    for (int s = s_begin; s < s_end; ++s) {
-      const int buf = (s - s_begin) & 1;
-      fetch(s + 1, reg_a);
+  for (int s = s_begin; s < s_end; s += DEPTH) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {
+      if (s + j >= s_end) break;
+      const int buf = (s + j - s_begin) & 1;
+      fetch(s + j + DEPTH, regs[j]);
       multiply(buf);
-      stash(buf ^ 1, reg_a);
+      stash(buf ^ 1, regs[(j + 1) % DEPTH]);  // slice s + j + 1
       __syncthreads();
     }
   }
@@ -486,10 +481,10 @@ template <int WM, int WN, int GM = 2, int GN = 2>
 static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
                         hipStream_t stream) {
   using Shape = TiledShape<WM, WN, GM, GN>;
-  constexpr bool kDeep = Shape::kDeep;
+  constexpr int kDepth = Shape::kDepth;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, kDeep, GM, GN>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, kDepth, GM, GN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLds);
     if (e != hipSuccess) {
       set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
@@ -503,7 +498,7 @@ static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, 
     set_error("mlr_gemm_bf16: too many tiles for one launch");
     return -1;
   }
-  gemm_tiled_kernel<WM, WN, kDeep, GM, GN><<<dim3(static_cast<unsigned>(groups)), Shape::kThreads, Shape::kLds, stream>>>(
+  gemm_tiled_kernel<WM, WN, kDepth, GM, GN><<<dim3(static_cast<unsigned>(groups)), Shape::kThreads, Shape::kLds, stream>>>(
       xb, wb, ep, QkvTarget{}, order, m, n, k);
   return 0;
 }
@@ -514,7 +509,7 @@ template <int WM, int WN, int GM = 2, int GN = 2>
 static int launch_tiled_qkv(const bf16* xb, const bf16* wb, GemmEpilogue ep, const QkvTarget& qkv, int m, int n, int k,
                             hipStream_t stream) {
   using Shape = TiledShape<WM, WN, GM, GN>;
-  constexpr bool kDeep = Shape::kDeep;
+  constexpr int kDepth = Shape::kDepth;
   static_assert(WN == 1 || WN == 2, "a rotated block finds its partner beside it or in the next wavefront");
   const int rot_pairs = qkv.cos != nullptr ? (qkv.heads + qkv.kv_heads) * (qkv.head_dim / 2) : 0;
   const int rot_tiles = (rot_pairs + Shape::BN / 2 - 1) / (Shape::BN / 2);
@@ -524,7 +519,7 @@ static int launch_tiled_qkv(const bf16* xb, const bf16* wb, GemmEpilogue ep, con
   MLR_REQUIRE(groups < (1ll << 31), "too many tiles for one launch");
   static bool prepared = false;
   if (!prepared) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, kDeep, GM, GN, true>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, kDepth, GM, GN, true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLds);
     if (e != hipSuccess) {
       set_error(std::string("mlr_qkv_rope_write_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
@@ -532,7 +527,7 @@ static int launch_tiled_qkv(const bf16* xb, const bf16* wb, GemmEpilogue ep, con
     }
     prepared = true;
   }
-  gemm_tiled_kernel<WM, WN, kDeep, GM, GN, true>
+  gemm_tiled_kernel<WM, WN, kDepth, GM, GN, true>
       <<<dim3(static_cast<unsigned>(groups)), Shape::kThreads, Shape::kLds, stream>>>(xb, wb, ep, qkv, order, m, n, k);
   MLR_LAUNCH_CHECK();
   return 0;
