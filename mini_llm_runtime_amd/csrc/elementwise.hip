@@ -32,10 +32,12 @@ __global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ ta
 // The not-yet-added delta is either one tensor in the engine's dtype or `slices`
 // float32 partial sums [slice, rows, hidden] of a product that was cut along k;
 // they are added in slice order, so the sum does not depend on timing.
-// One workgroup per row; a row of up to 256 * 4 * VPT elements stays in registers
-// between the statistics and the scaling (hidden must be a multiple of 4).
-template <typename T, typename TW, int VPT>
-__global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+// One workgroup per row; a row of up to THREADS * 4 * VPT elements stays in registers
+// between the statistics and the scaling (hidden must be a multiple of 4).  Few wide rows
+// (a decode step of a large model) take 1,024 threads each: a compute unit takes in what its
+// wavefronts keep in flight, and a row with eight slices of partial sums is 100 KB and more.
+template <typename T, typename TW, int VPT, int THREADS = 256>
+__global__ __launch_bounds__(THREADS) void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
                                                       const float* __restrict__ partial, int slices, int rows,
                                                       const TW* __restrict__ weight, T* __restrict__ out,
                                                       int hidden, float eps) {
@@ -49,7 +51,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
   f32x4 v[VPT];
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    const int i = min(threadIdx.x + j * 256, quads - 1);
+    const int i = min(threadIdx.x + j * THREADS, quads - 1);
     const int64_t at = row * hidden + 4 * i;
     v[j] = *reinterpret_cast<const f32x4*>(x + at);
     if (delta != nullptr) {
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
     f32x4 p[VPT][kSliceBatch];
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
-      const int i = min(threadIdx.x + j * 256, quads - 1);
+      const int i = min(threadIdx.x + j * THREADS, quads - 1);
 #pragma unroll
       for (int u = 0; u < kSliceBatch; ++u) {
         const int sl = min(s0 + u, slices - 1);
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
   const bool changed = delta != nullptr || slices > 0;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    const int i = threadIdx.x + j * 256;
+    const int i = threadIdx.x + j * THREADS;
     if (i >= quads) {
       v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
       continue;
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
   const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    const int i = threadIdx.x + j * 256;
+    const int i = threadIdx.x + j * THREADS;
     if (i >= quads) continue;
     const int64_t at = row * hidden + 4 * i;
 #pragma unroll
@@ -136,6 +138,10 @@ static void launch_rmsnorm(float* x, const void* delta, const float* partial, in
   const int quads = hidden / 4;
   if (hidden % 4 != 0 || quads > 256 * 8)
     rmsnorm_any_kernel<T, TW><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
+  else if (rows <= 64 && quads > 512 && quads <= 1024)
+    rmsnorm_kernel<T, TW, 1, 1024><<<rows, 1024, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
+  else if (rows <= 64 && quads > 1024)
+    rmsnorm_kernel<T, TW, 2, 1024><<<rows, 1024, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
   else if (quads <= 256)
     rmsnorm_kernel<T, TW, 1><<<rows, 256, 0, stream>>>(x, d, partial, slices, rows, w, o, hidden, eps);
   else if (quads <= 512)
