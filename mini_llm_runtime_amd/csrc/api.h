@@ -57,6 +57,15 @@ int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, 
                       int head_dim, int rotary_dim, int block_size, int num_pages, int write,
                       hipStream_t stream);
 
+// The query/key/value product of few tokens that came as `slices` float32 partial sums
+// [slice, tokens, (heads + 2 kv_heads) * head_dim] (mlr_gemm_bf16 with slices, the bias in slice
+// 0): added up in order, rounded to bfloat16, query and key heads rotated over the whole head
+// (cos, sin: [tokens, head_dim / 2], or null), queries to q_out [tokens, heads * head_dim], keys
+// and values into their cache slots (`write` 0: none).  bfloat16 only.
+int mlr_qkv_finish(const float* partial, int slices, const float* cos, const float* sin, const int* slots,
+                   void* key_pages, void* value_pages, void* q_out, int tokens, int heads, int kv_heads, int head_dim,
+                   int block_size, int num_pages, int write, hipStream_t stream);
+
 // y[M, N] = x[M, K] * w[N, K]^T (+ bias[N]); x, w in `dtype`; bias float32 when
 // bias_is_f32 else `dtype` (null: none); y float32 when out_is_f32 else `dtype`.
 // Plain 32-bit FMA arithmetic on every path (no matrix-core rounding).

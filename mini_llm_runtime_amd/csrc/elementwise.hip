@@ -280,6 +280,74 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   }
 }
 
+// ---- the query/key/value product that came as K slices -----------------------------------------
+// A wide product of few tokens streams its weights fastest through the LDS-tiled kernel cut
+// along K, which leaves float32 partial sums [slice, token, width] (the bias in slice 0).  This
+// kernel finishes them as the fused kernels would: the slices are added in their order, the sum
+// is rounded to bfloat16 (what the unfused product hands on), query and key heads are rotated
+// (qwen_model_runner.py:56-61: dim j with j + head_dim / 2), queries go to q_out
+// [token, heads * head_dim], keys and values into the token's cache slot (:105-109).  One
+// wavefront per (token, head).
+__global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict__ partial, int slices,
+                                                       const float* __restrict__ cos_t,
+                                                       const float* __restrict__ sin_t,
+                                                       const int* __restrict__ slots, bf16* __restrict__ key_pages,
+                                                       bf16* __restrict__ value_pages, bf16* __restrict__ q_out,
+                                                       int tokens, int heads, int kv_heads, int head_dim,
+                                                       int block_size, int num_pages) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;
+  const int half = head_dim / 2;
+  const int64_t width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  const int64_t slice_stride = static_cast<int64_t>(tokens) * width;
+  const float* row = partial + t * width + static_cast<int64_t>(head) * head_dim;
+  const bool rotated = cos_t != nullptr && head < heads + kv_heads;
+  // where this head's values go
+  bf16* q_row = nullptr;
+  bf16* key_row = nullptr;    // [head_dim] of the token's slot
+  bf16* value_col = nullptr;  // dim d at value_col[d * block_size]
+  if (head < heads) {
+    q_row = q_out + (static_cast<int64_t>(t) * heads + head) * head_dim;
+  } else if (slots != nullptr) {
+    const int slot = slots[t];
+    if (slot >= 0 && slot / block_size < num_pages) {
+      const int page = slot / block_size, off = slot - page * block_size;
+      if (head < heads + kv_heads)
+        key_row = key_pages + ((static_cast<int64_t>(page) * kv_heads + (head - heads)) * block_size + off) * head_dim;
+      else
+        value_col = value_pages + (static_cast<int64_t>(page) * kv_heads + (head - heads - kv_heads)) * head_dim * block_size + off;
+    }
+  }
+  for (int j = threadIdx.x; j < half; j += 64) {
+    float a = 0.f, b = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < slices; ++s) {
+      a += row[s * slice_stride + j];
+      b += row[s * slice_stride + j + half];
+    }
+    a = to_f32(f32_to_bf16(a));
+    b = to_f32(f32_to_bf16(b));
+    float ra = a, rb = b;
+    if (rotated) {
+      const float c = cos_t[static_cast<int64_t>(t) * half + j];
+      const float sn = sin_t[static_cast<int64_t>(t) * half + j];
+      ra = a * c - b * sn;
+      rb = b * c + a * sn;
+    }
+    const bf16 lo = f32_to_bf16(ra), hi = f32_to_bf16(rb);
+    if (q_row != nullptr) {
+      q_row[j] = lo;
+      q_row[j + half] = hi;
+    } else if (key_row != nullptr) {
+      key_row[j] = lo;
+      key_row[j + half] = hi;
+    } else if (value_col != nullptr) {
+      value_col[static_cast<int64_t>(j) * block_size] = lo;
+      value_col[static_cast<int64_t>(j + half) * block_size] = hi;
+    }
+  }
+}
+
 }  // namespace mlr
 
 using namespace mlr;
@@ -412,6 +480,23 @@ int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, 
     rope_kv_write_kernel<bf16><<<tokens, 256, 0, stream>>>(
         static_cast<bf16*>(qkv), cos, sin, slots, static_cast<bf16*>(key_pages),
         static_cast<bf16*>(value_pages), heads, kv_heads, head_dim, rotary_dim, block_size, num_pages, write);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_qkv_finish(const float* partial, int slices, const float* cos, const float* sin, const int* slots,
+                   void* key_pages, void* value_pages, void* q_out, int tokens, int heads, int kv_heads, int head_dim,
+                   int block_size, int num_pages, int write, hipStream_t stream) {
+  MLR_REQUIRE(partial && q_out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && tokens <= 65535 && heads > 0 && kv_heads > 0 && heads + 2 * kv_heads <= 65535, "bad sizes");
+  MLR_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "head_dim must be even");
+  MLR_REQUIRE(slices >= 1 && slices <= 64, "slices must lie within 1..64");
+  MLR_REQUIRE((cos == nullptr) == (sin == nullptr), "cos and sin come together");
+  MLR_REQUIRE(!write || (slots && key_pages && value_pages && block_size > 0 && num_pages > 0),
+              "a cache write needs slots, pages and their sizes");
+  qkv_finish_kernel<<<dim3(tokens, heads + 2 * kv_heads), 64, 0, stream>>>(
+      partial, slices, cos, sin, write ? slots : nullptr, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages),
+      static_cast<bf16*>(q_out), tokens, heads, kv_heads, head_dim, block_size, num_pages);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -36,6 +36,7 @@ _SIGNATURES = {
     "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_rope_table": ([_VP, _VP, _VP, _VP, _I, _I, _VP], _I),
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
@@ -521,6 +522,7 @@ class HipOps:
         write: bool = True,
         fused: Optional[bool] = None,
         mfma_kernel: int = 0,
+        sliced: Optional[bool] = None,
     ) -> torch.Tensor:
         """Query/key/value product, rotation of queries and keys, keys and values into the cache.
 
@@ -528,8 +530,11 @@ class HipOps:
         queries, for `paged_attention`.  In bfloat16 with a full rotation this is ONE kernel
         that rotates the sums and stores them where they belong (a row-splitting kernel for up
         to 64 tokens, a tiled one beyond) unless the product is large; everything else is the
-        product followed by `rope_kv_write`.  `fused` forces one of the two ways, `mfma_kernel` the fused kernel
-        (tests).
+        product followed by `rope_kv_write`.  Up to 64 tokens of a wide product (tens of
+        megabytes of weights) go a third way: the product cut
+        along k through the LDS-tiled kernel, which streams such weights twice as fast as the
+        row-splitting one, and a small kernel that adds the slices up, rotates and stores.
+        `fused` and `sliced` force a way, `mfma_kernel` the fused kernel (tests).
         """
         pending = x if isinstance(x, PendingNorm) and x.value is None else None
         if isinstance(x, PendingNorm) and pending is None:
@@ -543,6 +548,38 @@ class HipOps:
             and (rotation is None or rotation[2] == head_dim)
             and (m <= 16 or width * k * 2 < 1 << 31)
         )
+        if sliced is None:
+            # measured: the second kernel costs 3.5 to 5 us, which the tiled product wins back from
+            # 24 MB of weights on (from 4 tokens; 64 MB: from one), or from 8 MB beyond 32 tokens
+            weight_bytes = width * k * 2
+            pays = (
+                weight_bytes >= 64 << 20
+                or (weight_bytes >= 24 << 20 and m >= 4)
+                or (weight_bytes >= 8 << 20 and m > 32)
+            )
+            sliced = fused is None and can_fuse and pending is None and not mfma_kernel and m <= 64 and pays and k >= 512
+        elif sliced and not (can_fuse and pending is None and m <= 64 and k >= 512):
+            raise KernelError("the sliced query/key/value product takes up to 64 bfloat16 tokens and a full rotation")
+        if sliced:
+            slices = 8 if k >= 2048 else 4
+            partial = self.linear(x, weight, bias, partial_sums=True, slices=slices)
+            cos = sin = None
+            if rotation is not None:
+                cos, sin, _ = rotation
+                self._check(cos, "rotary cos", torch.float32, (m, head_dim // 2))
+                self._check(sin, "rotary sin", torch.float32, (m, head_dim // 2))
+            num_pages = 0
+            if write:
+                num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
+                self._check(slot_mapping, "slot mapping", torch.int32, (m,))
+            q = self._empty((m, num_heads * head_dim), self.dtype)
+            self._call(
+                "mlr_qkv_finish", self._ptr(partial), slices, self._ptr(cos), self._ptr(sin),
+                self._ptr(slot_mapping if write else None), self._ptr(key_pages if write else None),
+                self._ptr(value_pages if write else None), self._ptr(q), m, num_heads, num_kv_heads, head_dim,
+                block_size, num_pages, int(write), self._stream(),
+            )
+            return q
         if fused is None:
             # Measured at 2,048 tokens: the fused kernel wins while the product is small (0.5B to 3B
             # widths, and any width up to some 512 tokens); where the plain product would run in

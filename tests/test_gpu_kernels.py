@@ -350,6 +350,50 @@ def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads,
     assert torch.isnan(out[True][1]).all() == (not write)
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,tokens,rotate,write", [
+    (14, 2, 64, 896, 64, True, True), (14, 2, 64, 896, 33, True, True), (3, 1, 16, 520, 1, True, True),
+    (5, 1, 128, 1208, 8, True, True), (4, 4, 80, 640, 17, False, True), (6, 3, 48, 2056, 5, True, False),
+    (28, 4, 128, 3584, 8, True, True),
+])
+def test_sliced_qkv_product_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write):
+    """The third way of the query/key/value product (cut along k through the tiled kernel, then one
+    kernel that adds the slices, rotates and stores) against the product followed by the rotation
+    kernel: same queries, same pages, no other slot touched; and the way is chosen by itself for
+    a wide product."""
+    ops = ops_for(torch.bfloat16)
+    bs, pages = 8, max(9, tokens // 8 + 2)
+    width = (heads + 2 * kv_heads) * head_dim
+    x = _rand((tokens, hidden), torch.bfloat16, 171).cuda()
+    w = _rand((width, hidden), torch.bfloat16, 172, 0.2).cuda()
+    b = _rand((width,), torch.float32, 173).cuda()
+    rotation = None
+    if rotate:
+        pos = torch.tensor(([3, 0, 911, 17, 40000] + list(range(5, tokens)))[:tokens], dtype=torch.int32).cuda()
+        inv = (1.0 / (1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))).cuda()
+        cos, sin = ops.rope_table(pos, inv)
+        rotation = (cos, sin, head_dim)
+    g = torch.Generator().manual_seed(174)
+    slots = torch.randperm(pages * bs, generator=g)[:tokens].to(torch.int32)
+    if tokens > 2:
+        slots[2] = -1
+    slots = slots.cuda()
+    out = {}
+    for way in ("unfused", "sliced", "auto"):
+        kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=torch.bfloat16).cuda()
+        vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=torch.bfloat16).cuda()
+        kw = dict(fused=False, sliced=False) if way == "unfused" else (dict(sliced=True) if way == "sliced" else {})
+        q = ops.qkv_rope_write(x, w, b, rotation, slots, kp, vp, num_heads=heads, num_kv_heads=kv_heads,
+                               head_dim=head_dim, block_size=bs, write=write, **kw)
+        out[way] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
+    for name, a, c in zip(("queries", "key pages", "value pages"), out["unfused"], out["sliced"]):
+        assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
+        torch.testing.assert_close(torch.nan_to_num(c), torch.nan_to_num(a), msg=lambda m: f"{name}: {m}", **_tol(torch.bfloat16))
+    assert torch.isnan(out["sliced"][1]).all() == (not write)
+    if width * hidden * 2 >= 24 << 20 and tokens >= 4:
+        for a, c in zip(out["sliced"], out["auto"]):
+            assert torch.equal(torch.nan_to_num(a), torch.nan_to_num(c)), "the sliced way is chosen by itself here"
+
+
 # ---- attention ----------------------------------------------------------------------------------------
 def _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, seed, extra_pages=3, spike=False):
     """entries: list of (context_len, q_len).  Returns device inputs and the float64 expectation."""
