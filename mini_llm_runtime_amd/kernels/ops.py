@@ -748,8 +748,11 @@ class HipOps:
             # products, once there are enough of them to keep every compute unit busy all the same
             tiles, wide = plan.query_tiles, 0
             num_wide = int(getattr(plan, "num_wide_query_tiles", 0))
+            enough = self.tuning.wide_attention_groups
+            if int(getattr(plan, "long_prefix", 0)):
+                enough //= 2  # heavy tiles everywhere: one workgroup per compute unit is enough
             if (
-                num_wide * num_heads >= self.tuning.wide_attention_groups
+                num_wide * num_heads >= enough
                 and getattr(plan, "wide_query_tiles", None) is not None
                 and lib.mlr_attention_wide_tile() == WIDE_QUERY_TILE
             ):

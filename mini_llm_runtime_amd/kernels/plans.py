@@ -11,6 +11,7 @@ from ..parts.context import MixerPlan, PlanInput
 
 QUERY_TILE = 64  # queries of one request that the prompt kernel takes together
 WIDE_QUERY_TILE = 128  # and in its variant for long prompts (two blocks of queries per wavefront)
+LONG_PREFIX_KEYS = 4096  # mean number of keys before a tile from which a step counts as behind long prefixes
 PAGED_ATTENTION = "paged_attention"  # the plan's key: every mixer on these kernels shares one plan per step
 
 
@@ -36,12 +37,17 @@ def attention_plan(shape: PlanInput) -> MixerPlan:
     decodes = int(single.sum())
     tiles = query_tiles(shape.q_lens, shape.q_starts)
     wide = query_tiles(shape.q_lens, shape.q_starts, WIDE_QUERY_TILE)
+    # portions behind long cached prefixes: every tile has thousands of keys before it, so even few
+    # tiles keep the compute units busy for long and the wide tiles' lower cost per key wins
+    keys_before = [int(shape.q_starts[e]) + int(q0) for e, q0 in wide]
+    long_prefix = int(bool(keys_before) and sum(keys_before) >= LONG_PREFIX_KEYS * len(keys_before))
     return MixerPlan(
         key=PAGED_ATTENTION,
         arrays={"query_tiles": tiles, "wide_query_tiles": wide},
         sizes={
             "num_query_tiles": len(tiles),
             "num_wide_query_tiles": len(wide),
+            "long_prefix": long_prefix,
             "num_decode_entries": decodes,
             "max_decode_context": int(shape.max_context) if decodes else 0,
         },
