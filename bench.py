@@ -13,7 +13,8 @@ bytes it must read (every weight once and the live requests' cache) against
 8 TB/s.  Peaks are MI355X's published dense figures.  `points_7b` and `points_32b`
 (default run only; `--no-large` leaves them out) hold decode at batch 8 and the
 prefill for the two larger shapes, with the number of layers run and of the full
-model beside them.
+model beside them; `points_ctx16k` the same two measurements at a context of 16,384
+tokens for the 0.5B and the 7B shape.
 
 How it measures (the reference's harness rules, src/mini_llm_runtime/timing.py:49-82,
 141-160 and environment.py:37-93): untimed warm-up first; the timed steps between
@@ -45,6 +46,23 @@ PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 PROMPT_LEN = 2048
 CONTEXT_LEN = 4096
 BLOCK_SIZE = 16
+
+
+def long_context_points(args) -> dict:
+    """Decode at batch 8 and the prefill at a context of 16,384 tokens, for the 0.5B and the 7B shape."""
+    import copy
+
+    long_args = copy.copy(args)
+    long_args.prompt_len = 16384
+    out = {"context": long_args.prompt_len}
+    for tag, name, layers in (("0.5b", "qwen2.5-0.5b", None), ("7b", "qwen2.5-7b", 28)):
+        point = large_point(long_args, name, layers)
+        out[f"decode_b8_{tag}"] = point["decode_b8"]
+        out[f"decode_b8_{tag}_hbm_frac"] = point["decode_b8_hbm_frac"]
+        if "prefill" in point:
+            out[f"prefill_{tag}_ms"] = point["prefill_ms"]
+            out[f"prefill_{tag}_frac"] = point["prefill_frac"]
+    return out
 
 
 def parse_args() -> argparse.Namespace:
@@ -553,6 +571,8 @@ def main() -> int:
     if not args.no_large and args.config == "qwen2.5-0.5b" and args.layers is None and args.dtype == "bfloat16":
         line["points_7b"] = large_point(args, "qwen2.5-7b", 28)
         line["points_32b"] = large_point(args, "qwen2.5-32b", 16)
+        if args.prompt_len == PROMPT_LEN:
+            line["points_ctx16k"] = long_context_points(args)
     line["env"] = environment()
     print(json.dumps(line), flush=True)
     return 0
