@@ -442,7 +442,10 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
-    int window) {
+    int window, float* __restrict__ partial) {
+  // gridDim.y > 1: the keys of every tile are cut into that many runs, one workgroup each, which
+  // leave their unnormalised results in `partial` for attn_prefill_merge (few tiles behind a long
+  // context would otherwise be as many long chains on a few compute units).
   // Two groups of four wavefronts work on the same 64 queries; group g takes the key tiles
   // g, g + 2, g + 4, ... and the groups' states are merged at the end.  The heaviest tiles (the
   // end of a long prompt) bound the kernel's time by their chain of key tiles, one after the
@@ -507,7 +510,14 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   const int last_q = min(q0 + kWgQ, q_len) - 1;
   const int k_end = pos0 + last_q + 1;
   const int k_begin_raw = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
-  const int k_begin = (k_begin_raw / kTileK) * kTileK;
+  const int k_begin_all = (k_begin_raw / kTileK) * kTileK;
+  // this workgroup's run of the keys: whole turns of the loop below (all key groups together)
+  constexpr int kTurn = kKeyGroups * kTileK;
+  const int splits = gridDim.y;
+  const int turns = (k_end - k_begin_all + kTurn - 1) / kTurn;
+  const int turns_each = (turns + splits - 1) / splits;
+  const int k_begin = k_begin_all + static_cast<int>(blockIdx.y) * turns_each * kTurn;
+  const int k_stop = min(k_end, k_begin + turns_each * kTurn);  // keys from here on belong to the next run
   // the wavefront's own range (uniform within the wavefront)
   const int w_last = pos0 + min(q0 + wave * kWaveQ + kWaveQ - 1, q_len - 1);
   const int w_first = window > 0 ? max(0, pos0 + q0 + wave * kWaveQ - window + 1) : 0;
@@ -625,7 +635,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   TileInFlight flight;
   constexpr int kStep = kKeyGroups * kTileK;  // keys per turn of the loop, all groups together
   const int k_mine = k_begin + group * kTileK;  // this group's first tile
-  if (k_mine < k_end) {
+  if (k_mine < k_stop) {
     lookup(k_mine);
     fetch(k_mine, flight);
     lookup(k_mine + kStep);
@@ -633,9 +643,9 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   }
   __syncthreads();
   int buf = 0;
-  for (int kt0 = k_mine; kt0 - group * kTileK < k_end; kt0 += kStep, buf ^= 1) {  // as many turns for every group
-    const bool mine = kt0 < k_end;
-    const bool more = kt0 + kStep < k_end;
+  for (int kt0 = k_mine; kt0 - group * kTileK < k_stop; kt0 += kStep, buf ^= 1) {  // as many turns for every group
+    const bool mine = kt0 < k_stop;
+    const bool more = kt0 + kStep < k_stop;
     if (more) {
       fetch(kt0 + kStep, flight);  // in flight while this tile is computed
       lookup(kt0 + 2 * kStep);
@@ -783,6 +793,25 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     float l = l_run[b];
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
+    if (splits > 1) {
+      // this run's share, unnormalised: [tile, head, run, query of the tile, head size + 2]
+      float* dst = partial + (((static_cast<int64_t>(tile) * heads + head) * splits + blockIdx.y) * kWgQ +
+                              (wave * kWaveQ + b * 16 + col)) * kPartialStride;
+      typedef float f32x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int dt = 0; dt < kDimTiles; ++dt) {
+        const float nan = __builtin_nanf("");
+        *reinterpret_cast<f32x2_t*>(dst + dt * 16 + quarter * 4) =
+            f32x2_t{poisoned ? nan : acc[b][dt][0], poisoned ? nan : acc[b][dt][1]};
+        *reinterpret_cast<f32x2_t*>(dst + dt * 16 + quarter * 4 + 2) =
+            f32x2_t{poisoned ? nan : acc[b][dt][2], poisoned ? nan : acc[b][dt][3]};
+      }
+      if (quarter == 0) {
+        dst[D] = m_run[b];
+        dst[D + 1] = l;
+      }
+      continue;
+    }
     if (q_ok[b]) {
       const float inv = 1.0f / l;
       bf16* orow = out + (static_cast<int64_t>(t_first + qi[b]) * heads + head) * D;
@@ -795,6 +824,43 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
         *reinterpret_cast<u16x4_t*>(orow + dt * 16 + quarter * 4) = packed;
       }
     }
+  }
+}
+
+// Merge of the key runs of a prompt tile (see attn_prefill_kernel): for every query of the tile
+// and every head, m = max m_j, w_j = 2^(m_j - m), O = sum w_j a_j / sum w_j l_j, in the runs'
+// order.  One workgroup per (tile, head).
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ partial,
+                                                                 const int* __restrict__ tiles,
+                                                                 const int* __restrict__ cu_q,
+                                                                 bf16* __restrict__ out, int heads, int splits,
+                                                                 int tile_q) {
+  const int tile = blockIdx.x / heads;
+  const int head = blockIdx.x - tile * heads;
+  const int entry = tiles[2 * tile];
+  const int q0 = tiles[2 * tile + 1];
+  const int t_first = cu_q[entry];
+  const int q_len = cu_q[entry + 1] - t_first;
+  const float* base = partial + static_cast<int64_t>(blockIdx.x) * splits * tile_q * kPartialStride;
+  for (int idx = threadIdx.x; idx < tile_q * (D / 2); idx += 256) {
+    const int qq = idx / (D / 2);
+    const int d = (idx - qq * (D / 2)) * 2;
+    if (q0 + qq >= q_len) continue;
+    float mstar = -INFINITY;
+    for (int sp = 0; sp < splits; ++sp)
+      mstar = fmaxf(mstar, base[(static_cast<int64_t>(sp) * tile_q + qq) * kPartialStride + D]);
+    float num0 = 0.f, num1 = 0.f, den = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const float* row = base + (static_cast<int64_t>(sp) * tile_q + qq) * kPartialStride;
+      const float m = row[D];
+      const float w = (m == -INFINITY) ? 0.f : fast_exp2(m - mstar);
+      num0 += w * row[d];
+      num1 += w * row[d + 1];
+      den += w * row[D + 1];
+    }
+    bf16* orow = out + (static_cast<int64_t>(t_first + q0 + qq) * heads + head) * D;
+    orow[d] = f32_to_bf16(num0 / den);
+    orow[d + 1] = f32_to_bf16(num1 / den);
   }
 }
 
@@ -891,13 +957,25 @@ int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int*
 // size has none.
 int mlr_attention_wide_tile() { return D <= 128 ? 2 * kTileQ : 0; }
 
+// Floats of scratch mlr_attention_prefill needs when the keys of every tile are cut into
+// `splits` runs (0 for one run).
+int64_t mlr_attention_prefill_scratch(int num_tiles, int heads, int splits, int wide) {
+  if (splits <= 1) return 0;
+  return static_cast<int64_t>(num_tiles) * heads * splits * (wide ? 2 * kTileQ : kTileQ) * kPartialStride;
+}
+
 // Attention of the query tiles listed in `tiles` ([num_tiles][2]: entry, first
 // query of the tile within the entry's new tokens; 64 queries per tile, or
-// mlr_attention_wide_tile() with `wide`).
+// mlr_attention_wide_tile() with `wide`).  splits > 1: the keys of every tile are cut into that
+// many runs, each a workgroup of its own, and merged by a second kernel; `partial` then holds
+// mlr_attention_prefill_scratch floats.  For few tiles behind long contexts.
 int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
                           const int* block_table, int table_width, const int* tiles, int num_tiles, int wide,
                           const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
-                          int block_size, int num_pages, float scale, int window, hipStream_t stream) {
+                          int block_size, int num_pages, float scale, int window, int splits, float* partial,
+                          hipStream_t stream) {
+  MLR_REQUIRE(splits >= 1 && splits <= 64, "splits must lie within 1..64");
+  MLR_REQUIRE(splits == 1 || partial != nullptr, "several key runs need scratch memory");
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(num_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad sizes");
   MLR_REQUIRE(kv_heads <= 65535, "too many key/value heads");  // a page's elements fit 32 bits
@@ -928,7 +1006,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
     }
     configured = true;
   }
-  const dim3 grid(static_cast<unsigned>(num_tiles) * heads);
+  const dim3 grid(static_cast<unsigned>(num_tiles) * heads, splits);
   // a wavefront's 64 pieces of a tile lie in one page: whole key rows (D / 8 pieces each, a power
   // of two) that fit a page, and as many pieces of a value page
   const bool uniform = (D & (D - 1)) == 0 && D * block_size >= 512;
@@ -938,12 +1016,12 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
       attn_prefill_kernel<qb, true><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                         \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
-          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);           \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, partial);  \
     else                                                                                                      \
       attn_prefill_kernel<qb, false><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                        \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
-          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window);           \
+          static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, partial);  \
   } while (0)
   if constexpr (D <= 128) {
     if (wide)
@@ -955,6 +1033,12 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   }
 #undef MLR_PREFILL
   MLR_LAUNCH_CHECK();
+  if (splits > 1) {
+    const int tile_q = (wide && D <= 128) ? 2 * kTileQ : kTileQ;
+    attn_prefill_merge_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256, 0, stream>>>(
+        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q);
+    MLR_LAUNCH_CHECK();
+  }
   return 0;
 }
 

@@ -68,8 +68,9 @@ _SIGNATURES = {
         _I,
     ),
     "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_attention_prefill_scratch": ([_I, _I, _I, _I], _I64),
     "mlr_attention_prefill": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _VP, _VP],
         _I,
     ),
 }
@@ -758,11 +759,22 @@ class HipOps:
             ):
                 tiles, num_tiles, wide = plan.wide_query_tiles, num_wide, 1
             self._check(tiles, "query tiles", torch.int32, (num_tiles, 2))
+            # few tiles behind long contexts: as many long chains on a few compute units; their keys
+            # are cut into runs with a workgroup each, merged by a second kernel
+            groups = num_tiles * num_heads
+            key_runs = 1
+            if int(getattr(plan, "long_prefix", 0)) and groups < self.tuning.wide_attention_groups // 2:
+                key_runs = min(8, -(-self.tuning.wide_attention_groups // groups))
+            partial = None
+            if key_runs > 1:
+                partial = self._empty(
+                    (lib.mlr_attention_prefill_scratch(num_tiles, num_heads, key_runs, wide),), torch.float32
+                )
             self._call(
                 "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(tiles), num_tiles, wide, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
-                float(scale), int(window or 0), self._stream(), lib=lib,
+                float(scale), int(window or 0), key_runs, self._ptr(partial), self._stream(), lib=lib,
             )
         return out
 

@@ -442,8 +442,15 @@ def _plan(entries, token_entry, positions):
     cu = [0]
     for n in q_lens:
         cu.append(cu[-1] + n)
-    tiles = query_tiles(q_lens)
-    wide = query_tiles(q_lens, tile=128)
+    import numpy as np
+
+    from mini_llm_runtime_amd.kernels.plans import attention_plan
+    from mini_llm_runtime_amd.parts.context import PlanInput
+
+    q_starts = [c - ql for c, ql in entries]
+    tiles = query_tiles(q_lens, q_starts)
+    wide = query_tiles(q_lens, q_starts, tile=128)
+    planned = attention_plan(PlanInput(np.asarray(q_lens, dtype=np.int32), np.asarray(q_starts, dtype=np.int32), max(c for c, _ in entries)))
     singles = [c for c, ql in entries if ql == 1]
     return SimpleNamespace(
         num_entries=len(entries),
@@ -457,6 +464,7 @@ def _plan(entries, token_entry, positions):
         num_query_tiles=len(tiles),
         wide_query_tiles=torch.from_numpy(wide).cuda() if len(wide) else None,
         num_wide_query_tiles=len(wide),
+        long_prefix=planned.sizes["long_prefix"],
         num_decode_entries=len(singles),
         max_decode_context=max(singles, default=0),
     )
@@ -637,6 +645,25 @@ def test_prefill_attention_long_prompt_and_portion(ops_for, heads, kv_heads, hea
     ops = ops_for(torch.bfloat16) if not wide else _wide_ops()
     entries = [(long, long), (long - 250, 300), (77, 77)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 27, spike=True)
+    scale = head_dim**-0.5
+    got = ops.paged_attention(
+        q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
+        num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
+    ).cpu()
+    ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.double(), ref, **_tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,bs,wide", [(4, 2, 64, 16, False), (6, 2, 128, 16, False), (3, 1, 32, 8, True), (2, 2, 256, 32, False)])
+def test_prompt_portions_behind_long_contexts_in_key_runs(ops_for, heads, kv_heads, head_dim, bs, wide):
+    """Few query tiles behind thousands of cached tokens: the keys of every tile are cut into runs,
+    a workgroup each, and merged; portions of 2 to 200 tokens, a whole short prompt beside them (its
+    tiles have runs without keys), and a far key that carries the result."""
+    ops = ops_for(torch.bfloat16) if not wide else _wide_ops()
+    entries = [(9000, 200), (12000, 2), (70, 70), (8200, 65)]
+    q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 43, spike=True)
+    assert ctx.long_prefix == 1
     scale = head_dim**-0.5
     got = ops.paged_attention(
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
