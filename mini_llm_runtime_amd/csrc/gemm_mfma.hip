@@ -542,10 +542,8 @@ static int choose_slices(int groups, int ksteps, int allowed) {
   return slices;
 }
 
-// Tiles of a shape under the 64 x 64 and the 128 x 128 tiling.
+// Tiles of a shape under the 64 x 64 tiling.
 static int tiles_64(int m, int n) { return ((n + 63) / 64) * ((m + 63) / 64); }
-static int tiles_128(int m, int n) { return ((n + 127) / 128) * ((m + 127) / 128); }
-static int tiles_256(int m, int n) { return ((n + 255) / 256) * ((m + 255) / 256); }
 
 // Up to 16 tokens: the LDS-tiled kernel once its 64-feature tiles (times slices) fill seven
 // eighths of the compute units, the 16-feature streaming kernel below that.
@@ -558,28 +556,56 @@ static bool half_rows_fill_better(int blocks16) {
 }
 
 // Kernel and number of K slices for more than 64 tokens, when the consumer takes up to
-// `max_slices` partial sums.  A larger tile needs less L2 traffic per flop and wins once there
-// are enough of them to keep the compute units busy; the largest one wants K long enough to pay
-// for its prologue, or many tiles.  A narrow output with a long K (the feed-forward's second
-// product) has too few large tiles: cut along K it fills the compute units with large tiles all
-// the same, as long as every slice stays long.
+// `max_slices` partial sums: the pair with the smallest estimated time.  The estimate counts
+// rounds of workgroups over the 256 compute units.  A workgroup of a tiling spends `fixed` us
+// outside its K loop and, per 64-wide step of K, `alone` us when it has its compute unit to itself
+// or `busy` us times the workgroups resident beside each other (operand fetch and matrix cores
+// do not overlap within a compute unit, so co-resident workgroups queue); steps are faster, down
+// to 63 % of that, while only a part of the compute units has work (less traffic into L2).
+// Partial sums cost their consumer, a norm that streams at 5.7 TB/s, 4 bytes per slice and
+// element instead of 2.  Constants fitted to the measured times of the four products of a layer
+// at five model sizes (hidden 896 to 5120) and 96 to 2,048 tokens: rms error of the estimate
+// 9 %, the chosen pair within 1 % of the best one on average and 12 % at worst, where rules on
+// tile counts had been 8 % and 76 % off.
 struct GemmPlan {
   int kernel, slices;
 };
-static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
-  const int big = tiles_256(m, n), mid = tiles_128(m, n);
-  // 129..170 of the largest tiles leave a third of the compute units idle in one pass; three
-  // slices of a very long K fill two passes (2048 x 5120 x 27648: 536 us against 693 us whole)
-  if (max_slices >= 3 && big > 128 && big * 3 <= 512 && k >= 3 * 4096) return {44, 3};
-  if (big >= 144 && (big >= 512 || k >= 2048)) return {44, 1};
-  if (max_slices >= 2 && big * 2 >= 192 && k >= 8192) return {44, 2};
-  if (mid >= 256) return {22, 1};
-  if (mid >= 64) {
-    int slices = 1;
-    while (slices < max_slices && slices < 4 && mid * slices < 256 && k / (2 * slices) >= 1024) slices *= 2;
-    if (slices > 1) return {22, slices};
+struct TilingCost {
+  int kernel, tile, resident;
+  float alone, busy, fixed;
+};
+constexpr TilingCost kTilingCosts[] = {
+    {11, 64, 8, 0.294f, 0.2156f, 6.3f}, {22, 128, 2, 0.765f, 0.569f, 6.4f}, {44, 256, 1, 1.035f, 1.779f, 10.9f}};
+constexpr int kComputeUnits = 256;
+static float tiled_time_us(const TilingCost& c, int m, int n, int k, int slices) {
+  const int64_t tiles = static_cast<int64_t>((m + c.tile - 1) / c.tile) * ((n + c.tile - 1) / c.tile);
+  const int64_t groups = tiles * slices;
+  const int ksteps = (k + kBK - 1) / kBK;
+  const float per = static_cast<float>((ksteps + slices - 1) / slices);
+  auto step = [&](int resident, float fill) {
+    return fmaxf(c.alone, resident * c.busy * (0.626f + 0.374f * fill));
+  };
+  const int64_t capacity = static_cast<int64_t>(kComputeUnits) * c.resident;
+  const int64_t full = groups / capacity, rest = groups % capacity;
+  float t = full * (c.fixed + per * step(c.resident, 1.f));
+  if (rest > 0) {
+    const int resident = static_cast<int>((rest + kComputeUnits - 1) / kComputeUnits);
+    t += c.fixed + per * step(resident, fminf(1.f, static_cast<float>(rest) / kComputeUnits));
   }
-  return {11, choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 4))};
+  return t;
+}
+static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
+  GemmPlan best{11, 1};
+  float best_time = 0.f;
+  const int ksteps = (k + kBK - 1) / kBK;
+  for (const TilingCost& c : kTilingCosts)
+    for (int slices = 1; slices <= min(max_slices, 4); ++slices) {
+      if (slices > 1 && ksteps / slices < 8) break;  // every slice keeps a few steps
+      float t = tiled_time_us(c, m, n, k, slices);
+      if (slices > 1) t += (4.f * slices - 2.f) * m * n / 5.7e6f;
+      if (best_time == 0.f || t < best_time) best = {c.kernel, slices}, best_time = t;
+    }
+  return best;
 }
 
 // The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,

@@ -175,7 +175,8 @@ def test_linear_swiglu_epilogue(ops_for, dtype, m, inter, k):
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 896, 4864), (8, 896, 896), (16, 130, 2056), (33, 517, 2056), (64, 896, 4864), (8, 151936, 96),
-     (300, 517, 4104), (2048, 896, 4864), (130, 130, 1032), (1000, 1030, 8200), (2040, 3000, 8192)],
+     (300, 517, 4104), (2048, 896, 4864), (130, 130, 1032), (1000, 1030, 8200), (2040, 3000, 8192),
+     (520, 1030, 9480), (96, 3584, 3584)],
 )
 def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     """A narrow product of a few tokens may come back as float32 partial sums over slices of k;
@@ -207,6 +208,22 @@ def test_linear_partial_sums_feed_the_norm(ops_for, m, n, k):
     rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
     picked = ops.gather_rows(got, rows).cpu()
     assert torch.equal(picked, got.cpu()[..., [m - 1, 0], :])
+
+
+def test_k_slices_chosen_for_many_tokens(ops_for):
+    """The estimate that picks a tiling and a number of k slices for more than 64 tokens: never more
+    slices than the consumer takes or than keep a few steps of k each, one slice for a wide
+    product that fills the compute units by itself, several for a narrow one with a long k."""
+    lib = ops_for(torch.bfloat16).lib
+    for m in (65, 96, 300, 1000, 2048, 16384):
+        for n, k in ((896, 896), (896, 4864), (3584, 18944), (37888, 3584), (130, 520), (5120, 27648)):
+            for most in (1, 2, 3, 8):
+                slices = lib.mlr_gemm_bf16_slices(m, n, k, most)
+                assert 1 <= slices <= min(most, 4)
+                assert slices == 1 or (k + 63) // 64 // slices >= 8
+    assert lib.mlr_gemm_bf16_slices(2048, 37888, 3584, 8) == 1
+    assert lib.mlr_gemm_bf16_slices(1024, 3584, 18944, 8) > 1
+    assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
 @pytest.mark.parametrize("kernel", [16, 14, 11, 22, 44])
