@@ -535,10 +535,10 @@ static int launch_tiled_qkv(const bf16* xb, const bf16* wb, GemmEpilogue ep, con
 
 // K slices for a skinny product: enough workgroups to keep every compute unit
 // streaming, as long as a slice keeps a few MFMA steps.  1 unless `allowed`.
-static int choose_slices(int groups, int ksteps, int allowed) {
+static int choose_slices(int groups, int ksteps, int allowed, int enough = 256) {
   if (allowed <= 1) return 1;
   int slices = 1;
-  while (slices < allowed && groups * slices < 256 && ksteps / (slices * 2) >= 8) slices *= 2;
+  while (slices < allowed && groups * slices < enough && ksteps / (slices * 2) >= 8) slices *= 2;
   return slices;
 }
 
@@ -663,8 +663,9 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
     const int by_fill = choose_slices((n + 15) / 16, (k / 8 + 3) / 4, max_slices);
     return max(by_fill, min(min(4, max_slices), k / 2560));
   }
-  // more slices fill the compute units, but the norm that adds them up reads them all
-  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 8));
+  // 17 to 64 tokens: the small tiles keep few bytes in flight each, so two workgroups per compute
+  // unit before the cutting stops (32B down at 32 tokens: 320 workgroups 65 us, 640 workgroups 56 us)
+  return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 8), 512);
 }
 
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
