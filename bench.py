@@ -222,6 +222,7 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
     portions = long_prompt // portion
     warmups = 2  # a shape of step is run plainly when it first comes and recorded when it comes again
     mixed = [[] for _ in range(portions)]
+    behind = []
     for r in range(warmups + repeats):
         engine.submit(f"long{r}", ids(long_prompt), max_new_tokens=1)
         for i in range(portions):
@@ -231,7 +232,10 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
             assert batch.token_count == portion + decoders
             if r >= warmups:
                 mixed[i].append(ms)
-        assert not timed_step()[0].plan.prompt_ids
+        result, ms = timed_step()
+        assert not result.plan.prompt_ids
+        if r >= warmups:
+            behind.append(ms)
     by_portion = [median(times) for times in mixed]
     ms = sum(by_portion) / portions
     return {
@@ -246,6 +250,7 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
         "decoders_tpot_ms_alone": round(alone, 3),
         "prompt_tokens_per_s": round(portion * 1e3 / ms, 1),
         "mixed_steps_ms_by_portion": [round(x, 3) for x in by_portion],
+        "decode_step_behind_the_prompt_ms": round(median(behind), 3),
         "config": dict(
             workload_config(args, config, full_layers),
             decoders=decoders,

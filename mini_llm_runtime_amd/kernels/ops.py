@@ -750,8 +750,9 @@ class HipOps:
             tiles, wide = plan.query_tiles, 0
             num_wide = int(getattr(plan, "num_wide_query_tiles", 0))
             enough = self.tuning.wide_attention_groups
-            if int(getattr(plan, "long_prefix", 0)):
-                enough //= 2  # heavy tiles everywhere: one workgroup per compute unit is enough
+            behind = int(getattr(plan, "long_prefix", 0))  # 1: thousands of keys before every tile, 2: twice that
+            if behind:
+                enough = enough * 3 // 4  # heavy tiles everywhere: fewer of them keep the compute units busy
             if (
                 num_wide * num_heads >= enough
                 and getattr(plan, "wide_query_tiles", None) is not None
@@ -763,8 +764,8 @@ class HipOps:
             # are cut into runs with a workgroup each, merged by a second kernel
             groups = num_tiles * num_heads
             key_runs = 1
-            if int(getattr(plan, "long_prefix", 0)) and groups < self.tuning.wide_attention_groups // 2:
-                key_runs = min(8, -(-self.tuning.wide_attention_groups // groups))
+            if behind == 2 and groups < self.tuning.key_run_groups:
+                key_runs = min(8, -(-self.tuning.key_run_groups // groups))
             partial = None
             if key_runs > 1:
                 partial = self._empty(

@@ -11,7 +11,7 @@ from ..parts.context import MixerPlan, PlanInput
 
 QUERY_TILE = 64  # queries of one request that the prompt kernel takes together
 WIDE_QUERY_TILE = 128  # and in its variant for long prompts (two blocks of queries per wavefront)
-LONG_PREFIX_KEYS = 4096  # mean number of keys before a tile from which a step counts as behind long prefixes
+LONG_PREFIX_KEYS = 2048  # mean number of keys before a tile from which a step counts as behind long prefixes (twice: very long)
 PAGED_ATTENTION = "paged_attention"  # the plan's key: every mixer on these kernels shares one plan per step
 
 
@@ -37,10 +37,12 @@ def attention_plan(shape: PlanInput) -> MixerPlan:
     decodes = int(single.sum())
     tiles = query_tiles(shape.q_lens, shape.q_starts)
     wide = query_tiles(shape.q_lens, shape.q_starts, WIDE_QUERY_TILE)
-    # portions behind long cached prefixes: every tile has thousands of keys before it, so even few
+    # portions behind long cached prefixes: every tile has thousands of keys before it, so fewer
     # tiles keep the compute units busy for long and the wide tiles' lower cost per key wins
+    # (level 1); behind twice as many (level 2) few tiles have their keys cut into runs
     keys_before = [int(shape.q_starts[e]) + int(q0) for e, q0 in wide]
-    long_prefix = int(bool(keys_before) and sum(keys_before) >= LONG_PREFIX_KEYS * len(keys_before))
+    mean_before = sum(keys_before) / len(keys_before) if keys_before else 0
+    long_prefix = int(mean_before >= LONG_PREFIX_KEYS) + int(mean_before >= 2 * LONG_PREFIX_KEYS)
     return MixerPlan(
         key=PAGED_ATTENTION,
         arrays={"query_tiles": tiles, "wide_query_tiles": wide},

@@ -19,10 +19,14 @@ class KernelTuning:
     fuse_bytes: int = 1 << 30
     # Prompt attention takes tiles of 128 queries instead of 64 once tiles x heads reach this many
     # workgroups (fewer leave compute units idle behind the heaviest tiles).
+    # Behind thousands of cached keys every tile is heavy and three quarters of that are enough.
     wide_attention_groups: int = 512
+    # Behind twice as many keys, fewer workgroups than this have the keys of every tile cut into
+    # runs (up to 8) with a workgroup each, until there are this many.
+    key_run_groups: int = 384
 
     def __post_init__(self) -> None:
-        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups"):
+        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups"):
             value = getattr(self, name)
             if isinstance(value, bool) or not isinstance(value, int) or value <= 0:
                 raise ValueError(f"KernelTuning.{name} must be a positive integer")

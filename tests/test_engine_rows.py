@@ -285,6 +285,8 @@ def test_attention_plan_covers_every_query_once_in_both_tile_sizes():
         assert weights == sorted(weights, reverse=True), "tiles with the most keys before them come first"
     assert plan.sizes["long_prefix"] == 0
     behind = attention_plan(PlanInput(np.array([512, 1], dtype=np.int32), np.array([6000, 9000], dtype=np.int32), 16384))
-    assert behind.sizes["long_prefix"] == 1, "a portion behind 6,000 cached tokens"
+    assert behind.sizes["long_prefix"] == 2, "a portion behind 6,000 cached tokens"
+    nearer = attention_plan(PlanInput(np.array([512], dtype=np.int32), np.array([3000], dtype=np.int32), 16384))
+    assert nearer.sizes["long_prefix"] == 1, "a portion behind 3,000 cached tokens"
     no_prompts = attention_plan(PlanInput(np.ones(3, dtype=np.int32), np.zeros(3, dtype=np.int32), 64))
     assert no_prompts.sizes["num_query_tiles"] == 0 and no_prompts.arrays["wide_query_tiles"].shape == (0, 2)

@@ -678,9 +678,10 @@ def test_prompt_portions_behind_long_contexts_in_key_runs(ops_for, heads, kv_hea
     a workgroup each, and merged; portions of 2 to 200 tokens, a whole short prompt beside them (its
     tiles have runs without keys), and a far key that carries the result."""
     ops = ops_for(torch.bfloat16) if not wide else _wide_ops()
+    assert ops.tuning.key_run_groups > 9 * heads  # more than the tiles of this case: they are cut
     entries = [(9000, 200), (12000, 2), (70, 70), (8200, 65)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 43, spike=True)
-    assert ctx.long_prefix == 1
+    assert ctx.long_prefix == 2
     scale = head_dim**-0.5
     got = ops.paged_attention(
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
