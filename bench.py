@@ -237,6 +237,11 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
         if r >= warmups:
             behind.append(ms)
     by_portion = [median(times) for times in mixed]
+    # The engine launches a decode step ahead whenever the next step is known to be one.  The step of
+    # the last portion therefore launches the decode step behind it before it returns, and that one
+    # launches another (which the next prompt's arrival then discards); the waits of this loop at
+    # the end of both steps cover a decode step each that is no part of the portion.
+    by_portion[-1] += median(behind) - 2 * alone
     ms = sum(by_portion) / portions
     return {
         "metric": "mixed step: 2,048 prompt tokens beside 32 decoding requests (mean over the prompt's portions)",
