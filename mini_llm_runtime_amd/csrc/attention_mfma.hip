@@ -61,6 +61,19 @@ __device__ __forceinline__ RowOperand load_row(const bf16* row, bool valid, int 
   return r;
 }
 
+// The same for rows that a step reads once (cached keys at decode): the non-temporal hint lets
+// them pass the caches by.
+__device__ __forceinline__ RowOperand load_row_once(const bf16* row, int quarter) {
+  RowOperand r;
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) {
+    const bool inside = !(kHalfLast && s == kSteps - 1 && quarter >= 2);
+    r.step[s] = inside ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(row + s * 32 + quarter * 8))
+                       : zero_bf16x8();
+  }
+  return r;
+}
+
 // S^T tile [16 keys x 16 rows].
 __device__ __forceinline__ f32x4_t score_tile(const RowOperand& k, const RowOperand& q) {
   f32x4_t s = {0.f, 0.f, 0.f, 0.f};
@@ -129,8 +142,8 @@ __device__ __forceinline__ DecodeTile load_decode_tile(const bf16* __restrict__ 
     t.bad = t.bad || (!here_a && key_a >= first && key_a < ke);
     const int page_a = here_a ? pages.key_page[half] : 0;
     const int off_a = min(key_a, ke - 1) % block_size;
-    t.k[half] = load_row(key_pages + ((static_cast<int64_t>(page_a) * kv_heads + kvh) * block_size + off_a) * D,
-                         true, quarter);
+    t.k[half] = load_row_once(key_pages + ((static_cast<int64_t>(page_a) * kv_heads + kvh) * block_size + off_a) * D,
+                              quarter);
     // value operand: this lane's 4 keys are ts + half * 16 + quarter * 4 .. + 3, inside one page
     const int key_v = ts + half * 16 + quarter * 4;
     const bool here_v = static_cast<unsigned>(pages.value_page[half]) < static_cast<unsigned>(num_pages);
@@ -139,7 +152,8 @@ __device__ __forceinline__ DecodeTile load_decode_tile(const bf16* __restrict__ 
     const bf16* vbase = value_pages + (static_cast<int64_t>(page_v) * kv_heads + kvh) * D * block_size + off_v;
 #pragma unroll
     for (int dt = 0; dt < kDimTiles; ++dt)
-      t.v[dt][half] = *reinterpret_cast<const u32x2_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size);
+      t.v[dt][half] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x2_t*>(vbase + static_cast<int64_t>(dt * 16 + col) * block_size));
   }
   return t;
 }

@@ -40,6 +40,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* p, uns
 __device__ __forceinline__ bf16x8_t buffer_load_bf16x8(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_offset) {
   return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0));
 }
+// The same with the non-temporal hint, for bytes that are read once (weights of a few-token product).
+__device__ __forceinline__ bf16x8_t buffer_load_bf16x8_once(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_offset) {
+  return __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 2));
+}
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
