@@ -411,6 +411,8 @@ class HipOps:
         if isinstance(x, PendingNorm):
             if x.value is not None or slices not in (None, 1) or m > self.FUSED_NORM_TOKENS:
                 return None
+            if n * k * 2 > self.tuning.fuse_weight_bytes:
+                return None
             # no K slices here: every workgroup needs whole rows for the norm's statistics
             residual, norm_args = self._norm_arguments(x)
             y = self._empty((m, n // 2 if swiglu else n), out_dtype)
@@ -420,7 +422,7 @@ class HipOps:
             )
             x.residual = residual
             return y
-        if swiglu or not self.tuning.fuse_merge:
+        if swiglu or not self.tuning.fuse_merge or n * k * 2 > self.tuning.fuse_weight_bytes:
             return None
         if slices is None:
             slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices) if partial_sums else 1
@@ -590,7 +592,8 @@ class HipOps:
         elif fused and not can_fuse:
             raise KernelError("the fused query/key/value kernel takes bfloat16 tokens and a full rotation")
         if pending is not None and not (
-            fused and not mfma_kernel and m <= self.FUSED_NORM_TOKENS and width * k * 2 < 1 << 32
+            fused and not mfma_kernel and m <= self.FUSED_NORM_TOKENS
+            and width * k * 2 <= min(self.tuning.fuse_weight_bytes, (1 << 32) - 1)
         ):
             x, pending = self.settle(pending), None
         if not fused:

@@ -17,6 +17,12 @@ class KernelTuning:
     # only some 15 GB/s whatever the source: beyond this many bytes of prologue input per workgroup
     # the kernel of its own is the faster way.
     fuse_bytes: int = 1 << 30
+    # The fused kernels stream weights in blocks of 16 rows, half as fast as the LDS-tiled kernel once a
+    # matrix has tens of megabytes: beyond this many bytes of weight the norm and the merge keep kernels
+    # of their own.  Decode steps at batch 1 with everything fused / with this limit: 1.5B (gate-up
+    # 55 MB) 1.66 / 1.50 ms, 3B (90 MB) 2.42 / 2.25 ms, 7B (query/key/value 33 MB, output 26 MB)
+    # 3.29 / 3.21 ms; the 17 MB gate-up of 0.5B stays fused (0.75 ms against 0.79).
+    fuse_weight_bytes: int = 20 << 20
     # Prompt attention takes tiles of 128 queries instead of 64 once tiles x heads reach this many
     # workgroups (fewer leave compute units idle behind the heaviest tiles).
     # Behind thousands of cached keys every tile is heavy and three quarters of that are enough.
@@ -26,7 +32,7 @@ class KernelTuning:
     key_run_groups: int = 384
 
     def __post_init__(self) -> None:
-        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups"):
+        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups", "fuse_weight_bytes"):
             value = getattr(self, name)
             if isinstance(value, bool) or not isinstance(value, int) or value <= 0:
                 raise ValueError(f"KernelTuning.{name} must be a positive integer")

@@ -151,6 +151,11 @@ def test_norm_prologue_is_refused_where_it_does_not_pay(ops, gpu_device):
     pending = ops.defer_norm(x.clone(), nw[:64], 1e-6, None)
     plainly = ops.linear(ops.rmsnorm(x.clone(), nw[:64], 1e-6), w, None, kernel="fma")
     assert torch.equal(ops.linear(pending, w, None, kernel="fma"), plainly) and pending.residual is not None
+    # a weight beyond the limit streams faster through the tiled kernel: the norm runs on its own
+    heavy = HipOps(torch.bfloat16, gpu_device, tuning=KernelTuning(fuse_weight_bytes=1000))
+    pending = heavy.defer_norm(x.clone(), nw[:64], 1e-6, None)
+    assert pending is not None
+    assert torch.equal(heavy.linear(pending, w, None), ops.linear(ops.rmsnorm(x.clone(), nw[:64], 1e-6), w, None))
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [(14, 2, 64), (4, 1, 32), (8, 2, 128), (6, 2, 48), (5, 1, 80), (3, 3, 16)])
