@@ -680,7 +680,9 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
     if (bytes >= (20ll << 20) && max_slices >= 8 && k >= 8 * 256 && few_tokens_tiled(n, 4) && !few_tokens_tiled(n, 2))
       return 8;
     if (bytes >= (20ll << 20) && max_slices >= 4 && k >= 4 * 256 && few_tokens_tiled(n, 4)) return 4;
-    const int by_fill = choose_slices((n + 15) / 16, (k / 8 + 3) / 4, max_slices);
+    // the 16-feature kernel: two workgroups per compute unit before the cutting stops (1.5B down at 8
+    // tokens: 384 workgroups 11.8 us, 768 workgroups 9.8 us), at most 8 slices for the norm to add up
+    const int by_fill = choose_slices((n + 15) / 16, (k / 8 + 3) / 4, min(max_slices, 8), 512);
     return max(by_fill, min(min(4, max_slices), k / 2560));
   }
   // 17 to 64 tokens: the small tiles keep few bytes in flight each, so two workgroups per compute
