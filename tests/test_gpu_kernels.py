@@ -226,7 +226,7 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 14, 11, 22, 44])
+@pytest.mark.parametrize("kernel", [16, 14, 12, 11, 22, 44])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
