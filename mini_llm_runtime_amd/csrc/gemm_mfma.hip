@@ -578,12 +578,12 @@ static bool half_rows_fill_better(int blocks16) {
 // outside its K loop and, per 64-wide step of K, `alone` us when it has its compute unit to itself
 // or `busy` us times the workgroups resident beside each other (operand fetch and matrix cores
 // do not overlap within a compute unit, so co-resident workgroups queue); steps are faster, down
-// to 63 % of that, while only a part of the compute units has work (less traffic into L2).
+// to 72 % of that, while only a part of the compute units has work (less traffic into L2).
 // Partial sums cost their consumer, a norm that streams at 5.7 TB/s, 4 bytes per slice and
 // element instead of 2.  Constants fitted to the measured times of the four products of a layer
-// at five model sizes (hidden 896 to 5120) and 96 to 2,048 tokens: rms error of the estimate
-// 9 %, the chosen pair within 1 % of the best one on average and 12 % at worst, where rules on
-// tile counts had been 8 % and 76 % off.
+// at five model sizes (hidden 896 to 5120) and 96 to 2,048 tokens, with weights that rotate
+// through more memory than the caches hold: rms error of the estimate 8 %, the chosen pair within
+// 1 % of the best one on average, where rules on tile counts had been 8 % off and up to 76 %.
 struct GemmPlan {
   int kernel, slices;
 };
@@ -592,7 +592,7 @@ struct TilingCost {
   float alone, busy, fixed;
 };
 constexpr TilingCost kTilingCosts[] = {
-    {11, 64, 8, 0.294f, 0.2156f, 6.3f}, {22, 128, 2, 0.765f, 0.569f, 6.4f}, {44, 256, 1, 1.035f, 1.779f, 10.9f}};
+    {11, 64, 8, 0.401f, 0.251f, 6.4f}, {22, 128, 2, 0.966f, 0.603f, 6.5f}, {44, 256, 1, 1.15f, 1.937f, 10.5f}};
 constexpr int kComputeUnits = 256;
 static float tiled_time_us(const TilingCost& c, int m, int n, int k, int slices) {
   const int64_t tiles = static_cast<int64_t>((m + c.tile - 1) / c.tile) * ((n + c.tile - 1) / c.tile);
@@ -600,7 +600,7 @@ static float tiled_time_us(const TilingCost& c, int m, int n, int k, int slices)
   const int ksteps = (k + kBK - 1) / kBK;
   const float per = static_cast<float>((ksteps + slices - 1) / slices);
   auto step = [&](int resident, float fill) {
-    return fmaxf(c.alone, resident * c.busy * (0.626f + 0.374f * fill));
+    return fmaxf(c.alone, resident * c.busy * (0.724f + 0.276f * fill));
   };
   const int64_t capacity = static_cast<int64_t>(kComputeUnits) * c.resident;
   const int64_t full = groups / capacity, rest = groups % capacity;
