@@ -534,7 +534,7 @@ class HipOps:
         that rotates the sums and stores them where they belong (a row-splitting kernel for up
         to 64 tokens, a tiled one beyond) unless the product is large; everything else is the
         product followed by `rope_kv_write`.  Up to 64 tokens of a wide product (tens of
-        megabytes of weights) go a third way: the product cut
+        megabytes of weights), and 65 to 128 tokens from 8 MB on, go a third way: the product cut
         along k through the LDS-tiled kernel, which streams such weights twice as fast as the
         row-splitting one, and a small kernel that adds the slices up, rotates and stores.
         `fused` and `sliced` force a way, `mfma_kernel` the fused kernel (tests).
@@ -561,10 +561,19 @@ class HipOps:
                 or (weight_bytes >= 8 << 20 and m > 32)
             )
             sliced = fused is None and can_fuse and pending is None and not mfma_kernel and m <= 64 and pays and k >= 512
-        elif sliced and not (can_fuse and pending is None and m <= 64 and k >= 512):
-            raise KernelError("the sliced query/key/value product takes up to 64 bfloat16 tokens and a full rotation")
+            # 65 to 128 tokens: the fused tiled kernel reads the weights once per 64 tokens; cut along K
+            # where the estimate of the plain product says so, the product and the finishing kernel
+            # are 1.2 to 1.5 times faster from 8 MB of weights on (7B at 96 tokens: 33 us against 24)
+            if (
+                not sliced and fused is None and can_fuse and pending is None and not mfma_kernel
+                and 64 < m <= 128 and weight_bytes >= 8 << 20
+            ):
+                mid_slices = self.lib.mlr_gemm_bf16_slices(m, width, k, 4)
+                sliced = mid_slices > 1
+        elif sliced and not (can_fuse and pending is None and m <= 128 and k >= 512):
+            raise KernelError("the sliced query/key/value product takes up to 128 bfloat16 tokens and a full rotation")
         if sliced:
-            slices = 8 if k >= 2048 else 4
+            slices = (8 if k >= 2048 else 4) if m <= 64 else max(2, self.lib.mlr_gemm_bf16_slices(m, width, k, 4))
             partial = self.linear(x, weight, bias, partial_sums=True, slices=slices)
             cos = sin = None
             if rotation is not None:

@@ -370,7 +370,7 @@ def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads,
 @pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,tokens,rotate,write", [
     (14, 2, 64, 896, 64, True, True), (14, 2, 64, 896, 33, True, True), (3, 1, 16, 520, 1, True, True),
     (5, 1, 128, 1208, 8, True, True), (4, 4, 80, 640, 17, False, True), (6, 3, 48, 2056, 5, True, False),
-    (28, 4, 128, 3584, 8, True, True),
+    (28, 4, 128, 3584, 8, True, True), (28, 4, 128, 3584, 100, True, True), (6, 2, 64, 1032, 128, True, True),
 ])
 def test_sliced_qkv_product_equals_the_three_kernels(ops_for, heads, kv_heads, head_dim, hidden, tokens, rotate, write):
     """The third way of the query/key/value product (cut along k through the tiled kernel, then one
