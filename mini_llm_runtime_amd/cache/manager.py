@@ -113,6 +113,9 @@ class RequestCache:
     has_reservation: bool = False
     state_parity: int = 0
     pending_tokens: int = 0
+    # `tables` as int32 arrays, per group (array, entries that are valid, `table_stamp` they were made at)
+    table_arrays: dict = field(default_factory=dict, repr=False, compare=False)
+    table_stamp: int = 0  # counts changes of `tables` other than appended pages
 
     def live_blocks(self, group: int) -> list[int]:
         return [b for b in self.tables[group] if b >= 0]
@@ -121,28 +124,27 @@ class RequestCache:
         """`tables[group]` as int32; kept between steps and only extended when pages were
         appended, rebuilt when the table changed in any other way."""
         table = self.tables[group]
-        cache = self.__dict__.setdefault("_table_arrays", {})
-        kept = cache.get(group)
+        kept = self.table_arrays.get(group)
         n = len(table)
         if kept is not None:
             array, length, stamp = kept
-            if stamp == self.__dict__.get("_table_stamp", 0) and length <= n:
+            if stamp == self.table_stamp and length <= n:
                 if length < n:
                     if n > array.shape[0]:
                         grown = np.empty(max(n, 2 * array.shape[0]), dtype=np.int32)
                         grown[:length] = array[:length]
                         array = grown
                     array[length:n] = table[length:]
-                    cache[group] = (array, n, stamp)
+                    self.table_arrays[group] = (array, n, stamp)
                 return array[:n]
         array = np.empty(max(16, 2 * n), dtype=np.int32)
         array[:n] = table
-        cache[group] = (array, n, self.__dict__.get("_table_stamp", 0))
+        self.table_arrays[group] = (array, n, self.table_stamp)
         return array[:n]
 
     def tables_changed(self) -> None:
         """Entries of `tables` were overwritten or removed (not just appended)."""
-        self.__dict__["_table_stamp"] = self.__dict__.get("_table_stamp", 0) + 1
+        self.table_stamp += 1
 
 
 @dataclass

@@ -5,12 +5,14 @@
     python -m mini_llm_runtime_amd.cli random-model --config qwen2.5-0.5b --seed 0 --out DIR
 
 `generate` follows the reference's `experiments/greedy_generation_runner.py:19-25`
-(`--model`, `--prompt`, `--max-new-tokens`, `--local-files-only`); `engine` follows
-its `experiments/continuous_batch_engine_runner.py:32-52` (`--model`, `--block-size`,
-`--local-files-only`, `--output-dir`) and runs the same kind of demonstration:
-requests that join and leave a running batch, with a record of every step.  The
-reference's `--prefill-attention-backend` and `--prefill-kv-write-backend` choose
-between its PyTorch code paths; this engine has one kernel path and no such options.
+(`--model`, `--prompt`, `--max-new-tokens`); `engine` follows its
+`experiments/continuous_batch_engine_runner.py:32-52` (`--model`, `--block-size`,
+`--output-dir`) and runs the same kind of demonstration: requests that join and leave a
+running batch, with a record of every step.  Options of the reference without a
+counterpart: `--local-files-only` (its `--model` may name a hub repository to download;
+`--model` here is a folder and nothing is ever fetched, so there is nothing to switch off)
+and `--prefill-attention-backend` / `--prefill-kv-write-backend` (they choose between its
+PyTorch code paths; this engine has one kernel path).
 `--dtype` defaults to what the model folder's config.json says (`torch_dtype`); the page
 pool is `--num-blocks` pages or, without it, `--kv-memory-fraction` of the free device memory.
 
@@ -33,7 +35,6 @@ from typing import Any, Optional, Sequence
 def _add_model_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--model", required=True, type=Path, help="folder with config.json and model.safetensors")
     p.add_argument("--dtype", default=None, choices=("bfloat16", "float32"), help="default: config.json's torch_dtype")
-    p.add_argument("--local-files-only", action="store_true", help="accepted for compatibility; models are always local")
 
 
 def _ids(text: str) -> list[int]:

@@ -242,6 +242,15 @@ int mlr_sample_static(const float* logits, const float* temperature, const float
     set_error(std::string("mlr_sample_static: no usable current device: ") + hipGetErrorString(e));
     return -1;
   }
+  // The array whose address is used below is the current device's: a stream of another GPU would
+  // run the kernels there with this GPU's address.
+  hipDevice_t stream_device = -1;
+  if (hipStreamGetDevice(stream, &stream_device) == hipSuccess && stream_device != device) {
+    set_error("mlr_sample_static: the stream belongs to device " + std::to_string(stream_device) +
+              ", the current device is " + std::to_string(device) + "; make the stream's device current first");
+    return -1;
+  }
+  (void)hipGetLastError();  // a runtime without that query leaves an error behind: not this call's business
   float* scratch_ptr = nullptr;
   {
     std::lock_guard<std::mutex> lock(guard);

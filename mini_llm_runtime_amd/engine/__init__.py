@@ -2,7 +2,7 @@
 
 from .admission import PageAdmission, PagePromise
 from .config import EngineConfig, GraphLimits
-from .engine import ContinuousBatchEngine, EngineStepResult
+from .engine import ContinuousBatchEngine, EngineBrokenError, EngineStepResult
 from .factory import load_model, make_cache, parse_dtype
 from .generation import GenerationOutput, generate, greedy_generate
 from .metrics import RequestTimes, summarize
@@ -14,6 +14,7 @@ __all__ = [
     "BatchingPolicy",
     "ContinuousBatchEngine",
     "EndReason",
+    "EngineBrokenError",
     "EngineConfig",
     "EngineStepResult",
     "GenerationOutput",

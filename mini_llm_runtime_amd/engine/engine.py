@@ -58,16 +58,16 @@ class _ChosenTokens:
     right behind the sampling, BEFORE any later step is launched, and has an event of its own:
     waiting for it does not wait for what was launched after it."""
 
-    _spare: list = []  # pinned landing buffers not in use (making one costs a system call)
-
-    def __init__(self, on_device: torch.Tensor) -> None:
+    def __init__(self, on_device: torch.Tensor, spare: list) -> None:
+        """spare: the engine's pinned landing buffers that are not in use (making one costs a
+        system call); this object takes one and puts it back in `wait`."""
         self.on_device = on_device
         self._event = self._buffer = None
+        self._spare = spare
         if on_device.device.type != "cuda":
             self._host = on_device
             return
         count = on_device.numel()
-        spare = _ChosenTokens._spare
         self._buffer = spare.pop() if spare and spare[-1].numel() >= count else torch.empty(
             max(256, count), dtype=on_device.dtype, pin_memory=True
         )
@@ -80,10 +80,15 @@ class _ChosenTokens:
         if self._event is not None:
             self._event.synchronize()
         tokens = self._host.tolist()
-        if self._buffer is not None and len(_ChosenTokens._spare) < 8:
-            _ChosenTokens._spare.append(self._buffer)
+        if self._buffer is not None and len(self._spare) < 8:
+            self._spare.append(self._buffer)
         self._buffer = None
         return tokens
+
+
+class EngineBrokenError(RuntimeError):
+    """A step failed after the cache had counted its tokens (while tokens were chosen or copied):
+    scheduler and cache no longer agree, and no further step may run."""
 
 
 @dataclass
@@ -136,6 +141,8 @@ class ContinuousBatchEngine:
         self.lookahead_hits = 0
         self.lookahead_misses = 0
         self.lookahead_error: Optional[Exception] = None  # what switched the lookahead off, if anything did
+        self.broken: Optional[BaseException] = None  # what failed after a step's tokens had been counted
+        self._landing: list = []  # pinned buffers for chosen tokens that are not in use
         self.config: Optional[EngineConfig] = None  # set by from_model_dir
 
     @property
@@ -156,7 +163,7 @@ class ContinuousBatchEngine:
         single fields of it).  `ops` replaces the HIP kernel library (tests on the CPU)."""
         from ..config.model_config import read_config_json
         from ..models.registry import load_config
-        from .factory import blocks_from_free_memory, default_ops, load_model, make_cache
+        from .factory import blocks_from_free_memory, default_ops, load_model, make_cache, recording_reserve_bytes
 
         config = (config or EngineConfig()).with_overrides(**overrides)
         dtype = ops.dtype if ops is not None and config.dtype is None else config.resolved_dtype(read_config_json(model_dir))
@@ -165,8 +172,11 @@ class ContinuousBatchEngine:
         _, model = load_model(model_dir, dtype=dtype, device=ops.device)
         num_blocks = config.num_blocks
         if num_blocks is None:
+            reserve = recording_reserve_bytes(
+                model, config.graphs, dtype, config.max_running_requests, config.max_batch_tokens
+            )
             num_blocks = blocks_from_free_memory(
-                model, config.block_size, dtype, torch.device(ops.device), config.kv_memory_fraction
+                model, config.block_size, dtype, torch.device(ops.device), config.kv_memory_fraction, reserve
             )
         cache = make_cache(
             model,
@@ -254,6 +264,11 @@ class ContinuousBatchEngine:
     @torch.inference_mode()
     def step(self) -> Optional[EngineStepResult]:
         """Plan and run one step; None when nothing can run."""
+        if self.broken is not None:
+            raise EngineBrokenError(
+                f"an earlier step failed after the cache had counted its tokens ({type(self.broken).__name__}: "
+                f"{self.broken}); the engine cannot go on"
+            )
         started = self._clock_ns()
         try:
             with _traced(self.enable_tracing, "scheduler.schedule_step"):
@@ -268,6 +283,8 @@ class ContinuousBatchEngine:
         with _traced(self.enable_tracing, label):
             try:
                 flight = self._fly(plan)
+            except EngineBrokenError:
+                raise
             except BaseException:  # an interrupt, too, must not leave admitted requests and a plan behind
                 self._abandon_ahead()
                 with _traced(self.enable_tracing, "engine.rollback"):
@@ -310,12 +327,34 @@ class ContinuousBatchEngine:
                 ahead.output = self.runner.commit(ahead.output)
                 return ahead
             self._abandon_ahead()
+        self._check_offsets(plan)
         with _traced(self.enable_tracing, f"model.step:tokens={plan.token_count}"):
             output = self.runner.step(plan.entries, borrow_logits=True)  # sampled from right below
-        chosen = None
-        if output.logits is not None:
-            chosen = _ChosenTokens(self.sampler.sample(output.logits, *self._sampling_of(plan)))
+        # From here on the cache counts the step's tokens: a failure can no longer be undone by
+        # cancelling the plan (the same tokens would be fed again behind themselves).
+        try:
+            chosen = None
+            if output.logits is not None:
+                chosen = _ChosenTokens(self.sampler.sample(output.logits, *self._sampling_of(plan)), self._landing)
+        except BaseException as error:
+            self.broken = error
+            self._abandon_ahead()
+            raise EngineBrokenError(
+                f"choosing the tokens of step {plan.index} failed after the cache had counted them: "
+                f"{type(error).__name__}: {error}"
+            ) from error
         return _Flight(tuple(rid for rid, _ in output.rows), output, chosen)
+
+    def _check_offsets(self, plan: StepPlan) -> None:
+        """Every slice goes on exactly where its request's cache ends: the scheduler's count of
+        consumed tokens and the cache manager's count of cached ones must agree."""
+        for part in plan.slices:
+            cached = self.manager.get_request(part.request_id).num_tokens
+            if cached != part.offset:
+                raise RuntimeError(
+                    f"request {part.request_id!r}: the plan feeds tokens behind {part.offset} cached ones, "
+                    f"the cache holds {cached}"
+                )
 
     # ---- the step launched ahead ------------------------------------------------------------------
     def _look_ahead(self, plan: StepPlan, flight: _Flight) -> None:
@@ -360,7 +399,8 @@ class ContinuousBatchEngine:
         try:
             requests = [scheduler.request(rid) for rid in going_on]
             chosen = _ChosenTokens(
-                self.sampler.sample(launched.logits, [r.sampling for r in requests], [len(r.output) + 1 for r in requests])
+                self.sampler.sample(launched.logits, [r.sampling for r in requests], [len(r.output) + 1 for r in requests]),
+                self._landing,
             )
         except BaseException:
             self.runner.abort(launched)

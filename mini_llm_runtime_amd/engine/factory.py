@@ -72,14 +72,54 @@ def page_bytes(model: DecoderModel, block_size: int, dtype: torch.dtype) -> int:
     return total
 
 
-def blocks_from_free_memory(
-    model: DecoderModel, block_size: int, dtype: torch.dtype, device: torch.device, fraction: float
+def recording_reserve_bytes(
+    model: DecoderModel, limits: Any, dtype: torch.dtype, max_running_requests: int, max_batch_tokens: int
 ) -> int:
-    """Pages per pool that `fraction` of the device memory free right now holds."""
+    """An upper estimate of what the step function's recorded steps hold beside the weights and the
+    page pool: every recording owns its activations (per token about twice the output widths of one
+    layer's matrices, for tensors that live side by side, plus two float32 copies of the stream) and a
+    float32 logits buffer [wanted rows, vocab].  Single-token recordings exist per (batch padded to a
+    power of two, block table width), other steps per shape; `limits` (a `GraphLimits`) bounds both."""
+    if limits is None or not limits.enabled:
+        return 0
+    width = torch.empty((), dtype=dtype).element_size()
+    spec = model.spec
+    layer_widths = 0
+    for name, p in model.param_specs().items():
+        if name.startswith("layers.0.") and len(p.shape) == 2:
+            layer_widths += int(p.shape[0])
+    per_token = 2 * layer_widths * width + 8 * spec.hidden_size
+    logits_row = spec.vocab_size * 4
+    largest = 1
+    while largest < min(max_running_requests, limits.max_decode_batch):
+        largest *= 2
+    batches = []
+    b = 1
+    while b <= largest:
+        batches.append(b)
+        b *= 2
+    widths_each = -(-limits.max_decode_graphs // len(batches))
+    decode = sum(b * (per_token + logits_row) for b in batches) * widths_each
+    step_tokens = min(limits.max_step_tokens, max_batch_tokens)
+    steps = limits.max_step_graphs * (step_tokens * per_token + max_running_requests * logits_row)
+    return decode + steps
+
+
+def blocks_from_free_memory(
+    model: DecoderModel,
+    block_size: int,
+    dtype: torch.dtype,
+    device: torch.device,
+    fraction: float,
+    reserve_bytes: int = 0,
+) -> int:
+    """Pages per pool that `fraction` of the device memory free right now holds, after
+    `reserve_bytes` were set aside (for recorded steps: at most half of what is free)."""
     per_page = page_bytes(model, block_size, dtype)
     if per_page == 0:
         return 1  # a model without paged sites still gets a (never used) pool
     if device.type != "cuda":
         raise ValueError("kv_memory_fraction needs a GPU; give num_blocks instead")
     free, _ = torch.cuda.mem_get_info(device)
+    free -= min(int(reserve_bytes), free // 2)
     return blocks_for_memory(per_page, free, fraction)

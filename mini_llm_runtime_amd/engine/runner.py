@@ -14,6 +14,7 @@ qwen_model_runner.py:371-375, 495-503), result rows in the order of the batch
 
 from __future__ import annotations
 
+import warnings
 from dataclasses import dataclass, field
 from types import SimpleNamespace
 from typing import Any, Optional, Sequence
@@ -319,6 +320,25 @@ class ModelRunner:
     def _recordable(self) -> bool:
         return self.use_graphs and self._replayable
 
+    def _recording_ran_out_of_memory(self, error: BaseException) -> None:
+        """A recording (its private activations and logits buffer) did not fit beside the weights
+        and the page pool: every recording is dropped, which frees their memory, and steps run
+        unrecorded from here on."""
+        self.use_graphs = False
+        self._graphs.clear()
+        self._step_graphs.clear()
+        self._staging.clear()
+        self._step_seen.clear()
+        if self.device.type == "cuda":
+            torch.cuda.empty_cache()
+        warnings.warn(
+            f"recording a step as a HIP graph ran out of device memory ({error}); recordings are switched off "
+            "and every step launches its kernels one by one, which is slower.  Give the page pool less memory "
+            "(num_blocks, kv_memory_fraction) or lower the GraphLimits.",
+            RuntimeWarning,
+            stacklevel=3,
+        )
+
     def _step_key(self, layout: StepLayout, logit_rows: np.ndarray) -> Optional[tuple]:
         """(identity of a recording, the plans it was derived from): the sizes that fix every launch
         of a step; None when such steps are not recorded."""
@@ -582,8 +602,12 @@ class ModelRunner:
             borrowed = False
             key = None if capture_sites else self._graph_key(layout)
             if key is not None:
-                logits = self._forward_graph(key, layout, token_ids, logit_rows)
-                borrowed = True
+                try:
+                    logits = self._forward_graph(key, layout, token_ids, logit_rows)
+                    borrowed = True
+                except torch.cuda.OutOfMemoryError as error:
+                    self._recording_ran_out_of_memory(error)
+                    logits = self._forward_eager(layout, token_ids, logit_rows)
             elif capture_sites:
                 logits = self._forward_eager(layout, token_ids, logit_rows, captured)
             else:
@@ -594,8 +618,12 @@ class ModelRunner:
                     if len(self._step_seen) > 4096:
                         self._step_seen.clear()
                 if seen >= 2:
-                    logits = self._forward_recorded(keyed[0], keyed[1], layout, token_ids, logit_rows)
-                    borrowed = True
+                    try:
+                        logits = self._forward_recorded(keyed[0], keyed[1], layout, token_ids, logit_rows)
+                        borrowed = True
+                    except torch.cuda.OutOfMemoryError as error:
+                        self._recording_ran_out_of_memory(error)
+                        logits = self._forward_eager(layout, token_ids, logit_rows)
                 else:
                     logits = self._forward_eager(layout, token_ids, logit_rows)
             if borrowed and not borrow_logits and logits is not None:

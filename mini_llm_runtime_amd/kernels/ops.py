@@ -411,7 +411,7 @@ class HipOps:
         if isinstance(x, PendingNorm):
             if x.value is not None or slices not in (None, 1) or m > self.FUSED_NORM_TOKENS:
                 return None
-            if n * k * 2 > self.tuning.fuse_weight_bytes:
+            if n * k * 2 > min(self.tuning.fuse_weight_bytes, (1 << 32) - 1):  # 32-bit offsets into the weights
                 return None
             # no K slices here: every workgroup needs whole rows for the norm's statistics
             residual, norm_args = self._norm_arguments(x)
@@ -422,7 +422,7 @@ class HipOps:
             )
             x.residual = residual
             return y
-        if swiglu or not self.tuning.fuse_merge or n * k * 2 > self.tuning.fuse_weight_bytes:
+        if swiglu or not self.tuning.fuse_merge or n * k * 2 > min(self.tuning.fuse_weight_bytes, (1 << 32) - 1):
             return None
         if slices is None:
             slices = self.lib.mlr_gemm_bf16_slices(m, n, k, self.max_k_slices) if partial_sums else 1

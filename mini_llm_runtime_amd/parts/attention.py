@@ -8,6 +8,7 @@ from typing import Optional
 import torch
 
 from ..cache.spec import PagedKVSpec
+from ..kernels.limits import check_attention_sizes
 from .base import Mixer, Part, PositionEncoding
 from .context import MixerPlan, PlanInput, StepContext
 from .registry import build_part, register_part
@@ -52,6 +53,7 @@ class GQAAttention(Mixer):
             raise ValueError("num_heads must be a positive multiple of num_kv_heads")
         if head_dim <= 0:
             raise ValueError("head_dim must be > 0")
+        check_attention_sizes(num_heads, num_kv_heads, head_dim)  # refused here, not at the first step
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)

@@ -32,7 +32,6 @@ from typing import Any, Optional, Sequence, TextIO
 
 
 PAGE_TOKENS = 16  # default tokens per page of the replay pool
-ROUNDING = 64  # the caller counts every request's tokens rounded up to this (or to a larger page)
 MAX_LIVE = 8  # default number of request slots
 
 

@@ -20,8 +20,10 @@ ROOT = Path(__file__).resolve().parents[1]
 
 def test_option_names_follow_the_reference():
     p = cli.build_parser()
-    g = p.parse_args(["generate", "--model", "m", "--prompt-ids", "1,2 3", "--max-new-tokens", "4", "--local-files-only"])
-    assert g.prompt_ids == [1, 2, 3] and g.max_new_tokens == 4 and g.temperature == 0.0 and g.local_files_only
+    g = p.parse_args(["generate", "--model", "m", "--prompt-ids", "1,2 3", "--max-new-tokens", "4"])
+    assert g.prompt_ids == [1, 2, 3] and g.max_new_tokens == 4 and g.temperature == 0.0
+    with pytest.raises(SystemExit):  # nothing is ever downloaded: no option that would switch that off
+        p.parse_args(["generate", "--model", "m", "--prompt-ids", "1", "--local-files-only"])
     assert p.parse_args(["generate", "--model", "m", "--prompt", "hi"]).max_new_tokens == 8  # the reference's default
     e = p.parse_args(["engine", "--model", "m", "--block-size", "4", "--output-dir", "out"])
     assert e.block_size == 4 and e.output_dir == Path("out") and e.batching_policy == "continuous"

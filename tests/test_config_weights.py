@@ -66,6 +66,16 @@ def test_model_spec_takes_every_size_from_the_config():
     assert len(model.site_cache_specs()) == 3
 
 
+def test_a_head_size_no_kernel_runs_is_refused_when_the_model_is_built():
+    """Sizes that only slower kernels take build fine (a head size of 20, of 264 would not);
+    a head size beyond what any attention kernel keeps in registers is refused at once."""
+    ok = Qwen2Config.from_dict({**TINY_A, "head_dim": 256})
+    assert build_model(ok).layers[0].mixer.head_dim == 256
+    too_wide = Qwen2Config.from_dict({**TINY_A, "head_dim": 272})
+    with pytest.raises(ValueError, match="head_dim 272.*up to 256"):
+        build_model(too_wide)
+
+
 def test_random_model_is_seeded_and_loads(tmp_path):
     d1 = make_model_dir(tmp_path / "x", "A", seed=5)
     d2 = make_model_dir(tmp_path / "y", "A", seed=5)

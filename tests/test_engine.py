@@ -217,6 +217,46 @@ def test_failed_step_rolls_back_and_can_be_retried(tmp_path, backend, dtype):
     _check_greedy(engine.request("C").generated, pc, w, cfg, dtype)
 
 
+def test_a_failure_after_the_cache_counted_the_step_stops_the_engine(tmp_path):
+    """When choosing the tokens fails, the step's tokens are already cached: cancelling the plan
+    would feed them again behind themselves.  The engine refuses to go on instead, and leaves
+    the scheduler's plan outstanding rather than rolled back."""
+    from mini_llm_runtime_amd.engine.engine import EngineBrokenError
+
+    d = make_model_dir(tmp_path, "A", seed=26)
+    cfg, _ = read_weights(d)
+    engine = _engine(d, _ops("double", torch.float32), block_size=4, num_blocks=32, max_running=3)
+    engine.submit("A", random_tokens(7, cfg["vocab_size"], 1), max_new_tokens=4)
+    engine.step()
+    cached = engine.manager.get_request("A").num_tokens
+
+    def broken_sampler(*args, **kwargs):
+        raise RuntimeError("no tokens today")
+
+    engine.sampler.sample = broken_sampler
+    with pytest.raises(EngineBrokenError, match="no tokens today"):
+        engine.step()
+    assert engine.manager.get_request("A").num_tokens == cached + 1  # the step counted
+    assert engine.scheduler.active_ids == ("A",)  # and nothing was rolled back behind it
+    with pytest.raises(EngineBrokenError, match="cannot go on"):
+        engine.step()
+
+
+def test_a_plan_that_disagrees_with_the_cache_is_refused(tmp_path):
+    """Every slice must go on where its request's cache ends."""
+    d = make_model_dir(tmp_path, "A", seed=27)
+    cfg, _ = read_weights(d)
+    engine = _engine(d, _ops("double", torch.float32), block_size=4, num_blocks=32, max_running=3, lookahead=False)
+    engine.submit("A", random_tokens(9, cfg["vocab_size"], 1), max_new_tokens=4)
+    engine.step()
+    # a step behind the scheduler's back: the cache is now one token ahead of the plan to come
+    engine.runner.step([mlr.StepEntry.of("A", [1])])
+    with pytest.raises(RuntimeError, match="the cache holds"):
+        engine.step()
+    # the refused step was rolled back like any failed one
+    assert engine.scheduler.active_ids == ("A",) and not engine.manager.step_in_flight
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_decoding_one_step_ahead_changes_nothing_but_the_waiting(tmp_path, dtype):

@@ -98,6 +98,49 @@ def test_page_pool_from_free_memory_and_dtype_from_the_folder(tmp_path, gpu_devi
     assert engine.generate([prompt], max_new_tokens=4)[0] == plain.greedy(prompt, w, cfg, 4)
 
 
+def test_memory_set_aside_for_recorded_steps(tmp_path):
+    """The page pool is sized from what is free after the weights less an estimate of what
+    recorded steps will hold: nothing without recordings, more with more or larger ones."""
+    from mini_llm_runtime_amd.engine.factory import recording_reserve_bytes
+
+    d = make_model_dir(tmp_path, "A", seed=64)
+    cfg, _ = read_weights(d)
+    _, model = mlr.load_model(d, dtype=torch.float32, device="cpu")
+    base = recording_reserve_bytes(model, GraphLimits(), torch.bfloat16, 8, 2048)
+    assert recording_reserve_bytes(model, GraphLimits(enabled=False), torch.bfloat16, 8, 2048) == 0
+    assert recording_reserve_bytes(model, None, torch.bfloat16, 8, 2048) == 0
+    # at least the logits of one recording per padded batch size 1, 2, 4, 8
+    assert base >= (1 + 2 + 4 + 8) * cfg["vocab_size"] * 4
+    assert recording_reserve_bytes(model, GraphLimits(max_step_graphs=32), torch.bfloat16, 8, 2048) > base
+    assert recording_reserve_bytes(model, GraphLimits(), torch.bfloat16, 64, 2048) > base
+    assert recording_reserve_bytes(model, GraphLimits(), torch.bfloat16, 8, 8192) > base
+    assert recording_reserve_bytes(model, GraphLimits(), torch.float32, 8, 2048) > base
+
+
+@pytest.mark.gpu
+def test_a_recording_that_runs_out_of_memory_falls_back_to_plain_steps(tmp_path, gpu_device, monkeypatch):
+    """The condition is forced from the host (the graph object refuses to be made); the step must
+    still give the right logits, recordings must be off afterwards, and one warning says so."""
+    d = make_model_dir(tmp_path, "A", seed=65)
+    cfg, w = read_weights(d)
+    _, _, _, runner = make_runner(d, _ops("hip", torch.float32), block_size=BLOCK_SIZE["A"], num_blocks=16)
+    tokens = random_tokens(9, cfg["vocab_size"], 4)
+    ref = plain.forward(tokens, w, cfg)
+    runner.cache.create_request("r")
+    runner.step([StepEntry.of("r", tokens[:8], [7])])
+    assert runner.use_graphs
+
+    def no_memory(*args, **kwargs):
+        raise torch.cuda.OutOfMemoryError("forced by the test")
+
+    monkeypatch.setattr(torch.cuda, "CUDAGraph", no_memory)
+    with pytest.warns(RuntimeWarning, match="recordings are switched off"):
+        out = runner.step([StepEntry.of("r", tokens[8:], [0])])  # a single token: would be recorded
+    assert not runner.use_graphs and not runner._graphs
+    torch.testing.assert_close(out.logits[0].double().cpu(), ref[8], atol=1e-4, rtol=1e-4)
+    assert runner.cache.get_request("r").num_tokens == 9 and not runner.cache.step_in_flight
+
+
 # ---- the residual stream after every site -------------------------------------------------------------------
 @pytest.mark.parametrize("backend,dtype", CASES)
 @pytest.mark.parametrize("which", ["A", "B"])
