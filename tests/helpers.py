@@ -8,6 +8,7 @@ from pathlib import Path
 import torch
 
 from mini_llm_runtime_amd.config import Qwen2Config
+from mini_llm_runtime_amd.config.presets import load_preset
 from mini_llm_runtime_amd.engine.factory import load_model, make_cache
 from mini_llm_runtime_amd.engine.runner import ModelRunner, StepEntry
 from mini_llm_runtime_amd.weights import SafetensorsFile, write_random_model
@@ -79,8 +80,11 @@ TINY_D = dict(
     hidden_act="silu",
     tie_word_embeddings=False,
 )
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-BLOCK_SIZE = {"A": 16, "B": 8, "C": 32, "D": 4}
+# E: the `tiny-b` preset as it ships (width 128, four query heads on ONE key/value head: a group
+# of four; vocabulary 512, untied head), which the entry points' smoke run and the command line use.
+TINY_E = {k: v for k, v in load_preset("tiny-b").items() if k not in ("torch_dtype", "use_sliding_window")}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+BLOCK_SIZE = {"A": 16, "B": 8, "C": 32, "D": 4, "E": 8}
 
 
 def make_model_dir(tmp_path: Path, which: str, seed: int = 0, storage_dtype: str = "bfloat16") -> Path:

@@ -10,6 +10,7 @@ import torch
 import plain_qwen2 as plain
 from mini_llm_runtime_amd.kernels.pending import PendingMerge, PendingNorm
 from mini_llm_runtime_amd.kernels.tuning import KernelTuning
+from qkv_reference import check_qkv, qkv_reference
 from test_gpu_kernels import _attention_reference, _paged_case, _rand, _tol
 
 pytestmark = pytest.mark.gpu
@@ -127,6 +128,17 @@ def test_norm_prologue_of_the_query_key_value_product(ops, heads, kv_heads, head
                                head_dim=head_dim, block_size=bs)
         stream = h.residual if fused else xs
         out[fused] = (q.float().cpu(), kp.float().cpu(), vp.float().cpu(), stream.cpu())
+        if not fused:
+            normed = h
+    # both ways against the float64 value of product, rotation and rounding, from the normed rows of
+    # the norm kernel.  The kernel that norms for itself may land a normed value on the neighbouring
+    # bfloat16 value now and then: one such value moves a product by 2^-8 of its largest term.
+    slack = float((normed.double().abs().max(dim=1).values[:, None] * w.double().abs().max(dim=1).values[None, :]).max()) * 2.0**-8
+    reference = qkv_reference(normed, w, b, rotation[0] if rotate else None, rotation[1] if rotate else None, heads,
+                              kv_heads, head_dim, p_slack=slack)
+    for fused in (False, True):
+        check_qkv("norm inside" if fused else "norm kernel first", *out[fused][:3], slots, bs, reference, heads, kv_heads,
+                  head_dim, max_neighbours=0.03 if not fused else 0.1)
     for name, a, c in zip(("queries", "key pages", "value pages"), out[False], out[True]):
         assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
         torch.testing.assert_close(torch.nan_to_num(c), torch.nan_to_num(a), msg=lambda m: f"{name}: {m}", **_tol(torch.bfloat16))

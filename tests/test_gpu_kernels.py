@@ -13,6 +13,7 @@ import pytest
 import torch
 
 import plain_qwen2 as plain
+from qkv_reference import check_qkv, qkv_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -352,6 +353,10 @@ def test_fused_qkv_rotation_cache_write_equals_the_three_kernels(ops_for, heads,
                                head_dim=head_dim, block_size=bs, write=write, fused=fused,
                                mfma_kernel=kernel if fused else 0)
         out[fused] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
+    # each way against the float64 value of the operation, within one ulp per operand of the rotation
+    reference = qkv_reference(x, w, b, rotation[0] if rotate else None, rotation[1] if rotate else None, heads, kv_heads, head_dim)
+    for fused in (False, True):
+        check_qkv("fused" if fused else "three kernels", *out[fused], slots, bs, reference, heads, kv_heads, head_dim, write=write)
     for name, a, c in zip(("queries", "key pages", "value pages"), out[False], out[True]):
         assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
         if tokens <= 16 and (kernel == 16 or (kernel == 0 and tokens > 8)):
@@ -402,6 +407,9 @@ def test_sliced_qkv_product_equals_the_three_kernels(ops_for, heads, kv_heads, h
         q = ops.qkv_rope_write(x, w, b, rotation, slots, kp, vp, num_heads=heads, num_kv_heads=kv_heads,
                                head_dim=head_dim, block_size=bs, write=write, **kw)
         out[way] = (q[:, : heads * head_dim].float().cpu(), kp.float().cpu(), vp.float().cpu())
+    reference = qkv_reference(x, w, b, rotation[0] if rotate else None, rotation[1] if rotate else None, heads, kv_heads, head_dim)
+    for way in out:
+        check_qkv(way, *out[way], slots, bs, reference, heads, kv_heads, head_dim, write=write)
     for name, a, c in zip(("queries", "key pages", "value pages"), out["unfused"], out["sliced"]):
         assert torch.equal(torch.isnan(a), torch.isnan(c)), f"{name}: other slots written"
         torch.testing.assert_close(torch.nan_to_num(c), torch.nan_to_num(a), msg=lambda m: f"{name}: {m}", **_tol(torch.bfloat16))
@@ -409,6 +417,67 @@ def test_sliced_qkv_product_equals_the_three_kernels(ops_for, heads, kv_heads, h
     if width * hidden * 2 >= 24 << 20 and tokens >= 4:
         for a, c in zip(out["sliced"], out["auto"]):
             assert torch.equal(torch.nan_to_num(a), torch.nan_to_num(c)), "the sliced way is chosen by itself here"
+
+
+def _drawn_qkv_case(case):
+    """The shape, positions and way that a seeded draw gives for `case`: head size, heads, width,
+    tokens, rotation, cache write, way (chosen by shape, fused, sliced), page size, positions."""
+    import random
+
+    rng = random.Random(9000 + case)
+    head_dim = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 256])
+    kv_heads = rng.choice([1, 2, 3, 4, 8])
+    heads = kv_heads * rng.choice([1, 2, 4, 7])
+    hidden = 8 * rng.choice([rng.randint(2, 60), rng.randint(60, 300), rng.randint(300, 700)])
+    tokens = rng.choice([1, 2, 3, rng.randint(4, 8), rng.randint(9, 16), rng.randint(17, 64), rng.randint(65, 400), rng.randint(400, 2100)])
+    if (heads + 2 * kv_heads) * head_dim * hidden > 6e7:
+        hidden = 8 * rng.randint(8, 100)
+    rotate, write = rng.random() < 0.85, rng.random() < 0.85
+    way = rng.choice(["auto", "fused", "sliced"])
+    bs = rng.choice([8, 16, 32])
+    positions = [rng.randint(0, 100000) for _ in range(tokens)] if rotate else None
+    return head_dim, kv_heads, heads, hidden, tokens, rotate, write, way, bs, positions
+
+
+@pytest.mark.parametrize("case", [23, 127, 182, 369, 5, 77])
+def test_qkv_ways_where_two_roundings_meet_a_subtraction(ops_for, case):
+    """Four drawn shapes (23, 127, 182, 369, of some 500) in which the fused or sliced way and the
+    three kernels differ by more than a relative bound on the RESULT allows, in one or two elements
+    each (|difference| 0.016 to 0.0625): the product of such an element lies at the middle between
+    two bfloat16 values, the two ways sum it in different orders and round it to different
+    neighbours, and the rotation then subtracts two products of nearly equal size, so one ulp of an
+    operand is many ulps of the result.  Both ways are within one ulp per operand of the float64
+    value, which is all that can be asked; two more draws stand for the ordinary case."""
+    head_dim, kv_heads, heads, hidden, tokens, rotate, write, way, bs, positions = _drawn_qkv_case(case)
+    ops = ops_for(torch.bfloat16)
+    pages = max(9, tokens // bs + 3)
+    width = (heads + 2 * kv_heads) * head_dim
+    x = _rand((tokens, hidden), torch.bfloat16, 71 + case).cuda()
+    w = _rand((width, hidden), torch.bfloat16, 72 + case, 0.2).cuda()
+    b = _rand((width,), torch.float32, 73 + case).cuda()
+    rotation = cos = sin = None
+    if rotate:
+        pos = torch.tensor(positions, dtype=torch.int32).cuda()
+        inv = (1.0 / (1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))).cuda()
+        cos, sin = ops.rope_table(pos, inv)
+        rotation = (cos, sin, head_dim)
+    g = torch.Generator().manual_seed(74 + case)
+    slots = torch.randperm(pages * bs, generator=g)[:tokens].to(torch.int32)
+    if tokens > 2:
+        slots[2] = -1
+    slots = slots.cuda()
+    reference = qkv_reference(x, w, b, cos, sin, heads, kv_heads, head_dim)
+    ways = {"three kernels": dict(fused=False)}
+    ways[way] = {} if way == "auto" else (dict(fused=True) if way == "fused" else dict(sliced=True))
+    if way == "sliced" and (tokens > 64 or hidden < 512 or not rotate):
+        ways[way] = {}
+    for name, kw in ways.items():
+        kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=torch.bfloat16).cuda()
+        vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=torch.bfloat16).cuda()
+        q = ops.qkv_rope_write(x, w, b, rotation, slots, kp, vp, num_heads=heads, num_kv_heads=kv_heads,
+                               head_dim=head_dim, block_size=bs, write=write, **kw)
+        check_qkv(name, q.float().cpu(), kp.float().cpu(), vp.float().cpu(), slots, bs, reference, heads, kv_heads,
+                  head_dim, write=write)
 
 
 # ---- attention ----------------------------------------------------------------------------------------
