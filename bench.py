@@ -11,10 +11,12 @@ timed steps between device synchronisations.  One JSON line is printed:
 `prefill` is one 2,048-token prompt; `roofline` prices the decode step by the
 bytes it must read (every weight once and the live requests' cache) against
 8 TB/s.  Peaks are MI355X's published dense figures.  `points_7b` and `points_32b`
-(default run only; `--no-large` leaves them out) hold decode at batch 8 and the
-prefill for the two larger shapes, with the number of layers run and of the full
-model beside them; `points_ctx16k` the same two measurements at a context of 16,384
-tokens for the 0.5B and the 7B shape.
+(default run only; `--no-large` leaves them out) hold decode at batch 1, 8 and 64 (tokens a
+second, step time, share of the HBM bound) and the prefill for the two larger shapes, the
+7B shape's burst workload and the 32B shape's chunked workload (below) as `burst` and
+`chunked`, with the number of layers run and of the full model beside them;
+`points_ctx16k` decode at batch 8 and the prefill at a context of 16,384 tokens for the 0.5B
+and the 7B shape.  `peak_memory_gb` (per shape) is the most device memory the run held.
 
 How it measures (the reference's harness rules, src/mini_llm_runtime/timing.py:49-82,
 141-160 and environment.py:37-93): untimed warm-up first; the timed steps between
@@ -55,7 +57,7 @@ def long_context_points(args) -> dict:
     long_args = copy.copy(args)
     long_args.prompt_len = 16384
     out = {"context": long_args.prompt_len}
-    for tag, name, layers in (("0.5b", "qwen2.5-0.5b", None), ("7b", "qwen2.5-7b", 28)):
+    for tag, name, layers in (("0.5b", "qwen2.5-0.5b", None), ("7b", "qwen2.5-7b", None)):
         point = large_point(long_args, name, layers)
         out[f"decode_b8_{tag}"] = point["decode_b8"]
         out[f"decode_b8_{tag}_hbm_frac"] = point["decode_b8_hbm_frac"]
@@ -81,6 +83,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked"))
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
+    p.add_argument("--layers-32b", type=int, default=None, help="layers of the 32B shape's points (default: all 64)")
     return p.parse_args()
 
 
@@ -473,34 +476,83 @@ class Bench:
             "samples_ms": [round(x, 3) for x in host],
         }
 
-    def close(self) -> None:
+    def peak_memory(self) -> dict:
+        """Device memory in GiB: the most this process's tensors held at one time since the shape was
+        set up (weights, page pool, recorded steps and their buffers; the reference records the same
+        counter, src/mini_llm_runtime/timing.py:141-160), the most the allocator had reserved for
+        them, and what the driver counts as in use on the device right now."""
+        import torch
+
+        free, total = torch.cuda.mem_get_info(self.device)
+        gib = float(2**30)
+        return {
+            "allocated": round(torch.cuda.max_memory_allocated(self.device) / gib, 2),
+            "reserved": round(torch.cuda.max_memory_reserved(self.device) / gib, 2),
+            "device_in_use": round((total - free) / gib, 2),
+        }
+
+    def collect(self) -> None:
         import gc
 
         import torch
 
-        for name in ("runner", "cache", "model", "sampler"):
-            setattr(self, name, None)
         gc.collect()
         torch.cuda.empty_cache()
 
+    def close(self) -> None:
+        for name in ("runner", "cache", "model", "sampler"):
+            setattr(self, name, None)
+        self.collect()
 
-def large_point(args, name: str, layers: int) -> dict:
-    """Decode at batch 8 and the prefill for a larger shape, `layers` of its layers."""
-    bench = Bench(args, name, layers, [8])
+
+def large_point(args, name: str, layers, batches=(8,), workload: str = "") -> dict:
+    """Decode at the given batch sizes and the prefill for a shape, `layers` of its layers (None: all of
+    them), peak device memory, and with `workload` the burst or the chunked workload as a compact
+    sub-object."""
+    import torch
+
+    bench = Bench(args, name, layers, list(batches))
     try:
+        torch.cuda.reset_peak_memory_stats(bench.device)
         warmup, steps = max(2, args.warmup // 2), max(8, args.steps // 2)
-        run = bench.decode(8, warmup, steps)
-        point = {
-            "layers": bench.config.num_hidden_layers,
-            "layers_full_model": bench.full_layers,
-            "decode_b8": round(8e3 / run["ms"], 1),
-            "decode_b8_ms": round(run["ms"], 4),
-            "decode_b8_ms_device": round(run["ms_device"], 4),
-            "decode_b8_hbm_frac": bench.roofline(8, run["ms"], warmup, steps)["frac"],
-        }
+        point = {"layers": bench.config.num_hidden_layers, "layers_full_model": bench.full_layers}
+        for b in batches:
+            run = bench.decode(b, warmup, steps)
+            point[f"decode_b{b}"] = round(b * 1e3 / run["ms"], 1)
+            point[f"decode_b{b}_ms"] = round(run["ms"], 4)
+            if b == 8:
+                point["decode_b8_ms_device"] = round(run["ms_device"], 4)
+            point[f"decode_b{b}_hbm_frac"] = bench.roofline(b, run["ms"], warmup, steps)["frac"]
         if not args.no_prefill:
             pre = bench.prefill(repeats=3)
             point.update(prefill=pre["value"], prefill_ms=pre["ms"], prefill_frac=pre["frac"])
+        point["peak_memory_gb"] = bench.peak_memory()
+        if workload:
+            bench.runner = bench.cache = None  # the workloads size a cache of their own
+            bench.collect()
+            line = (burst if workload == "burst" else chunked)(
+                args, bench.config, bench.full_layers, bench.model, bench.ops, bench.device
+            )
+            if workload == "burst":
+                point["burst"] = {
+                    "generated_tokens_per_s": line["value"],
+                    "total_tokens_per_s": line["total_tokens_per_s"],
+                    "median_ttft_ms": line["median_ttft_ms"],
+                    "median_tpot_ms": line["median_tpot_ms"],
+                    "seconds": line["seconds"],
+                    "requests": line["config"]["requests"],
+                    "max_batch_tokens": line["config"]["max_batch_tokens"],
+                }
+            else:
+                point["chunked"] = {
+                    "mixed_step_ms": line["value"],
+                    "decoders_tpot_ms_beside_the_prompt": line["decoders_tpot_ms_beside_the_prompt"],
+                    "decoders_tpot_ms_alone": line["decoders_tpot_ms_alone"],
+                    "prompt_tokens_per_s": line["prompt_tokens_per_s"],
+                    "decoders": line["config"]["decoders"],
+                    "prompt_len": line["config"]["prompt_len"],
+                    "portion": line["config"]["portion"],
+                }
         return point
     finally:
         bench.close()
@@ -538,6 +590,7 @@ def main() -> int:
     prefill = None if args.no_prefill else bench.prefill()
     kv_per_token = bench.kv_bytes_per_token()
     full_layers = bench.full_layers
+    peak_memory = bench.peak_memory()
     bench.close()
 
     line = {
@@ -577,10 +630,14 @@ def main() -> int:
         "roofline": roofline,
         "points": points,
         "step_samples": summary(main_run["samples"], args.samples),
+        "peak_memory_gb": peak_memory,
     }
     if not args.no_large and args.config == "qwen2.5-0.5b" and args.layers is None and args.dtype == "bfloat16":
-        line["points_7b"] = large_point(args, "qwen2.5-7b", 28)
-        line["points_32b"] = large_point(args, "qwen2.5-32b", 16)
+        # the other configurations' measurements: decode at batch 1, 8 and 64 and the prefill for the 7B
+        # shape and the whole 32B shape (64 layers, 65 GB of weights), the burst of 64 requests on the
+        # 7B shape, the 8,192-token prompt in portions beside 32 decoding requests on the 32B shape
+        line["points_7b"] = large_point(args, "qwen2.5-7b", None, (1, 8, 64), "burst")
+        line["points_32b"] = large_point(args, "qwen2.5-32b", args.layers_32b, (1, 8, 64), "chunked")
         if args.prompt_len == PROMPT_LEN:
             line["points_ctx16k"] = long_context_points(args)
     line["env"] = environment()

@@ -47,3 +47,5 @@ def test_default_line_keeps_the_contract(tmp_path):
     roof = line["roofline"]
     assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert set(line["points"]) == {"decode_b1", "decode_b64"}
+    memory = line["peak_memory_gb"]  # weights (about 1 GB) and the page pool at least, the card's 288 GB at most
+    assert 1.0 < memory["allocated"] <= memory["reserved"] < 288 and memory["device_in_use"] >= memory["reserved"]

@@ -65,6 +65,7 @@ def test_static_scratch_sampling_equals_the_one_with_a_buffer():
     _both(lib, rows=1, vocab=17, seed=3)
 
 
+@torch.inference_mode()  # as the engine records its steps (torch's capture state was made under it by then)
 def test_static_scratch_sampling_inside_a_graph_capture():
     """A capture forbids allocation: the call is recorded after one call outside (the address of
     the array is looked up at the first call), then replayed with new logits each time and
