@@ -84,7 +84,28 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
     p.add_argument("--layers-32b", type=int, default=None, help="layers of the 32B shape's points (default: all 64)")
+    p.add_argument("--tuning", default="", help="KernelTuning fields to change, e.g. finish_stream=false,decode_partition=128")
     return p.parse_args()
+
+
+def kernel_tuning(text: str):
+    """A KernelTuning with the fields named in `text` (name=value, comma separated) changed; None for none."""
+    from dataclasses import fields, replace
+
+    from mini_llm_runtime_amd.kernels.tuning import KernelTuning
+
+    if not text:
+        return None
+    kinds = {f.name: f.type for f in fields(KernelTuning)}
+    changes = {}
+    for item in text.split(","):
+        name, _, value = item.partition("=")
+        name = name.strip()
+        if name not in kinds:
+            raise SystemExit(f"--tuning: KernelTuning has no field {name!r} (it has {', '.join(sorted(kinds))})")
+        default = getattr(KernelTuning(), name)
+        changes[name] = value.strip().lower() in ("1", "true", "yes", "on") if isinstance(default, bool) else int(value)
+    return replace(KernelTuning(), **changes)
 
 
 def median(values):
@@ -338,7 +359,7 @@ class Bench:
         self.dtype = parse_dtype(args.dtype)
         self.short = "bf16" if self.dtype == torch.bfloat16 else "fp32"
         self.device = torch.device("cuda", 0)
-        self.ops = default_ops(self.dtype, self.device)
+        self.ops = default_ops(self.dtype, self.device, kernel_tuning(args.tuning))
         self.model = build_model(self.config)
         bind_random_weights(self.model, seed=args.seed, dtype=self.dtype, device=self.device)
         self.batches = batches
@@ -632,6 +653,8 @@ def main() -> int:
         "step_samples": summary(main_run["samples"], args.samples),
         "peak_memory_gb": peak_memory,
     }
+    if args.tuning:
+        line["tuning"] = args.tuning
     if not args.no_large and args.config == "qwen2.5-0.5b" and args.layers is None and args.dtype == "bfloat16":
         # the other configurations' measurements: decode at batch 1, 8 and 64 and the prefill for the 7B
         # shape and the whole 32B shape (64 layers, 65 GB of weights), the burst of 64 requests on the

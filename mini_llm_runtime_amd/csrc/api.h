@@ -83,18 +83,36 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
 // tokens x 64 features), 11, 22, 44 (LDS-tiled with 64 x 64, 128 x 128, 256 x 256 tiles) force
 // one, for tests and tuning.  Any `slices` within
 // 1..64 is accepted with a float32 [slices, m, n] output.
+// row_sumsq (null: none): the rows of x still owe their normalisation (mlr_gemm_residual_bf16 made
+// them): float32 [m, sumsq_parts] partial sums of squares of every row of the residual stream; the
+// sums of row i are scaled by rsqrt(sum_p row_sumsq[i, p] / k + norm_eps) before the bias.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y,
-                  int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k, hipStream_t stream);
+                  int out_is_f32, int swiglu, int slices, int kernel, int m, int n, int k,
+                  const float* row_sumsq, int sumsq_parts, float norm_eps, hipStream_t stream);
+
+// A product that finishes the residual stream (gemm_stream.hip): y = a w^T (+ bias), a [m, k] and w
+// [n, k] bfloat16; then, every workgroup for its own columns of all rows, stream[m, n] (float32, in
+// place) += y, h[m, n] (bfloat16) = norm_weight * stream (the next norm's weight, float32 or
+// bfloat16; its division by the root mean square is left to the consumer), and sumsq[m, parts] =
+// this workgroup's share of every row's sum of squares of the new stream, parts =
+// mlr_gemm_residual_parts(m, n).  One kernel where a product cut along k needs a second one to add
+// the slices up, to add the residual and to norm; it pays while a workgroup can afford to read all
+// m rows of a (up to 64 tokens, n a multiple of 4, k of 8).
+int mlr_gemm_residual_parts(int m, int n);
+int mlr_gemm_residual_bf16(const void* a, const void* w, const void* bias, int bias_is_f32, float* stream,
+                           const void* norm_weight, int norm_weight_is_f32, void* h, float* sumsq, int m, int n,
+                           int k, hipStream_t stream_handle);
 
 // The query/key/value product fused with bias, rotation (cos, sin: [m, head_dim / 2] float32,
 // or null), the queries' store to q_out [m, heads * head_dim] and the keys' and values' store
 // into their cache slots (`write` 0: no cache write).  kernel: 0 chooses; 16 the row-splitting
 // kernel (up to 64 tokens); 8 its variant with 8 weight rows a workgroup (up to 8 tokens); 11,
-// 22, 44 the tiled kernels as in mlr_gemm_bf16.
+// 22, 44 the tiled kernels as in mlr_gemm_bf16.  row_sumsq, sumsq_parts, norm_eps as there.
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
                             const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
-                            int write, int kernel, hipStream_t stream);
+                            int write, int kernel, const float* row_sumsq, int sumsq_parts, float norm_eps,
+                            hipStream_t stream);
 
 // Products of up to 16 tokens that make their own activations (gemm_fused.hip).
 // Norm prologue: h = RMSNorm(x_in + delta) * norm_weight with the delta a bfloat16 [m, k]

@@ -14,7 +14,85 @@ struct GemmEpilogue {
   void* y;
   int out_is_f32;
   int swiglu;  // store silu(v0) * v2, silu(v1) * v3 into a row of N / 2
+  // Rows whose normalisation is still owed (see gemm_stream.hip): x holds weight * stream, not yet
+  // divided by the root mean square of the stream.  The sums of a row m are then scaled by
+  // rsqrt(sum_p row_sumsq[m, p] / K + eps) before the bias: the factor is the same for the whole
+  // row, so it commutes with the product.  Null: no scaling.
+  const float* row_sumsq = nullptr;  // [M, sumsq_parts]: partial sums of squares of every stream row
+  int sumsq_parts = 0;
+  float norm_eps = 0.f;
 };
+
+// The scaling factors of rows m0 .. m0 + count - 1 into `scales` (LDS), by all wavefronts of the
+// workgroup (a whole number of them): wavefront w takes the rows w, w + waves, ..., its lanes the
+// partial sums lane, lane + 64, ... of a row, added in that fixed order.  The work comes in two
+// halves so that the loads can be sent before the product's own loads and be added up after its
+// loop, when they have long arrived: a wait for them in front of the loop would put a trip to L2
+// before the first weight is asked for.  `issue` sends the loads of up to ROWS rows per wavefront
+// and LOADS partial sums per lane and row; `finish` adds up, and fetches whatever `issue` could
+// not hold the slow way (shapes beyond ROWS x waves rows or 64 x LOADS partial sums).  The
+// caller's next __syncthreads() makes the factors visible.
+template <int ROWS, int LOADS>
+struct RowScaleLoads {
+  float v[ROWS][LOADS];
+  bool held;  // the registers hold everything
+};
+
+template <int ROWS, int LOADS>
+__device__ __forceinline__ void row_scales_issue(const GemmEpilogue& ep, RowScaleLoads<ROWS, LOADS>& t, int m0, int count,
+                                                 int M) {
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int waves = blockDim.x / kWave;
+  t.held = count <= ROWS * waves && ep.sumsq_parts <= kWave * LOADS;
+  if (!t.held) return;
+  // range-checked buffer loads, no condition around any of them (a load inside a conditional block
+  // makes the compiler wait for every outstanding load where the block ends): what is past a row's
+  // partial sums or past the last row reads zero
+  const __amdgpu_buffer_rsrc_t buf = make_buffer(ep.row_sumsq, static_cast<unsigned>(M) * ep.sumsq_parts * 4u);
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    const int row = wave + i * waves;
+    const int m = m0 + row;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+      const int p = lane + j * kWave;
+      const unsigned off = (row < count && m < M && p < ep.sumsq_parts)
+                               ? (static_cast<unsigned>(m) * ep.sumsq_parts + p) * 4u
+                               : kOutOfBuffer;
+      t.v[i][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(buf, off, 0, 0));
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);  // sent here, ahead of the product's loads
+}
+
+template <int ROWS, int LOADS>
+__device__ __forceinline__ void row_scales_finish(const GemmEpilogue& ep, const RowScaleLoads<ROWS, LOADS>& t, int m0,
+                                                  int count, int M, int K, float* scales) {
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int waves = blockDim.x / kWave;
+  if (t.held) {
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      const int row = wave + i * waves;
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) s += t.v[i][j];
+      s = wave_sum(s);
+      if (lane == 0 && row < count) scales[row] = m0 + row < M ? 1.0f / sqrtf(s / static_cast<float>(K) + ep.norm_eps) : 0.f;
+    }
+    return;
+  }
+  for (int row = wave; row < count; row += waves) {
+    const int m = m0 + row;
+    float s = 0.f;
+    if (m < M)
+      for (int p = lane; p < ep.sumsq_parts; p += kWave) s += ep.row_sumsq[static_cast<int64_t>(m) * ep.sumsq_parts + p];
+    s = wave_sum(s);
+    if (lane == 0) scales[row] = m < M ? 1.0f / sqrtf(s / static_cast<float>(K) + ep.norm_eps) : 0.f;
+  }
+}
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 

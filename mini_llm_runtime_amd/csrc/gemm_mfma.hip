@@ -50,6 +50,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
                                                                        int K) {
   constexpr int U = MT > 2 ? 4 : 8;  // k-steps in flight per wavefront
   __shared__ float red[WAVES][MT][kWave][4];
+  __shared__ float scales[MT * 16];
+  RowScaleLoads<MT * 16 / WAVES, 4 / MT> owed;  // up to 256 partial sums a row for 16 tokens, 64 for 64 tokens
+  if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, 0, min(M, MT * 16), M);
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int r = lane % 16;
@@ -110,6 +113,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][mt][lane][i] = acc[mt][i];
+  if (ep.row_sumsq != nullptr) row_scales_finish(ep, owed, 0, min(M, MT * 16), M, K, scales);
   __syncthreads();
   if (wave != 0) return;
 #pragma unroll
@@ -119,6 +123,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] += red[ww][mt][lane][i];
     const int token = mt * 16 + r;
+    if (ep.row_sumsq != nullptr && token < M) {
+      const float scale = scales[token];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= scale;
+    }
     if constexpr (!QKV) {
       finish4(ep, blockIdx.y, slices, token, n0 + q * 4, M, N, v);
     } else {
@@ -142,6 +151,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_qkv8_kernel(const bf16
                                                                       QkvTarget qkv, int M, int N, int K) {
   constexpr int U = 8;  // k-steps in flight per wavefront
   __shared__ float red[WAVES][kWave][4];
+  __shared__ float scales[8];
+  RowScaleLoads<8 / WAVES, 4> owed;
+  if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, 0, min(M, 8), M);
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int r = lane % 16;
@@ -186,6 +198,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_qkv8_kernel(const bf16
 
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+  if (ep.row_sumsq != nullptr) row_scales_finish(ep, owed, 0, min(M, 8), M, K, scales);
   __syncthreads();
   if (wave != 0) return;
   // lane (r < 8, q < 2) owns weight slots 4q..4q+3 of token r: its own quadrant over the first
@@ -196,6 +209,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_qkv8_kernel(const bf16
   for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] += red[ww][lane][i] + red[ww][other][i];
+  if (ep.row_sumsq != nullptr && r8 < M) {
+    const float scale = scales[r8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] *= scale;
+  }
   const int qq = q & 1;
   qkv_finish_pairs(ep, qkv, head, rotated, row_of(qq * 4) - head * qkv.head_dim, block_in_head * 4, qq == 0, 16,
                    min(r8, M - 1), owner && r8 < M, v);
@@ -263,6 +281,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* const lds = reinterpret_cast<bf16*>(smem);
   constexpr int kBuffer = (BM + BN) * kLd;
+  __shared__ float scales[BM];  // of the tile's token rows, when their normalisation is still owed
 
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
@@ -275,6 +294,10 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
   place_workgroup(order, blockIdx.x, slice, mt, nt);
   const int n0 = nt * BN;
   const int m0 = mt * BM;
+  // (tiles of up to 64 tokens hold their rows' partial sums in registers over the loop; larger
+  // tiles never see such rows in practice and fetch them the slow way)
+  RowScaleLoads<(BM <= 64 ? BM / (GM * GN) : 1), (BM <= 64 ? 2 : 1)> owed;
+  if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, m0, BM, M);
   const int chunks = K / 8;
   const int slices = order.slices;
   const int k_slices = (K + kBK - 1) / kBK;
@@ -401,16 +424,22 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
     }
   }
 
+  if (ep.row_sumsq != nullptr) {
+    row_scales_finish(ep, owed, m0, BM, M, K, scales);
+    __syncthreads();
+  }
   if constexpr (!QKV) {
 #pragma unroll
     for (int i = 0; i < WN; ++i)
 #pragma unroll
       for (int j = 0; j < WM; ++j) {
         const int m = m0 + (wm * WM + j) * 32 + r32;
+        const float scale = ep.row_sumsq != nullptr ? scales[(wm * WM + j) * 32 + r32] : 1.f;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int n = n0 + (wn * WN + i) * 32 + g * 8 + h * 4;
-          const float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+          const float v[4] = {acc[i][j][g * 4 + 0] * scale, acc[i][j][g * 4 + 1] * scale, acc[i][j][g * 4 + 2] * scale,
+                              acc[i][j][g * 4 + 3] * scale};
           finish4(ep, slice, slices, m, n, M, N, v);
         }
       }
@@ -427,6 +456,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float v = acc[i][j][g * 4 + e];
+            if (ep.row_sumsq != nullptr) v *= scales[(wm * WM + j) * 32 + r32];
             if (ep.bias != nullptr && row0[i][g] >= 0) v += load_as_f32(ep.bias, row0[i][g] + e, ep.bias_is_f32);
             acc[i][j][g * 4 + e] = to_f32(f32_to_bf16(v));
           }
@@ -703,7 +733,8 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
 // mlr_gemm_bf16_slices; not with swiglu) y is float32 [slices, m, n]: partial sums
 // over slices of k, the bias in slice 0, for the consumer to add up.
 int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, void* y, int out_is_f32,
-                  int swiglu, int slices, int kernel, int m, int n, int k, hipStream_t stream) {
+                  int swiglu, int slices, int kernel, int m, int n, int k, const float* row_sumsq, int sumsq_parts,
+                  float norm_eps, hipStream_t stream) {
   MLR_REQUIRE(x && w && y, "null pointer");
   MLR_REQUIRE(m > 0 && n > 0 && k > 0, "sizes must be > 0");
   MLR_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
@@ -713,7 +744,9 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
   MLR_REQUIRE(slices == 1 || (!swiglu && out_is_f32), "partial sums are float32, without SwiGLU");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
               "x and w must be 16-byte aligned");
-  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu};
+  MLR_REQUIRE(row_sumsq == nullptr || (sumsq_parts > 0 && sumsq_parts <= (1 << 16) && norm_eps >= 0.f),
+              "sums of squares come with their number per row (1..65536) and an eps >= 0");
+  GemmEpilogue ep{bias, bias_is_f32, y, out_is_f32, swiglu, row_sumsq, sumsq_parts, norm_eps};
   if (kernel == 0) kernel = choose_kernel(m, n, k, slices);
   if (gemm_bf16(static_cast<const bf16*>(x), static_cast<const bf16*>(w), ep, m, n, k, slices, kernel, stream) != 0)
     return -1;
@@ -729,8 +762,11 @@ int mlr_gemm_bf16(const void* x, const void* w, const void* bias, int bias_is_f3
 int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int bias_is_f32, const float* cos,
                             const float* sin, const int* slots, void* key_pages, void* value_pages, void* q_out,
                             int m, int k, int heads, int kv_heads, int head_dim, int block_size, int num_pages,
-                            int write, int kernel, hipStream_t stream) {
+                            int write, int kernel, const float* row_sumsq, int sumsq_parts, float norm_eps,
+                            hipStream_t stream) {
   MLR_REQUIRE(x && w && q_out, "null pointer");
+  MLR_REQUIRE(row_sumsq == nullptr || (sumsq_parts > 0 && sumsq_parts <= (1 << 16) && norm_eps >= 0.f),
+              "sums of squares come with their number per row (1..65536) and an eps >= 0");
   MLR_REQUIRE(m > 0, "no tokens");
   MLR_REQUIRE(k > 0 && k % 8 == 0 && k <= (1 << 20), "k must be a positive multiple of 8, at most 2^20");
   MLR_REQUIRE(heads > 0 && kv_heads > 0 && head_dim >= 16 && head_dim % 16 == 0, "head_dim must be a multiple of 16");
@@ -743,7 +779,7 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
               "operands must be 16-byte aligned");
   const int64_t n = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
   MLR_REQUIRE(n / 16 < (1ll << 31), "too many rows for one launch");
-  GemmEpilogue ep{bias, bias_is_f32, nullptr, 0, 0};
+  GemmEpilogue ep{bias, bias_is_f32, nullptr, 0, 0, row_sumsq, sumsq_parts, norm_eps};
   QkvTarget target{cos, sin, write ? slots : nullptr, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages),
                    static_cast<bf16*>(q_out), heads, kv_heads, head_dim, block_size, num_pages};
   const bf16* xb = static_cast<const bf16*>(x);

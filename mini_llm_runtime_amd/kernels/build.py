@@ -61,6 +61,7 @@ CORE = Module(
         "gemm_simple.hip",
         "gemm_mfma.hip",
         "gemm_fused.hip",
+        "gemm_stream.hip",
         "attention_simple.hip",
         "sampling.hip",
     ),

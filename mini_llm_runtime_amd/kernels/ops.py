@@ -18,7 +18,7 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from . import build
-from .pending import PendingMerge, PendingNorm
+from .pending import PendingLinear, PendingMerge, PendingNorm, PendingScale
 from .tuning import KernelTuning
 
 _VP = ctypes.c_void_p
@@ -38,10 +38,12 @@ _SIGNATURES = {
     "mlr_rope_kv_write": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP], _I),
-    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP], _I),
+    "mlr_gemm_residual_parts": ([_I, _I], _I),
+    "mlr_gemm_residual_bf16": ([_VP, _VP, _VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
     "mlr_qkv_rope_write_bf16": (
-        [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP],
         _I,
     ),
     "mlr_gemm_norm_fused_bf16": (
@@ -225,6 +227,7 @@ class HipOps:
         self._check(x, "residual stream", torch.float32, (None, None))
         rows, hidden = x.shape
         self._check(weight, "norm weight", (torch.float32, self.dtype), (hidden,))
+        delta = self.settle(delta)
         plain = partial = None
         slices = 0
         if delta is not None and delta.dim() == 3:
@@ -242,6 +245,7 @@ class HipOps:
     def add_(self, x: torch.Tensor, delta: torch.Tensor) -> None:
         """x (float32) += delta (the engine's dtype, or float32), in place."""
         self._check(x, "residual stream", torch.float32)
+        delta = self.settle(delta)
         self._check(delta, "residual delta", (self.dtype, torch.float32), tuple(x.shape))
         self._call("mlr_add", self._ptr(x), self._ptr(delta), _dtype_code(delta.dtype), x.numel(), self._stream())
 
@@ -253,7 +257,12 @@ class HipOps:
         self._call("mlr_scale_softcap", self._ptr(x), float(scale), float(cap or 0.0), x.numel(), self._stream())
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
-        """x[rows] for x [T, H], or x[:, rows] for a stack [S, T, H]."""
+        """x[rows] for x [T, H], or x[:, rows] for a stack [S, T, H].  Of a product that has not run,
+        the product of the chosen rows of its input, still not run: a row's values are then made by
+        the same kernels whether it was chosen or all rows were taken."""
+        if isinstance(x, PendingLinear):
+            return PendingLinear(self.gather_rows(self.settle(x.x), rows), x.weight, x.bias)
+        x = self.settle(x)
         self._check(x, "rows source", (torch.float32, torch.bfloat16))
         if x.dim() not in (2, 3):
             raise KernelError("gather_rows takes [T, H] or [S, T, H]")
@@ -280,6 +289,8 @@ class HipOps:
     def defer_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor]):
         """The norm of `rmsnorm` as a `PendingNorm` when the product behind it could compute it
         in its own kernel (bfloat16, few tokens, a narrow model); else None."""
+        if isinstance(delta, PendingLinear):
+            return self._finish_stream(x, weight, float(eps), delta)  # None: the caller's norm kernel settles it
         if not (self.tuning.fuse_norm and self.dtype == torch.bfloat16 and x.dim() == 2):
             return None
         rows, hidden = x.shape
@@ -297,6 +308,12 @@ class HipOps:
                 h.value = self.rmsnorm(h.x, h.weight, h.eps, delta=h.delta)
                 h.residual = h.x
             return h.value
+        if isinstance(h, PendingScale):
+            if h.value is None:
+                h.value = self.rmsnorm(h.residual, h.weight, h.eps)
+            return h.value
+        if isinstance(h, PendingLinear):
+            return self.linear(h.x, h.weight, h.bias, partial_sums=True)
         if isinstance(h, PendingMerge):
             out = self._empty((h.tokens, h.heads * h.head_dim), self.dtype)
             self._call(
@@ -305,6 +322,48 @@ class HipOps:
             )
             return out
         return h
+
+    def _can_finish_stream(self, m: int, n: int, k: int) -> bool:
+        """Whether the product [m, k] x [n, k]^T may run as the kernel that adds its result to the
+        residual stream itself (`mlr_gemm_residual_bf16`)."""
+        t = self.tuning
+        return (
+            t.finish_stream and self.dtype == torch.bfloat16 and k % 8 == 0 and n % 4 == 0
+            and max(1, t.finish_min_tokens) <= m <= min(64, t.finish_max_tokens)
+            and n * k * 2 <= t.finish_weight_bytes and m * k * 2 <= t.finish_activation_bytes
+        )
+
+    def _finish_stream(self, x: torch.Tensor, weight: torch.Tensor, eps: float, pending: PendingLinear):
+        """Run a pending product as the kernel that adds it to the stream `x` (in place) and leaves
+        the norm's activations short of the factor per row: a `PendingScale`."""
+        self._check(x, "residual stream", torch.float32, (None, None))
+        rows, hidden = x.shape
+        a = self.settle(pending.x)  # attention still in partitions is merged by its own kernel
+        m, k = a.shape
+        if m != rows or pending.weight.shape[0] != hidden or not self._can_finish_stream(m, hidden, k):
+            return None
+        self._check(a, "linear input", self.dtype, (m, k))
+        self._check(pending.weight, "linear weight", self.dtype, (hidden, k))
+        self._check(weight, "norm weight", (torch.float32, self.dtype), (hidden,))
+        bias = pending.bias
+        if bias is not None:
+            self._check(bias, "linear bias", (torch.float32, self.dtype), (hidden,))
+        parts = self.lib.mlr_gemm_residual_parts(m, hidden)
+        h = self._empty((m, hidden), self.dtype)
+        sumsq = self._empty((m, parts), torch.float32)
+        self._call(
+            "mlr_gemm_residual_bf16", self._ptr(a), self._ptr(pending.weight), self._ptr(bias),
+            int(bias is not None and bias.dtype == torch.float32), self._ptr(x), self._ptr(weight),
+            int(weight.dtype == torch.float32), self._ptr(h), self._ptr(sumsq), m, hidden, k, self._stream(),
+        )
+        return PendingScale(h, sumsq, weight, eps, x)
+
+    @staticmethod
+    def _no_scale() -> tuple:
+        return (_VP(None), 0, 0.0)
+
+    def _scale_arguments(self, h: PendingScale) -> tuple:
+        return (self._ptr(h.sumsq), h.sumsq.shape[1], float(h.eps))
 
     def _norm_arguments(self, h: PendingNorm):
         """(checked tensors, ctypes arguments) of a norm prologue; allocates the updated stream."""
@@ -337,8 +396,13 @@ class HipOps:
         partial_sums: bool = False,
         mfma_kernel: int = 0,
         slices: Optional[int] = None,
+        for_stream: bool = False,
     ) -> torch.Tensor:
         """x [M, K] times weight [N, K] transposed, plus bias [N]; F.linear semantics.
+
+        for_stream: the result is a part's output and goes nowhere but into the next norm as its
+        delta (as with partial_sums); it may then come back unrun, as a `PendingLinear` that the norm
+        runs together with the addition to the residual stream.
 
         bfloat16 products run on the matrix cores when k is a multiple of 8; float32
         products, and everything with kernel="fma", run as plain 32-bit FMA arithmetic.
@@ -353,11 +417,25 @@ class HipOps:
         """
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
+        if for_stream:
+            partial_sums = True
+            m, k = x.shape
+            if (
+                kernel == "auto" and not swiglu and not mfma_kernel and slices is None and out_dtype in (None, self.dtype)
+                and not isinstance(x, (PendingNorm, PendingScale)) and self._can_finish_stream(m, weight.shape[0], k)
+            ):
+                return PendingLinear(x, weight, bias)
         if isinstance(x, (PendingNorm, PendingMerge)):
             fused = self._linear_fused(x, weight, bias, out_dtype, kernel, swiglu, partial_sums, mfma_kernel, slices)
             if fused is not None:
                 return fused
             x = self.settle(x)
+        scale = self._no_scale()
+        if isinstance(x, PendingScale):
+            if x.value is None and kernel == "auto" and self.dtype == torch.bfloat16 and x.h.shape[1] % 8 == 0:
+                scale, x = self._scale_arguments(x), x.h  # the product scales its sums row by row
+            else:
+                x = self.settle(x)
         self._check(x, "linear input", self.dtype, (None, None))
         m, k = x.shape
         self._check(weight, "linear weight", self.dtype, (None, k))
@@ -385,7 +463,7 @@ class HipOps:
                 out_f32 = int(out_dtype == torch.float32)
             self._call(
                 "mlr_gemm_bf16", self._ptr(x), self._ptr(weight), self._ptr(bias), bias_f32, self._ptr(y), out_f32,
-                int(swiglu), slices, int(mfma_kernel), m, n, k, self._stream(),
+                int(swiglu), slices, int(mfma_kernel), m, n, k, *scale, self._stream(),
             )
             return y
         y = self._empty((m, n // 2 if swiglu else n), out_dtype)
@@ -542,6 +620,12 @@ class HipOps:
         pending = x if isinstance(x, PendingNorm) and x.value is None else None
         if isinstance(x, PendingNorm) and pending is None:
             x = x.value
+        scaled = None  # rows that still owe their normalisation: every way below ends in a product that pays it
+        if isinstance(x, PendingScale):
+            if x.value is None and self.dtype == torch.bfloat16 and x.h.shape[1] % 8 == 0:
+                scaled = x
+            else:
+                x = self.settle(x)
         m, k = x.shape
         width = (num_heads + 2 * num_kv_heads) * head_dim
         can_fuse = (
@@ -574,7 +658,7 @@ class HipOps:
             raise KernelError("the sliced query/key/value product takes up to 128 bfloat16 tokens and a full rotation")
         if sliced:
             slices = (8 if k >= 2048 else 4) if m <= 64 else max(2, self.lib.mlr_gemm_bf16_slices(m, width, k, 4))
-            partial = self.linear(x, weight, bias, partial_sums=True, slices=slices)
+            partial = self.linear(x, weight, bias, partial_sums=True, slices=slices)  # scales each slice, if owed
             cos = sin = None
             if rotation is not None:
                 cos, sin, _ = rotation
@@ -612,6 +696,9 @@ class HipOps:
                 num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size, write=write,
             )
             return qkv
+        scale = self._no_scale()
+        if scaled is not None:
+            scale, x = self._scale_arguments(scaled), scaled.h
         if pending is None:
             self._check(x, "linear input", self.dtype, (None, None))
         self._check(weight, "qkv weight", self.dtype, (width, k))
@@ -643,7 +730,7 @@ class HipOps:
             int(bias is not None and bias.dtype == torch.float32), self._ptr(cos), self._ptr(sin),
             self._ptr(slot_mapping if write else None), self._ptr(key_pages if write else None),
             self._ptr(value_pages if write else None), self._ptr(q), m, k, num_heads, num_kv_heads, head_dim,
-            block_size, num_pages, int(write), mfma_kernel, self._stream(),
+            block_size, num_pages, int(write), mfma_kernel, *scale, self._stream(),
         )
         return q
 

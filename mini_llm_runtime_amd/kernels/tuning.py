@@ -31,8 +31,27 @@ class KernelTuning:
     # runs (up to 8) with a workgroup each, until there are this many.
     key_run_groups: int = 384
 
+    # The last product of a part (output projection, down projection) as a kernel that owns whole
+    # output columns and adds them to the residual stream itself, with the next norm left as one
+    # factor per row for the product behind it: one kernel instead of a product cut along k plus a
+    # norm kernel.  Measured inside a replayed graph at 0.5B sizes (microseconds a call, weights of 24
+    # layers in turn): the norm kernel it saves costs 2.7, the product that owns its columns costs 1.0
+    # more than the one cut along k for the output projection (1.6 MB: 4.4 against 3.3) and 3.0 more
+    # for the down projection (8.7 MB, k = 4,864: 7.9 against 4.9: few workgroups, each held to the
+    # 20 GB/s that a compute unit takes in), and the consumer's scaling costs 0.7 to 1.0.  So it pays
+    # for small matrices only, 0.7 us a layer at 5 to 8 tokens, and loses everywhere else: below 5
+    # tokens to the norm done in the consumer's prologue, from 9 tokens on to the activations that
+    # every workgroup reads.  The limits below say where it is used.
+    finish_stream: bool = True
+    finish_weight_bytes: int = 4 << 20
+    finish_activation_bytes: int = 160 << 10
+    finish_min_tokens: int = 5
+    finish_max_tokens: int = 8
+
     def __post_init__(self) -> None:
-        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups", "fuse_weight_bytes"):
+        for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups", "fuse_weight_bytes",
+                     "finish_weight_bytes", "finish_activation_bytes", "finish_min_tokens",
+                     "finish_max_tokens"):
             value = getattr(self, name)
             if isinstance(value, bool) or not isinstance(value, int) or value <= 0:
                 raise ValueError(f"KernelTuning.{name} must be a positive integer")

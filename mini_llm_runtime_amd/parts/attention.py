@@ -142,4 +142,4 @@ class GQAAttention(Mixer):
             defer_merge=True,  # the output product is the only reader
             plan=ctx.plan(getattr(ops, "ATTENTION_PLAN", None)),
         )
-        return ops.linear(attended, self.o_weight, self.o_bias_vec, partial_sums=True)
+        return ops.linear(attended, self.o_weight, self.o_bias_vec, for_stream=True)  # the next norm's delta

@@ -53,7 +53,8 @@ class Norm(Part):
         """x: float32 residual stream [T, H].  When `delta` is given, first x += delta
         (in place, summed in 32-bit); returns norm(x) in the engine's dtype.  `delta` is a
         part's output: [T, H] in the engine's dtype, or, from a part that ends in
-        `ops.linear(..., partial_sums=True)`, a float32 stack [S, T, H] whose sum over S it is."""
+        `ops.linear(..., for_stream=True)`, whatever that returned (a float32 stack [S, T, H] whose
+        sum over S it is, or a product that has not run): the kernel library's norm takes all of them."""
         raise NotImplementedError
 
 

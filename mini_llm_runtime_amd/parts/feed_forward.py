@@ -42,4 +42,4 @@ class SwiGLU(FeedForward):
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
         hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
-        return ops.linear(hidden, self.down_weight, None, partial_sums=True)
+        return ops.linear(hidden, self.down_weight, None, for_stream=True)  # the next norm's delta

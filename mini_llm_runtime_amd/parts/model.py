@@ -162,6 +162,7 @@ class DecoderModel:
                 rows = ops.gather_rows(x, logit_rows)
                 if delta is not None:
                     own = ops.gather_rows(delta, logit_rows)
+                    own = getattr(ops, "settle", lambda t: t)(own)  # a product that has not run yet, run now
                     rows = rows + (own.sum(0) if own.dim() == 3 else own.float())
                 site_outputs.append(rows)
         if logit_rows is None or logit_rows.numel() == 0:
@@ -171,7 +172,11 @@ class DecoderModel:
         else:
             rows = ops.gather_rows(x, logit_rows)
             delta_rows = ops.gather_rows(delta, logit_rows) if delta is not None else None
-        h = self.final_norm.forward(ctx, rows, delta_rows)
+        # the head is a product like any other: it may take a norm that has not run
+        if self.final_norm.can_defer:
+            h = self.final_norm.forward(ctx, rows, delta_rows, defer=True)
+        else:
+            h = self.final_norm.forward(ctx, rows, delta_rows)
         logits = ops.linear(h, self.head_weight, self.head_bias, out_dtype=torch.float32)
         if spec.logit_scale != 1.0 or spec.logit_softcap is not None:
             ops.scale_softcap_(logits, spec.logit_scale, spec.logit_softcap)

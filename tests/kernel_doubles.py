@@ -51,7 +51,7 @@ class TorchOps:
         return (x[:, rows.long()] if x.dim() == 3 else x[rows.long()]).contiguous()
 
     # matrix products ---------------------------------------------------------------------
-    def linear(self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False):
+    def linear(self, x, weight, bias=None, out_dtype=None, kernel="auto", swiglu=False, partial_sums=False, for_stream=False):
         self._count("linear")
         y = x.float() @ weight.float().t()
         if bias is not None:

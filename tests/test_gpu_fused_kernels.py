@@ -234,3 +234,168 @@ def test_mixed_batches_and_single_partitions_do_not_defer(ops):
     assert isinstance(ops.paged_attention(q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, **kw), torch.Tensor)
     q, kp, vp, table, ctx, *_ = _paged_case([(600, 1), (500, 20)], 4, 2, 32, 16, torch.bfloat16, 105)
     assert isinstance(ops.paged_attention(q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, **kw), torch.Tensor)
+
+
+# ---- the product that finishes the residual stream, and the products that pay the norm it owes --------------
+def _wide_open(gpu_device):
+    """The kernels at every token count they take, not only where the engine chooses them."""
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    return HipOps(torch.bfloat16, gpu_device, tuning=KernelTuning(
+        finish_min_tokens=1, finish_max_tokens=64, finish_weight_bytes=1 << 30, finish_activation_bytes=1 << 30))
+
+
+_STREAM_SHAPES = [
+    (1, 64, 64), (3, 896, 896), (4, 132, 200), (5, 100, 72), (8, 896, 4864), (9, 896, 896), (12, 132, 200), (16, 260, 1032),
+    (17, 256, 512), (24, 100, 264), (32, 896, 896), (33, 64, 128), (50, 520, 264), (64, 896, 1024),
+]
+
+
+@pytest.mark.parametrize("m,n,k", _STREAM_SHAPES)
+@pytest.mark.parametrize("bias,weight_f32", [(None, False), ("f32", True), ("bf16", False)])
+def test_product_that_finishes_the_stream(gpu_device, m, n, k, bias, weight_f32):
+    """stream += a W^T + b in the product's own kernel (4, 8 or 16 features a workgroup, one to four
+    blocks of tokens), the next norm's activations short of their factor per row, and every row's sum
+    of squares in parts: each against float64; then the products that pay the factor (plain, SwiGLU)
+    against float64 and against the norm kernel followed by the same product."""
+    from mini_llm_runtime_amd.kernels.pending import PendingLinear, PendingScale
+
+    ops = _wide_open(gpu_device)
+    a = _rand((m, k), torch.bfloat16, 201, 0.7)
+    w = _rand((n, k), torch.bfloat16, 202, 0.1)
+    b = None if bias is None else _rand((n,), torch.float32 if bias == "f32" else torch.bfloat16, 203)
+    x = _rand((m, n), torch.float32, 204, 1.5)
+    nw = (1 + _rand((n,), torch.float32, 205, 0.1)).to(torch.float32 if weight_f32 else torch.bfloat16)
+    eps = 1e-5
+    new_stream = x.double() + a.double() @ w.double().t() + (0 if b is None else b.double())
+    pending = ops.linear(a.cuda(), w.cuda(), None if b is None else b.cuda(), for_stream=True)
+    assert isinstance(pending, PendingLinear)
+    xd = x.cuda()
+    owed = ops.defer_norm(xd, nw.cuda(), eps, pending)
+    assert isinstance(owed, PendingScale) and owed.residual is xd
+    torch.testing.assert_close(xd.cpu().double(), new_stream, atol=2e-4 * k**0.5, rtol=1e-5)
+    # h: the stream as the kernel left it times the weight, rounded once
+    expect_h = (nw.double() * xd.cpu().double()).float().to(torch.bfloat16)
+    torch.testing.assert_close(owed.h.cpu().float(), expect_h.float(), atol=0, rtol=2**-7)
+    assert float((owed.h.cpu() != expect_h).double().mean()) < 0.01
+    assert owed.sumsq.shape == (m, ops.lib.mlr_gemm_residual_parts(m, n))
+    torch.testing.assert_close(owed.sumsq.double().sum(1).cpu(), xd.cpu().double().pow(2).sum(1), atol=0, rtol=1e-5)
+    # the settled form is the plain norm of the stream
+    normed = plain.rms_norm(xd.cpu().double(), nw.double(), eps)
+    # consumers: y = normed W2^T + b2, the factor applied to the sums
+    n2 = 4 * (37 + m)
+    w2 = _rand((n2, n), torch.bfloat16, 206, 0.1)
+    b2 = _rand((n2,), torch.float32, 207)
+    scale = torch.rsqrt(xd.cpu().double().pow(2).mean(1, keepdim=True) + eps)
+    exact = (owed.h.cpu().double() * scale) @ w2.double().t()  # from the very activations the kernel read
+    got = ops.linear(owed, w2.cuda(), b2.cuda())
+    torch.testing.assert_close(got.cpu().double(), exact + b2.double(), atol=2e-2, rtol=1.6e-2)
+    torch.testing.assert_close(got.cpu().double(), normed @ w2.double().t() + b2.double(), atol=6e-2, rtol=3e-2)
+    wide = ops.linear(owed, w2.cuda(), b2.cuda(), out_dtype=torch.float32)
+    if n % 8 == 0:
+        torch.testing.assert_close(wide.cpu().double(), exact + b2.double(), atol=1e-3 * n**0.5, rtol=1e-4)
+    else:  # no matrix-core product at this width: the norm is settled by its own kernel, then the plain product
+        torch.testing.assert_close(wide.cpu().double(), normed @ w2.double().t() + b2.double(), atol=6e-2, rtol=3e-2)
+    two = ops.linear(ops.rmsnorm(xd.clone(), nw.cuda(), eps), w2.cuda(), b2.cuda())
+    torch.testing.assert_close(got.float(), two.float(), atol=6e-2, rtol=3e-2)
+    # the two ways round differently (weight * stream rounded, then scaled; or normed, then rounded): on
+    # average they stay within an ulp of bfloat16 (2^-7 of a value) of each other
+    assert float((got.float() - two.float()).abs().mean()) < 2.0**-7 * float(two.float().abs().mean())
+    glu = ops.linear(owed, w2.cuda(), None, swiglu=True)
+    quads = exact.view(m, -1, 4)
+    gate, up = quads[..., :2], quads[..., 2:]
+    torch.testing.assert_close(glu.cpu().double(), (gate * torch.sigmoid(gate) * up).reshape(m, -1), atol=2e-2, rtol=3e-2)
+    # every matrix-core kernel that takes these tokens pays the factor the same way
+    for kernel in (16, 14, 11, 12):
+        if (kernel == 16 and m > 16) or (kernel == 14 and m > 32) or n % 8:
+            continue
+        forced = ops.linear(owed, w2.cuda(), b2.cuda(), out_dtype=torch.float32, mfma_kernel=kernel)
+        torch.testing.assert_close(forced.cpu().double(), exact + b2.double(), atol=1e-3 * n**0.5, rtol=1e-4, msg=lambda s: f"kernel {kernel}: {s}")
+    # and cut along k, every slice scaled, the bias in the first
+    if n % 8 == 0 and n >= 128:
+        sliced = ops.linear(owed, w2.cuda(), b2.cuda(), partial_sums=True, slices=2)
+        torch.testing.assert_close(sliced.sum(0).cpu().double(), exact + b2.double(), atol=1e-3 * n**0.5, rtol=1e-4)
+    # settled, it is the norm kernel's own result
+    assert torch.equal(ops.settle(owed), ops.rmsnorm(xd.clone(), nw.cuda(), eps))
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,hidden,tokens", [
+    (4, 2, 16, 64, 3), (14, 2, 64, 896, 8), (14, 2, 64, 896, 5), (3, 1, 32, 96, 13), (6, 2, 48, 72, 30), (14, 2, 64, 896, 64),
+    (4, 1, 32, 128, 100), (14, 2, 64, 896, 300),
+])
+@pytest.mark.parametrize("rotate", [True, False])
+def test_query_key_value_product_pays_the_owed_norm(gpu_device, heads, kv_heads, head_dim, hidden, tokens, rotate):
+    """Every way of the query/key/value product (the row-splitting kernels with 8 and 16 rows, the tiled
+    one, product then rotation kernel, cut along k) on activations that still owe their factor per
+    row, against the float64 value computed from the very activations and sums of squares it read."""
+    from mini_llm_runtime_amd.kernels.pending import PendingScale
+
+    ops = _wide_open(gpu_device)
+    bs, pages = 8, max(9, tokens // 8 + 2)
+    width = (heads + 2 * kv_heads) * head_dim
+    h = _rand((tokens, hidden), torch.bfloat16, 211, 2.0).cuda()
+    parts = 7 if tokens % 2 else 70
+    sumsq = (torch.rand(tokens, parts, generator=torch.Generator().manual_seed(212)) * hidden * 3 / parts).cuda()
+    eps = 1e-6
+    w = _rand((width, hidden), torch.bfloat16, 213, 0.2).cuda()
+    b = _rand((width,), torch.float32, 214).cuda()
+    rotation = None
+    if rotate:
+        pos = torch.tensor(([3, 0, 911, 17, 40000] + list(range(5, tokens)))[:tokens], dtype=torch.int32).cuda()
+        inv = (1.0 / (1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))).cuda()
+        cos, sin = ops.rope_table(pos, inv)
+        rotation = (cos, sin, head_dim)
+    g = torch.Generator().manual_seed(215)
+    slots = torch.randperm(pages * bs, generator=g)[:tokens].to(torch.int32)
+    if tokens > 2:
+        slots[2] = -1
+    slots = slots.cuda()
+    factor = torch.rsqrt(sumsq.double().sum(1, keepdim=True).cpu() / hidden + eps)
+    # the kernel multiplies float32 sums by a float32 factor: one more rounding of 2^-24, inside e_sum's allowance
+    reference = qkv_reference(h.cpu().double() * factor, w, b, rotation[0] if rotate else None, rotation[1] if rotate else None,
+                              heads, kv_heads, head_dim)
+    ways = {"chosen": {}, "three kernels": dict(fused=False)}
+    if tokens <= 8:
+        ways["8 rows"] = dict(fused=True, mfma_kernel=8)
+    if tokens <= 64:
+        ways["16 rows"] = dict(fused=True, mfma_kernel=16)
+    ways["tiled"] = dict(fused=True, mfma_kernel=11)
+    if tokens <= 128 and hidden >= 512 and rotate:
+        ways["cut along k"] = dict(sliced=True)
+    for name, kw in ways.items():
+        owed = PendingScale(h, sumsq, torch.ones(hidden, dtype=torch.bfloat16).cuda(), eps, torch.zeros(tokens, hidden).cuda())
+        kp = torch.full((pages, kv_heads, bs, head_dim), float("nan"), dtype=torch.bfloat16).cuda()
+        vp = torch.full((pages, kv_heads, head_dim, bs), float("nan"), dtype=torch.bfloat16).cuda()
+        q = ops.qkv_rope_write(owed, w, b, rotation, slots, kp, vp, num_heads=heads, num_kv_heads=kv_heads,
+                               head_dim=head_dim, block_size=bs, **kw)
+        check_qkv(name, q.float().cpu(), kp.float().cpu(), vp.float().cpu(), slots, bs, reference, heads, kv_heads, head_dim)
+
+
+def test_stream_finishing_product_is_used_where_it_pays(gpu_device):
+    """By default only small matrices at 5 to 8 tokens go that way; everything else keeps the product
+    cut along k and the norm kernel.  A product that is not taken that way, or that meets a norm which
+    cannot run it, comes out as before."""
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+    from mini_llm_runtime_amd.kernels.pending import PendingLinear
+
+    ops = HipOps(torch.bfloat16, gpu_device)
+    w_small = _rand((896, 896), torch.bfloat16, 221, 0.1).cuda()
+    w_large = _rand((896, 4864), torch.bfloat16, 222, 0.1).cuda()
+    for m, expect in ((1, False), (4, False), (5, True), (8, True), (9, False), (64, False)):
+        out = ops.linear(_rand((m, 896), torch.bfloat16, 223).cuda(), w_small, None, for_stream=True)
+        assert isinstance(out, PendingLinear) == expect, m
+    assert not isinstance(ops.linear(_rand((8, 4864), torch.bfloat16, 224).cuda(), w_large, None, for_stream=True), PendingLinear)
+    assert not isinstance(HipOps(torch.float32, gpu_device).linear(torch.zeros(8, 64).cuda(), torch.zeros(64, 64).cuda(), None, for_stream=True), PendingLinear)
+    # a pending product that reaches the plain norm, an addition or a gather is run as a product of its own
+    a = _rand((6, 896), torch.bfloat16, 225).cuda()
+    pending = ops.linear(a, w_small, None, for_stream=True)
+    assert isinstance(pending, PendingLinear)
+    x = _rand((6, 896), torch.float32, 226).cuda()
+    nw = torch.ones(896, dtype=torch.bfloat16).cuda()
+    direct = ops.rmsnorm(x.clone(), nw, 1e-6, delta=ops.linear(a, w_small, None, partial_sums=True))
+    assert torch.equal(ops.rmsnorm(x.clone(), nw, 1e-6, delta=pending), direct)
+    rows = torch.tensor([4, 1], dtype=torch.int32).cuda()
+    picked = ops.gather_rows(pending, rows)
+    assert isinstance(picked, PendingLinear) and picked.shape == (2, 896)
+    torch.testing.assert_close(ops.settle(picked).float().sum(0) if ops.settle(picked).dim() == 3 else ops.settle(picked).float(),
+                               (a[rows.long()].float() @ w_small.float().t()), atol=3e-2, rtol=2e-2)
