@@ -115,9 +115,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
     for (int i = 0; i < 4; ++i) red[wave][mt][lane][i] = acc[mt][i];
   if (ep.row_sumsq != nullptr) row_scales_finish(ep, owed, 0, min(M, MT * 16), M, K, scales);
   __syncthreads();
-  if (wave != 0) return;
+  // Slab mt is finished by wavefront mt % WAVES: the epilogue of a slab waits for memory more than once
+  // (rotation tables, cache slots, the stores), and one wavefront doing four slabs in turn was a third
+  // of the kernel's time at 64 tokens.
+  if (wave >= MT) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
+    if (mt % WAVES != wave) continue;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
@@ -661,8 +665,16 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
 // rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 12 = gemm_tiled with tiles of 64
 // tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products.
+// A small matrix (an output projection of a narrow model) at 17 to 64 tokens: the tiled kernels have
+// too few tiles of it to keep the compute units busy, the row-splitting kernel with its 16 features a
+// workgroup has four times as many workgroups (0.5B output projection with the norm behind it, in a
+// replayed graph: 32 tokens 9.0 us tiled in 2 slices, 6.4 row-splitting in 4; 64 tokens 9.4 and 7.3).
+// Larger matrices read the tokens too often that way (0.5B gate-up at 64 tokens: 10 us tiled, 16).
+static bool small_matrix(int n, int k) { return static_cast<int64_t>(n) * k * 2 <= (4ll << 20); }
+
 static int choose_kernel(int m, int n, int k, int slices) {
   if (m <= 16 && !few_tokens_tiled(n, slices)) return 16;
+  if (m <= 64 && small_matrix(n, k)) return 16;
   if (m <= 32) return 14;
   // 33 to 64 tokens: tiles of 128 features read the tokens half as often per weight byte and stream
   // faster once there are enough of them (32B gate-up at 64 tokens, 432 tiles: 128 to 103 us; the 7B
@@ -676,12 +688,14 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
                      int kernel, hipStream_t stream) {
   switch (kernel) {
     case 16: {
-      if (m > 16) {
-        set_error("mlr_gemm_bf16: the streaming kernel takes up to 16 tokens");
+      if (m > 64) {
+        set_error("mlr_gemm_bf16: the streaming kernel takes up to 64 tokens");
         return -1;
       }
       dim3 grid((n + 15) / 16, slices);
-      gemm_skinny_split_kernel<4, false, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
+      if (m <= 16) gemm_skinny_split_kernel<4, false, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
+      else if (m <= 32) gemm_skinny_split_kernel<4, false, 2><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
+      else gemm_skinny_split_kernel<4, false, 4><<<grid, 256, 0, stream>>>(xb, wb, ep, QkvTarget{}, m, n, k);
       return 0;
     }
     case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
@@ -721,6 +735,9 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
     const int by_fill = choose_slices((n + 15) / 16, (k / 8 + 3) / 4, min(max_slices, 8), 512);
     return max(by_fill, min(min(4, max_slices), k / 2560));
   }
+  // 17 to 64 tokens of a small matrix: the row-splitting kernel (see choose_kernel) cut into 4 where
+  // every slice keeps a few steps of k
+  if (small_matrix(n, k)) return (k / 8 + 3) / 4 >= 16 ? min(4, max_slices) : 1;
   // 17 to 64 tokens: the small tiles keep few bytes in flight each, so two workgroups per compute
   // unit before the cutting stops (32B down at 32 tokens: 320 workgroups 65 us, 640 workgroups 56 us)
   return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 8), 512);

@@ -243,8 +243,35 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     total = got.cpu().double().sum(0) if slices > 1 else got.cpu().double()
     torch.testing.assert_close(total, ref, atol=2e-3, rtol=1e-4)
     if kernel != 16:
-        with pytest.raises(Exception, match="16 tokens"):
+        with pytest.raises(Exception, match="64 tokens"):
             ops.linear(x.cuda(), w.cuda(), mfma_kernel=16)
+
+
+@pytest.mark.parametrize("m", [17, 31, 32, 33, 50, 64])
+@pytest.mark.parametrize("slices", [1, 4])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_row_splitting_kernel_takes_up_to_64_tokens(ops_for, m, slices, swiglu):
+    """The streaming kernel with two and four slabs of 16 tokens (chosen for small matrices, forced
+    here at a width that is no multiple of its 16 rows), whole, cut along k, and with SwiGLU."""
+    if swiglu and slices > 1:
+        pytest.skip("partial sums have no SwiGLU")
+    ops = ops_for(torch.bfloat16)
+    n, k = 204, 904
+    x = _rand((m, k), torch.bfloat16, 64)
+    w = _rand((n, k), torch.bfloat16, 65, 0.05)
+    b = None if swiglu else _rand((n,), torch.float32, 66)
+    ref = x.double() @ w.double().t() + (0 if b is None else b.double())
+    if swiglu:
+        quads = ref.view(m, -1, 4)
+        ref = (quads[..., :2] * torch.sigmoid(quads[..., :2]) * quads[..., 2:]).reshape(m, -1)
+    got = ops.linear(x.cuda(), w.cuda(), None if b is None else b.cuda(), out_dtype=torch.float32, partial_sums=slices > 1,
+                     mfma_kernel=16, slices=slices, swiglu=swiglu)
+    total = got.cpu().double().sum(0) if slices > 1 else got.cpu().double()
+    torch.testing.assert_close(total, ref, atol=2e-3, rtol=1e-4)
+    # and by itself for a small matrix: the same values as when forced
+    if not swiglu:
+        chosen = ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32)
+        assert torch.equal(chosen, ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, mfma_kernel=16))
 
 
 # ---- rotary encoding and cache write ----------------------------------------------------------------
