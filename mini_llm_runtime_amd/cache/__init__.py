@@ -2,7 +2,8 @@
 
 from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
 from .manager import CacheManager, CacheStats, KVGroup, RequestCache, StepLayout, VisibilityError
-from .spec import PagedKVSpec, SlotStateSpec
+from .spec import PagedKVSpec, PagedSpec, SiteCacheSpec, SlotSpec, SlotStateSpec
+from .views import KVView, StateView
 
 __all__ = [
     "BlockAllocator",
@@ -10,7 +11,12 @@ __all__ = [
     "CacheManager",
     "CacheStats",
     "KVGroup",
+    "KVView",
     "PagedKVSpec",
+    "PagedSpec",
+    "SiteCacheSpec",
+    "SlotSpec",
+    "StateView",
     "RequestCache",
     "SlotPool",
     "SlotStateSpec",

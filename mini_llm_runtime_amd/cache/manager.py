@@ -14,11 +14,10 @@ Beyond the reference: several groups (each with pages and a free list of its
 own), windows (pages that every later query has passed are given back at
 commit), capacity promised by count instead of by pinning pages, and state slots.
 
-Page layout: keys [site, page, kv_head, offset in page, head_dim], the reference's
-inner order (src/mini_llm_runtime/paged_kv_cache.py:287-318); values are kept
-transposed inside a page, [site, page, kv_head, head_dim, offset in page], because
-the matrix cores want the index that is summed over (the key position, for the
-probability-times-value product) to be the fastest one of both operands.
+What lives in a page, and in which order, is the business of the sites' cache specs
+(`cache/spec.py`): the manager counts pages, rows and tokens and never asks what kind a
+spec is.  A spec attaches its site to one of the two stores (`add_paged_site`,
+`add_slot_site`), brings the tensors, and makes the view a mixer is handed.
 """
 
 from __future__ import annotations
@@ -30,24 +29,19 @@ import numpy as np
 import torch
 
 from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
-from .spec import PagedKVSpec, SlotStateSpec
+from .spec import PagedSpec, SiteCacheSpec, SlotSpec
 
-SiteSpec = Union[PagedKVSpec, SlotStateSpec, None]
-
-_TORCH_DTYPES = {
-    "float32": torch.float32,
-    "bfloat16": torch.bfloat16,
-    "int32": torch.int32,
-}
+SiteSpec = Optional[SiteCacheSpec]
 
 
 class KVGroup:
-    """Execution sites whose caches have the same shape and window share one pool."""
+    """Execution sites whose paged caches have equal specs share one pool: the tensors the spec
+    makes (each [sites, pages, ...]) and one free list."""
 
     def __init__(
         self,
         index: int,
-        spec: PagedKVSpec,
+        spec: PagedSpec,
         sites: Sequence[int],
         num_blocks: int,
         block_size: int,
@@ -60,12 +54,23 @@ class KVGroup:
         self.site_position = {site: i for i, site in enumerate(self.sites)}
         self.allocator = BlockAllocator(num_blocks)
         self.block_size = block_size
-        shape = (len(self.sites), num_blocks, spec.num_kv_heads, block_size, spec.head_dim)
-        # never zeroed: stale bytes must be unreachable, not clean
-        self.key = torch.empty(shape, dtype=dtype, device=device)
-        self.value = torch.empty(
-            (len(self.sites), num_blocks, spec.num_kv_heads, spec.value_dim, block_size), dtype=dtype, device=device
-        )
+        self.tensors: dict[str, torch.Tensor] = dict(spec.page_tensors(len(self.sites), num_blocks, block_size, dtype, device))
+        for name, t in self.tensors.items():
+            if t.dim() < 2 or tuple(t.shape[:2]) != (len(self.sites), num_blocks):
+                raise ValueError(f"pool tensor {name!r} must be [sites, pages, ...], got {tuple(t.shape)}")
+
+    @property
+    def key(self) -> Optional[torch.Tensor]:
+        return self.tensors.get("key")
+
+    @property
+    def value(self) -> Optional[torch.Tensor]:
+        return self.tensors.get("value")
+
+    def pages_of(self, site: int) -> dict[str, torch.Tensor]:
+        """One site's share of the pool's tensors, each [pages, ...]."""
+        i = self.site_position[site]
+        return {name: t[i] for name, t in self.tensors.items()}
 
     @property
     def num_blocks(self) -> int:
@@ -89,7 +94,7 @@ class KVGroup:
         return min(full, bounded)
 
     def storage_bytes(self) -> int:
-        return (self.key.numel() + self.value.numel()) * self.key.element_size()
+        return sum(t.numel() * t.element_size() for t in self.tensors.values())
 
 
 class StateBank:
@@ -97,10 +102,12 @@ class StateBank:
     writes the other, commit swaps them, so an aborted step changes nothing.  Two spare rows
     behind them belong to nobody: the padded entries of a recorded step read and write those."""
 
-    def __init__(self, site: int, spec: SlotStateSpec, num_slots: int, device: torch.device) -> None:
+    def __init__(self, site: int, spec: SlotSpec, num_slots: int, device: torch.device) -> None:
         self.site = site
         self.spec = spec
-        self.tensor = torch.zeros((num_slots * 2 + 2, *spec.shape), dtype=_TORCH_DTYPES[spec.dtype], device=device)
+        self.tensor = spec.bank(num_slots * 2 + 2, device)
+        if self.tensor.shape[0] != num_slots * 2 + 2:
+            raise ValueError("a state bank must have two rows per request slot and two spare ones")
 
 
 @dataclass
@@ -227,10 +234,13 @@ class CacheManager:
         self.device = torch.device(device)
         self.site_specs = tuple(site_specs)
 
-        grouped: dict[PagedKVSpec, list[int]] = {}
+        # every spec attaches its site to one of the two stores
+        self._paged_sites: dict[PagedSpec, list[int]] = {}
+        self.state_banks: dict[int, StateBank] = {}
         for site, spec in enumerate(self.site_specs):
-            if isinstance(spec, PagedKVSpec):
-                grouped.setdefault(spec, []).append(site)
+            if spec is not None:
+                spec.attach(self, site)
+        grouped = self._paged_sites
         counts = [num_blocks] * len(grouped) if isinstance(num_blocks, int) else list(num_blocks)
         if len(counts) != len(grouped):
             raise ValueError(f"num_blocks names {len(counts)} pools, the model has {len(grouped)} groups")
@@ -239,11 +249,6 @@ class CacheManager:
             for i, (spec, sites) in enumerate(grouped.items())
         ]
         self._site_group: dict[int, KVGroup] = {s: g for g in self.groups for s in g.sites}
-        self.state_banks: dict[int, StateBank] = {
-            site: StateBank(site, spec, self.max_requests, self.device)
-            for site, spec in enumerate(self.site_specs)
-            if isinstance(spec, SlotStateSpec)
-        }
         self.slots = SlotPool(self.max_requests)
         self._requests: dict[str, RequestCache] = {}
         self._pending: Optional[list[_PendingEntry]] = None
@@ -269,15 +274,45 @@ class CacheManager:
         except KeyError:
             raise KeyError(f"unknown request {request_id!r}") from None
 
+    # ---- what the specs call -------------------------------------------------------------------
+    def add_paged_site(self, site: int, spec: PagedSpec) -> None:
+        """`site` keeps something per token in pages; sites with equal specs share a pool."""
+        self._paged_sites.setdefault(spec, []).append(site)
+
+    def add_slot_site(self, site: int, spec: SlotSpec) -> None:
+        """`site` keeps a state of fixed size per request."""
+        self.state_banks[site] = StateBank(site, spec, self.max_requests, self.device)
+
     def group_of_site(self, site: int) -> KVGroup:
         return self._site_group[site]
 
     def site_pools(self, site: int) -> tuple[torch.Tensor, torch.Tensor, int]:
-        """(key pages [page, kv_head, offset, head_dim], value pages [page, kv_head, head_dim, offset],
-        group index) of one site."""
+        """(key pages, value pages, group index) of one site with keys and values in pages."""
         group = self._site_group[site]
-        i = group.site_position[site]
-        return group.key[i], group.value[i], group.index
+        pages = group.pages_of(site)
+        return pages["key"], pages["value"], group.index
+
+    def site_view(self, site: int, owner: int, block_tables, slot_mappings, state_read, state_write):
+        """What the mixer at execution site `site` is handed of the cache that site `owner` keeps
+        (its own, or an earlier site's that it only reads), for a step whose metadata is given per
+        pool (block tables, slot mappings) and per entry (state rows); None when `owner` keeps nothing.
+        The view is made by the owner's spec."""
+        group = self._site_group.get(owner)
+        if group is not None:
+            return group.spec.view(
+                group.pages_of(owner),
+                block_table=block_tables[group.index],
+                slot_mapping=slot_mappings[group.index],
+                block_size=self.block_size,
+                writable=site == owner,
+                site=site,
+                owner=owner,
+                tracker=self.visibility_tracker,
+            )
+        bank = self.state_banks.get(owner)
+        if bank is not None:
+            return bank.spec.view(bank.tensor, state_read, state_write)
+        return None
 
     @property
     def step_in_flight(self) -> bool:
@@ -574,5 +609,6 @@ class CacheManager:
     def poison(self) -> None:
         """Fill every page with NaN so that a read of an unwritten slot shows (tests)."""
         for g in self.groups:
-            g.key.fill_(float("nan"))
-            g.value.fill_(float("nan"))
+            for t in g.tensors.values():
+                if t.is_floating_point():
+                    t.fill_(float("nan"))

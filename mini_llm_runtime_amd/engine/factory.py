@@ -10,7 +10,6 @@ from typing import Any, Optional, Sequence, Union
 import torch
 
 from ..cache.manager import CacheManager
-from ..cache.spec import PagedKVSpec
 from ..config.model_config import ModelConfig
 from ..models.registry import build_model, load_config
 from ..parts.model import DecoderModel
@@ -67,8 +66,8 @@ def page_bytes(model: DecoderModel, block_size: int, dtype: torch.dtype) -> int:
     width = torch.empty((), dtype=dtype).element_size()
     total = 0
     for spec in model.site_cache_specs():
-        if isinstance(spec, PagedKVSpec):
-            total += spec.bytes_per_token(width) * block_size
+        if spec is not None:
+            total += spec.page_bytes(block_size, width)  # 0 for what does not live in pages
     return total
 
 

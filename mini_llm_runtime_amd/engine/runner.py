@@ -23,8 +23,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, StepLayout
-from ..cache.spec import PagedKVSpec, SlotStateSpec
-from ..parts.context import KVView, MixerPlan, PlanInput, StateView, StepContext
+from ..parts.context import MixerPlan, PlanInput, StepContext
 from ..parts.model import DecoderModel
 
 
@@ -257,25 +256,13 @@ class ModelRunner:
                 fields[name] = view(at)
                 at += 1
             ctx.plans[plan.key] = SimpleNamespace(**fields)
+        # every site's view is made by the spec of the site whose cache it uses: the step function
+        # does not know what kinds of cache there are
         for site in range(self.model.num_sites):
             source = self.model.cache_site_of(site)
-            spec = self.cache.site_specs[source]
-            if isinstance(spec, PagedKVSpec):
-                key, value, g = self.cache.site_pools(source)
-                ctx.kv_views[site] = KVView(
-                    key=key,
-                    value=value,
-                    block_table=tables[g],
-                    slot_mapping=slot_maps[g],
-                    block_size=self.cache.block_size,
-                    window=spec.window,
-                    writable=source == site,
-                    site=site,
-                    owner=source,
-                    tracker=self.cache.visibility_tracker,
-                )
-            elif isinstance(spec, SlotStateSpec):
-                ctx.state_views[site] = StateView(self.cache.state_banks[source].tensor, state_read, state_write)
+            view = self.cache.site_view(site, source, tables, slot_maps, state_read, state_write)
+            if view is not None:
+                ctx.site_views[site] = view
         return ctx
 
     def _stage(self, arrays: list[np.ndarray]):
@@ -293,7 +280,7 @@ class ModelRunner:
         site_outputs: Optional[list] = None,
     ) -> Optional[torch.Tensor]:
         longest = int(layout.context_lens.max())
-        plans = self._plans(PlanInput(layout.q_lens, layout.q_starts, longest))
+        plans = self._plans(PlanInput(layout.q_lens, layout.q_starts, longest, layout, token_ids))
         host, spans = self._stage(self._arrays(layout, token_ids, logit_rows, plans))
         dev = host.to(self.device, non_blocking=True)
         ctx = self._context(
@@ -339,13 +326,13 @@ class ModelRunner:
             stacklevel=3,
         )
 
-    def _step_key(self, layout: StepLayout, logit_rows: np.ndarray) -> Optional[tuple]:
+    def _step_key(self, layout: StepLayout, logit_rows: np.ndarray, token_ids: Optional[np.ndarray] = None) -> Optional[tuple]:
         """(identity of a recording, the plans it was derived from): the sizes that fix every launch
         of a step; None when such steps are not recorded."""
         if not self._recordable() or layout.num_tokens > self.max_graph_tokens:
             return None
         width = self._table_width(layout)
-        plans = self._plans(PlanInput(layout.q_lens, layout.q_starts, width * self.cache.block_size))
+        plans = self._plans(PlanInput(layout.q_lens, layout.q_starts, width * self.cache.block_size, layout, token_ids))
         key = ("step", layout.num_tokens, layout.num_entries, width, int(logit_rows.size), self._plan_sizes(plans))
         return key, plans
 
@@ -431,12 +418,16 @@ class ModelRunner:
             slot[2].synchronize()  # the copy that last read this buffer
         return slot
 
-    def _padded_plans(self, padded: int, width: int, q_starts: Optional[np.ndarray] = None) -> list[MixerPlan]:
+    def _padded_plans(
+        self, padded: int, width: int, layout: Optional[StepLayout] = None, token_ids: Optional[np.ndarray] = None
+    ) -> list[MixerPlan]:
         """Plans of a batch of `padded` single tokens whose contexts fit `width` pages."""
         starts = np.zeros(padded, dtype=np.int32)
-        if q_starts is not None:
-            starts[: len(q_starts)] = q_starts
-        return self._plans(PlanInput(np.ones(padded, dtype=np.int32), starts, width * self.cache.block_size))
+        if layout is not None:
+            starts[: len(layout.q_starts)] = layout.q_starts
+        return self._plans(
+            PlanInput(np.ones(padded, dtype=np.int32), starts, width * self.cache.block_size, layout, token_ids)
+        )
 
     def _fill_padded(self, views, layout: StepLayout, token_ids: np.ndarray, graph) -> None:
         """`_arrays(..., pad_entries, table_width)` written into the views of a staging buffer.
@@ -464,7 +455,7 @@ class ModelRunner:
             table[count:] = -1
         padded, width, sizes, has_plan_arrays = graph[5]
         if has_plan_arrays:  # plans whose arrays depend on the step's data are made again
-            plans = self._padded_plans(padded, width, layout.q_starts)
+            plans = self._padded_plans(padded, width, layout, token_ids)
             if self._plan_sizes(plans) != sizes:
                 raise RuntimeError("a mixer's plan for a batch of single tokens changed its sizes between steps")
             at = first + 2 * groups
@@ -479,7 +470,7 @@ class ModelRunner:
         padded, width = key
         graph = self._graphs.pop(key, None)
         if graph is None:
-            plans = self._padded_plans(padded, width, layout.q_starts)
+            plans = self._padded_plans(padded, width, layout, token_ids)
             arrays = self._arrays(layout, token_ids, logit_rows, plans, padded, width)
             buf, spans = _pack_int32(arrays)
             slot = self._graph_staging(key, spans, buf.size)
@@ -611,7 +602,7 @@ class ModelRunner:
             elif capture_sites:
                 logits = self._forward_eager(layout, token_ids, logit_rows, captured)
             else:
-                keyed = self._step_key(layout, logit_rows)
+                keyed = self._step_key(layout, logit_rows, token_ids)
                 seen = 0
                 if keyed is not None:
                     seen = self._step_seen[keyed[0]] = self._step_seen.get(keyed[0], 0) + 1

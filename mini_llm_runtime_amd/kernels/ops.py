@@ -793,8 +793,6 @@ class HipOps:
             and block_size % 4 == 0
             and stride % 8 == 0
         )
-        if plan is None:
-            plan = ctx  # callers that keep the plan's fields on the batch description itself
         num_tiles = int(getattr(plan, "num_query_tiles", 0))
         num_decode = int(getattr(plan, "num_decode_entries", 0))
         if use_mfma and num_tiles + num_decode == 0:

@@ -11,6 +11,9 @@ from typing import Any, Optional
 import numpy as np
 import torch
 
+from ..cache.views import KVView, StateView  # noqa: F401  (part of this module's surface)
+
+
 @dataclass(frozen=True)
 class PlanInput:
     """What a mixer may look at when it plans its kernels for a step: the new tokens and the
@@ -20,6 +23,13 @@ class PlanInput:
     q_lens: np.ndarray  # [R] tokens of this step
     q_starts: np.ndarray  # [R] tokens cached before it
     max_context: int
+    # The step itself, for plans that need more than its shape: the cache manager's `StepLayout` (host
+    # arrays: request ids and slots, positions, block tables and slot mappings per pool, state rows) and
+    # the token ids.  Both are None when only a shape exists (the probe when a runner is built).  For a
+    # recorded step of single tokens, padded to a power of two, they describe the real entries while
+    # q_lens and q_starts are padded.
+    layout: Any = None
+    token_ids: Optional[np.ndarray] = None
 
 
 @dataclass
@@ -32,46 +42,6 @@ class MixerPlan:
     key: Any
     arrays: dict  # name -> np.ndarray (int32)
     sizes: dict  # name -> int
-
-
-@dataclass
-class KVView:
-    """Pages of one site: keys [page, kv_head, offset, head_dim], values
-    [page, kv_head, head_dim, offset], the block table rows of the step's entries
-    and the slot of each new token."""
-
-    key: torch.Tensor
-    value: torch.Tensor
-    block_table: torch.Tensor  # [R, max pages] int32, -1 where there is no page
-    slot_mapping: torch.Tensor  # [T] int32: page * block_size + offset
-    block_size: int
-    window: Optional[int]
-    writable: bool  # False when the site reads another site's cache
-    site: int = -1  # the execution site this view was made for
-    owner: int = -1  # the site that owns the pages (== site when writable)
-    tracker: Any = None  # the cache manager's visibility check, when it is switched on
-
-    def written(self) -> None:
-        """The mixer reports that it has stored the step's keys and values of this site."""
-        if self.tracker is not None:
-            self.tracker.note_write(self.site, self.owner)
-
-    def reading(self) -> None:
-        """The mixer reports that it is about to read this site's pages, the step's own
-        tokens included.  With the check switched on this raises unless the owning site
-        has written them."""
-        if self.tracker is not None:
-            self.tracker.note_read(self.site, self.owner)
-
-
-@dataclass
-class StateView:
-    """Fixed-size state of one site: read rows `read_rows`, write rows `write_rows`
-    of `tensor` ([2 * slots, ...]); the manager swaps them at commit."""
-
-    tensor: torch.Tensor
-    read_rows: torch.Tensor  # [R] int32
-    write_rows: torch.Tensor  # [R] int32
 
 
 @dataclass
@@ -91,8 +61,7 @@ class StepContext:
     max_context_len: int
     host: Any  # the StepLayout (numpy arrays) for parts that work on the host; None while a step is recorded
     logits_for_all: bool = False  # the wanted rows are all tokens, in order: no gather needed
-    kv_views: dict[int, KVView] = field(default_factory=dict)
-    state_views: dict[int, StateView] = field(default_factory=dict)
+    site_views: dict[int, Any] = field(default_factory=dict)  # execution site -> what its cache spec made for this step
     plans: dict[Any, Any] = field(default_factory=dict)  # MixerPlan.key -> its sizes and device arrays, as attributes
     memo: dict[Any, Any] = field(default_factory=dict)
 
@@ -101,8 +70,21 @@ class StepContext:
         the plan's sizes and, as device tensors, its arrays."""
         return self.plans.get(key)
 
+    def cache(self, site: int) -> Any:
+        """The view of the cache that execution site `site` uses in this step, as its spec made it."""
+        return self.site_views[site]
+
     def kv(self, site: int) -> KVView:
-        return self.kv_views[site]
+        return self.site_views[site]
 
     def state(self, site: int) -> StateView:
-        return self.state_views[site]
+        return self.site_views[site]
+
+    # the views by the names they had when there were two kinds
+    @property
+    def kv_views(self) -> dict[int, Any]:
+        return self.site_views
+
+    @property
+    def state_views(self) -> dict[int, Any]:
+        return self.site_views

@@ -11,7 +11,6 @@ from typing import Iterator, Mapping, Optional
 
 import torch
 
-from ..cache.spec import PagedKVSpec, SlotStateSpec
 from .base import Block, Part
 from .context import StepContext
 from .registry import build_part
@@ -181,12 +180,3 @@ class DecoderModel:
         if spec.logit_scale != 1.0 or spec.logit_softcap is not None:
             ops.scale_softcap_(logits, spec.logit_scale, spec.logit_softcap)
         return logits
-
-
-def site_spec_kinds(model: DecoderModel) -> tuple[int, int]:
-    """(sites with paged keys and values, sites with fixed-size state)."""
-    specs = model.site_cache_specs()
-    return (
-        sum(isinstance(s, PagedKVSpec) for s in specs),
-        sum(isinstance(s, SlotStateSpec) for s in specs),
-    )

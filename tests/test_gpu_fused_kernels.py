@@ -11,7 +11,7 @@ import plain_qwen2 as plain
 from mini_llm_runtime_amd.kernels.pending import PendingMerge, PendingNorm
 from mini_llm_runtime_amd.kernels.tuning import KernelTuning
 from qkv_reference import check_qkv, qkv_reference
-from test_gpu_kernels import _attention_reference, _paged_case, _rand, _tol
+from test_gpu_kernels import _attend, _attention_reference, _paged_case, _rand, _tol
 
 pytestmark = pytest.mark.gpu
 
@@ -190,9 +190,9 @@ def test_merge_as_the_prologue_of_the_output_product(ops, heads, kv_heads, head_
     bo = _rand((hidden,), torch.float32, 101).cuda()
     args = (q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx)
     kw = dict(num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=16, scale=scale, window=window)
-    pending = tuned.paged_attention(*args, defer_merge=True, **kw)
+    pending = _attend(tuned, *args, defer_merge=True, **kw)
     assert isinstance(pending, PendingMerge) and pending.splits > 1
-    attended = tuned.paged_attention(*args, **kw)
+    attended = _attend(tuned, *args, **kw)
     ref_att = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, window)
     torch.testing.assert_close(attended.cpu().double(), ref_att, **_tol(torch.bfloat16))
     assert torch.equal(tuned.settle(pending), attended), "the merge on its own gives what the attention call gives"
@@ -220,7 +220,7 @@ def test_merge_prologue_keeps_the_poison_of_a_missing_page(ops):
     q, kp, vp, table, ctx, *_ = _paged_case(entries, 4, 2, 32, 16, torch.bfloat16, 102)
     table[1, 3] = -1
     wo = _rand((40, 128), torch.bfloat16, 103, 0.1).cuda()
-    pending = ops.paged_attention(q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, num_heads=4, num_kv_heads=2,
+    pending = _attend(ops, q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, num_heads=4, num_kv_heads=2,
                                   head_dim=32, block_size=16, scale=0.2, window=None, defer_merge=True)
     assert isinstance(pending, PendingMerge)
     out = ops.linear(pending, wo, None).float().cpu()
@@ -231,9 +231,9 @@ def test_mixed_batches_and_single_partitions_do_not_defer(ops):
     """Only a batch of single tokens whose keys are cut into partitions defers its merge."""
     kw = dict(num_heads=4, num_kv_heads=2, head_dim=32, block_size=16, scale=0.2, window=None, defer_merge=True)
     q, kp, vp, table, ctx, *_ = _paged_case([(40, 1), (30, 1)], 4, 2, 32, 16, torch.bfloat16, 104)
-    assert isinstance(ops.paged_attention(q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, **kw), torch.Tensor)
+    assert isinstance(_attend(ops, q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, **kw), torch.Tensor)
     q, kp, vp, table, ctx, *_ = _paged_case([(600, 1), (500, 20)], 4, 2, 32, 16, torch.bfloat16, 105)
-    assert isinstance(ops.paged_attention(q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, **kw), torch.Tensor)
+    assert isinstance(_attend(ops, q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx, **kw), torch.Tensor)
 
 
 # ---- the product that finishes the residual stream, and the products that pay the norm it owes --------------

@@ -39,6 +39,12 @@ def ops_for(gpu_device):
     return get
 
 
+def _attend(ops, *args, **kw):
+    """`paged_attention` with the launch plan that these tests keep on the batch description itself."""
+    kw.setdefault("plan", args[4])
+    return ops.paged_attention(*args, **kw)
+
+
 def _rand(shape, dtype, seed, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(shape, generator=g) * scale).to(dtype)
@@ -609,7 +615,8 @@ def test_paged_attention_mixed_batch(ops_for, dtype, heads, kv_heads, head_dim, 
     entries = [(1, 1), (bs, 1), (bs + 1, 1), (37, 37), (70, 5), (4 * bs + 1, 2), (130, 1), (2 * bs, bs)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 21)
     scale = head_dim**-0.5
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
     ).cpu()
@@ -645,7 +652,8 @@ def _wide_ops():
 
 def _check_window(ops, dtype, window, heads, kv_heads, head_dim, bs, entries):
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 22)
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=0.2, window=window,
     ).cpu()
@@ -661,7 +669,8 @@ def test_paged_attention_far_key_among_hundreds(ops_for, dtype):
     entries = [(700, 1), (515, 3), (2049, 1)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, dtype, 23, spike=True)
     scale = head_dim**-0.5
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
     ).cpu()
@@ -687,7 +696,8 @@ def test_paged_attention_merge_needs_global_weights(ops_for):
     q[0, 0] = 1.0
     ctx = _plan([(5, 1)], [0], [4])
     table = torch.tensor([[0, 1]], dtype=torch.int32)
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=1, num_kv_heads=1, head_dim=16, block_size=bs, scale=1.0, window=None,
     ).cpu()
@@ -700,7 +710,8 @@ def test_paged_attention_bad_page_poisons(ops_for):
     entries = [(20, 1)]
     q, kp, vp, table, ctx, *_ = _paged_case(entries, 2, 1, 16, 8, torch.float32, 24)
     table[0, 1] = -1
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=2, num_kv_heads=1, head_dim=16, block_size=8, scale=0.25, window=None,
     ).cpu()
@@ -712,7 +723,8 @@ def test_attention_matches_library_special_case(ops_for):
     ops = ops_for(torch.float32)
     heads, head_dim, bs, n = 3, 32, 8, 29
     q, kp, vp, table, ctx, dense, te, pos = _paged_case([(n, n)], heads, heads, head_dim, bs, torch.float32, 25)
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=heads, head_dim=head_dim, block_size=bs, scale=head_dim**-0.5, window=None,
     ).cpu()
@@ -737,8 +749,8 @@ def test_decode_attention_partitions(ops_for, heads, kv_heads, head_dim, partiti
         scale = head_dim**-0.5
         args = (q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx)
         kw = dict(num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=16, scale=scale, window=None)
-        got = ops.paged_attention(*args, **kw).cpu()
-        fma = ops.paged_attention(*args, kernel="fma", **kw).cpu()
+        got = _attend(ops, *args, **kw).cpu()
+        fma = _attend(ops, *args, kernel="fma", **kw).cpu()
     finally:
         ops.decode_partition = old
     ref = _attention_reference(q, dense, te, pos, heads, kv_heads, head_dim, scale, None)
@@ -759,7 +771,8 @@ def test_prefill_attention_long_prompt_and_portion(ops_for, heads, kv_heads, hea
     entries = [(long, long), (long - 250, 300), (77, 77)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 27, spike=True)
     scale = head_dim**-0.5
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
     ).cpu()
@@ -779,7 +792,8 @@ def test_prompt_portions_behind_long_contexts_in_key_runs(ops_for, heads, kv_hea
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 43, spike=True)
     assert ctx.long_prefix == 2
     scale = head_dim**-0.5
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
     ).cpu()
@@ -797,7 +811,8 @@ def test_attention_at_a_long_context(ops_for):
     entries = [(20000, 1), (19000, 64), (33, 33)]
     q, kp, vp, table, ctx, dense, te, pos = _paged_case(entries, heads, kv_heads, head_dim, bs, torch.bfloat16, 41, spike=True)
     scale = head_dim**-0.5
-    got = ops.paged_attention(
+    got = _attend(
+        ops,
         q.cuda(), kp.cuda(), vp.cuda(), table.cuda(), ctx,
         num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, block_size=bs, scale=scale, window=None,
     ).cpu()
