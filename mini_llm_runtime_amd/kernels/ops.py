@@ -325,7 +325,7 @@ class HipOps:
 
     def _can_finish_stream(self, m: int, n: int, k: int) -> bool:
         """Whether the product [m, k] x [n, k]^T may run as the kernel that adds its result to the
-        residual stream itself (`mlr_gemm_residual_bf16`)."""
+        residual stream itself (`mlr_gemm_residual_bf16`): where the limits of the tuning say so."""
         t = self.tuning
         return (
             t.finish_stream and self.dtype == torch.bfloat16 and k % 8 == 0 and n % 4 == 0

@@ -47,6 +47,10 @@ class KernelTuning:
     finish_activation_bytes: int = 160 << 10
     finish_min_tokens: int = 5
     finish_max_tokens: int = 8
+    # (For more than 64 tokens the same was tried as an epilogue of the tiled kernels and lost: 0.5B
+    # prompt of 2,048 tokens 4.31 to 4.47 ms.  A lane of the matrix cores' accumulator holds four
+    # features of ONE token, so the float32 stream is read and written 16 bytes at a time at a stride of
+    # a row, where the norm kernel reads whole rows.)
 
     def __post_init__(self) -> None:
         for name in ("decode_partition", "decode_max_groups", "max_k_slices", "wide_attention_groups", "key_run_groups", "fuse_weight_bytes",

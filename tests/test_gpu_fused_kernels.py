@@ -289,7 +289,8 @@ def test_product_that_finishes_the_stream(gpu_device, m, n, k, bias, weight_f32)
     scale = torch.rsqrt(xd.cpu().double().pow(2).mean(1, keepdim=True) + eps)
     exact = (owed.h.cpu().double() * scale) @ w2.double().t()  # from the very activations the kernel read
     got = ops.linear(owed, w2.cuda(), b2.cuda())
-    torch.testing.assert_close(got.cpu().double(), exact + b2.double(), atol=2e-2, rtol=1.6e-2)
+    if n % 8 == 0:  # (else there is no matrix-core product: the norm is settled by its own kernel)
+        torch.testing.assert_close(got.cpu().double(), exact + b2.double(), atol=2e-2, rtol=1.6e-2)
     torch.testing.assert_close(got.cpu().double(), normed @ w2.double().t() + b2.double(), atol=6e-2, rtol=3e-2)
     wide = ops.linear(owed, w2.cuda(), b2.cuda(), out_dtype=torch.float32)
     if n % 8 == 0:
@@ -307,7 +308,7 @@ def test_product_that_finishes_the_stream(gpu_device, m, n, k, bias, weight_f32)
     torch.testing.assert_close(glu.cpu().double(), (gate * torch.sigmoid(gate) * up).reshape(m, -1), atol=2e-2, rtol=3e-2)
     # every matrix-core kernel that takes these tokens pays the factor the same way
     for kernel in (16, 14, 11, 12):
-        if (kernel == 16 and m > 16) or (kernel == 14 and m > 32) or n % 8:
+        if (kernel == 14 and m > 32) or n % 8:
             continue
         forced = ops.linear(owed, w2.cuda(), b2.cuda(), out_dtype=torch.float32, mfma_kernel=kernel)
         torch.testing.assert_close(forced.cpu().double(), exact + b2.double(), atol=1e-3 * n**0.5, rtol=1e-4, msg=lambda s: f"kernel {kernel}: {s}")
