@@ -84,14 +84,14 @@ __device__ __forceinline__ void row_scales_finish(const GemmEpilogue& ep, const 
     }
     return;
   }
-  // a thread per row, its partial sums one after the other (large tiles: many rows, few partial sums)
-  (void)lane, (void)wave, (void)waves;
-  for (int row = threadIdx.x; row < count; row += blockDim.x) {
+  // what the registers could not hold: a wavefront per row in turn, its lanes over the row's partial sums
+  for (int row = wave; row < count; row += waves) {
     const int m = m0 + row;
     float s = 0.f;
     if (m < M)
-      for (int p = 0; p < ep.sumsq_parts; ++p) s += ep.row_sumsq[static_cast<int64_t>(m) * ep.sumsq_parts + p];
-    scales[row] = m < M ? 1.0f / sqrtf(s / static_cast<float>(K) + ep.norm_eps) : 0.f;
+      for (int p = lane; p < ep.sumsq_parts; p += kWave) s += ep.row_sumsq[static_cast<int64_t>(m) * ep.sumsq_parts + p];
+    s = wave_sum(s);
+    if (lane == 0) scales[row] = m < M ? 1.0f / sqrtf(s / static_cast<float>(K) + ep.norm_eps) : 0.f;
   }
 }
 

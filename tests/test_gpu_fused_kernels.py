@@ -248,6 +248,7 @@ def _wide_open(gpu_device):
 _STREAM_SHAPES = [
     (1, 64, 64), (3, 896, 896), (4, 132, 200), (5, 100, 72), (8, 896, 4864), (9, 896, 896), (12, 132, 200), (16, 260, 1032),
     (17, 256, 512), (24, 100, 264), (32, 896, 896), (33, 64, 128), (50, 520, 264), (64, 896, 1024),
+    (8, 3584, 264), (20, 4104, 136),  # more parts a row than a consumer holds in registers: its slower way
 ]
 
 
