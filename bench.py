@@ -32,6 +32,11 @@ tokens in turn, 2,048 tokens a step: generated tokens a second, medians of the t
 first token and of the time between tokens.  `chunked`: 32 requests decode at context 2,048
 while one 8,192-token prompt is taken in four portions of 2,048 tokens beside them: the time of
 such a mixed step, which is also the time between the decoding requests' tokens.
+`library`: where one prompt step's time goes, by entry point of the kernel library (device events
+around every call of an untimed extra step), and beside it what the vendor library's routines take
+for the same shapes on the same card (torch's linear for the four products of a layer, its
+scaled_dot_product_attention for the attention): a yardstick for the hand-written kernels; none of
+those routines is on the engine's path.
 """
 
 from __future__ import annotations
@@ -80,7 +85,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--prompt-len", type=int, default=PROMPT_LEN)
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked"))
+    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library"))
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
     p.add_argument("--layers-32b", type=int, default=None, help="layers of the 32B shape's points (default: all 64)")
@@ -287,6 +292,88 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
             prompt_len=long_prompt,
             portion=portion,
         ),
+    }
+
+
+def library_yardstick(args, bench) -> dict:
+    """One prompt step with device events around every call into the kernel library, summed by entry
+    point (products by their weight's shape), and the vendor library's time for the layer's four
+    products and its attention at the same sizes."""
+    import torch
+    import torch.nn.functional as F
+
+    from mini_llm_runtime_amd.engine.runner import StepEntry
+
+    config, tokens, device = bench.config, args.prompt_len, bench.device
+    layers = config.num_hidden_layers
+    events = []
+    plain_call = bench.ops._call
+
+    def timed_call(name, *call_args, lib=None):
+        label = name
+        if name == "mlr_gemm_bf16":
+            label = f"{name} n={call_args[10]} k={call_args[11]}" + (" swiglu" if call_args[6] else "")
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        plain_call(name, *call_args, lib=lib)
+        end.record()
+        events.append((label, begin, end))
+
+    def step(rid):
+        bench.cache.create_request(rid)
+        bench.runner.step([StepEntry.of(rid, bench.prompt(), (tokens - 1,))], borrow_logits=True)
+        bench.sync()
+        bench.cache.release_request(rid)
+
+    bench.runner.use_graphs = False  # events cannot be recorded into a graph
+    step("warm")
+    bench.ops._call = timed_call
+    try:
+        step("timed")
+    finally:
+        bench.ops._call = plain_call
+    entry_points = {}
+    for label, begin, end in events:
+        row = entry_points.setdefault(label, {"calls": 0, "us": 0.0})
+        row["calls"] += 1
+        row["us"] += begin.elapsed_time(end) * 1e3
+    for row in entry_points.values():
+        row["us"] = round(row["us"], 1)
+        row["us_per_call"] = round(row["us"] / row["calls"], 1)
+
+    def timed(fn, repeats=10):
+        for _ in range(3):
+            fn()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        bench.sync()
+        begin.record()
+        for _ in range(repeats):
+            fn()
+        end.record()
+        bench.sync()
+        return round(begin.elapsed_time(end) * 1e3 / repeats, 1)
+
+    gen = torch.Generator(device=device).manual_seed(args.seed)
+    rand = lambda *shape: (torch.randn(*shape, device=device, generator=gen) * 0.05).to(bench.dtype)  # noqa: E731
+    d, heads, kv = config.head_dim, config.num_attention_heads, config.num_key_value_heads
+    hidden, inter = config.hidden_size, config.intermediate_size
+    library = {}
+    for name, n, k in (("qkv", (heads + 2 * kv) * d, hidden), ("o", hidden, heads * d), ("gate_up", 2 * inter, hidden),
+                       ("down", hidden, inter)):
+        x, w = rand(tokens, k), rand(n, k)
+        library[f"linear_{name} n={n} k={k}"] = timed(lambda: F.linear(x, w))
+        del x, w
+    q, key, value = rand(1, heads, tokens, d), rand(1, heads, tokens, d), rand(1, heads, tokens, d)
+    library["scaled_dot_product_attention causal"] = timed(lambda: F.scaled_dot_product_attention(q, key, value, is_causal=True))
+    return {
+        "metric": "prompt step by entry point, and the vendor library's routines at the same sizes",
+        "unit": "us",
+        "n_gpus": 1,
+        "dtype": bench.short,
+        "config": {"model": f"{args.config} shape", "layers": layers, "prompt_len": tokens, "hidden_size": hidden,
+                   "intermediate_size": inter, "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": d},
+        "entry_points": dict(sorted(entry_points.items(), key=lambda item: -item[1]["us"])),
+        "library_us_per_call": library,
     }
 
 
@@ -592,6 +679,12 @@ def main() -> int:
     bench = Bench(args, args.config, args.layers, batches)
     config = bench.config
 
+    if args.workload == "library":
+        line = library_yardstick(args, bench)
+        bench.close()
+        line["env"] = environment()
+        print(json.dumps(line), flush=True)
+        return 0
     if args.workload != "decode":
         work = burst if args.workload == "burst" else chunked
         bench.runner = bench.cache = None  # these workloads size a cache of their own

@@ -79,6 +79,8 @@ int mlr_gemm_simple(const void* x, const void* w, const void* bias, int bias_is_
 // mlr_gemm_bf16_slices returned for this shape) y is float32 [slices, m, n]: partial
 // sums over slices of k, the bias in slice 0, for the consumer to add up in order.
 int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
+// The kernel mlr_gemm_bf16 chooses for a shape cut into `slices` (its `kernel` argument's numbers).
+int mlr_gemm_bf16_kernel(int m, int n, int k, int slices);
 // `kernel` 0 lets the shape choose; 16 (streaming, up to 16 tokens), 14 (LDS-tiled, tiles of 32
 // tokens x 64 features), 11, 22, 44 (LDS-tiled with 64 x 64, 128 x 128, 256 x 256 tiles) force
 // one, for tests and tuning.  Any `slices` within

@@ -240,8 +240,10 @@ struct TiledShape {
   static constexpr int kLds = 2 * (BM + BN) * kLd * 2;              // bytes, two buffers
   // slices of K in flight ahead of the one in LDS: one for the large tiles, two for the small ones
   // (a slice of their work is shorter than a trip to memory; four were no faster, also for the
-  // tile of few tokens, which only streams weights)
-  static constexpr int kDepth = WM * WN >= 4 || GM * GN > 4 ? 1 : 2;
+  // tile of few tokens, which only streams weights), three for the tile of 160 features, which has
+  // its compute unit to itself and two wavefronts to keep the loads going (7B gate-up at 64 tokens:
+  // one slice ahead 70 us, three 58, four 60)
+  static constexpr int kDepth = WN == 5 ? 3 : (WM * WN >= 4 || GM * GN > 4 ? 1 : 2);
 };
 
 // Workgroup -> (slice, token tile, feature tile).  Consecutive workgroups go to the eight
@@ -664,7 +666,9 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 // 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 14 = gemm_tiled
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
 // rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 12 = gemm_tiled with tiles of 64
-// tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products.
+// tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products, 15 = gemm_tiled with
+// tiles of 64 tokens x 160 features (two wavefronts) for 41 to 64 tokens of products whose tiles then
+// make whole rounds over the compute units.
 // A small matrix (an output projection of a narrow model) at 17 to 64 tokens: the tiled kernels have
 // too few tiles of it to keep the compute units busy, the row-splitting kernel with its 16 features a
 // workgroup has four times as many workgroups (0.5B output projection with the norm behind it, in a
@@ -672,13 +676,40 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 // Larger matrices read the tokens too often that way (0.5B gate-up at 64 tokens: 10 us tiled, 16).
 static bool small_matrix(int n, int k) { return static_cast<int64_t>(n) * k * 2 <= (4ll << 20); }
 
+// 33 to 64 tokens, whole K (gate-up, the output head): such a product streams its weight once, and
+// it is done when the busiest compute unit has streamed its share.  Per tiling, that share is the
+// rows of the tiles that land on one compute unit, and the rate is what a compute unit takes in
+// with that tiling, measured in a replayed graph at 64 tokens (GB/s; `alone`: one tile per unit):
+//   64 features: 21;  128 features: 23 alone, 26 beside another;  160 features: 20 alone, 27.
+// 7B gate-up (37,888 rows): 592 / 296 / 237 tiles -> 64 / 68 / 58 us; a 27,648-row gate-up with k
+// 5,120: 66 / 58 / 78; 32B gate-up: 128 / 105 / 120; the 7B output head: 238 / 211 / 198.  Up to
+// 40 tokens the 160-feature tile was never ahead.
+static int choose_mid_tiles(int m, int n) {
+  struct Tiling {
+    int kernel, features;
+    float alone, beside;
+  };
+  constexpr Tiling kTilings[] = {{11, 64, 21.f, 21.f}, {12, 128, 23.f, 26.f}, {15, 160, 20.f, 27.f}};
+  int best = 11;
+  float best_time = 0.f;
+  for (const Tiling& t : kTilings) {
+    if (t.kernel == 15 && m <= 40) continue;
+    const int64_t tiles = (n + t.features - 1) / t.features;
+    const int64_t per_unit = (tiles + kComputeUnits - 1) / kComputeUnits;
+    const float time = static_cast<float>(per_unit * t.features) / (per_unit > 1 ? t.beside : t.alone);
+    if (best_time == 0.f || time < best_time) best = t.kernel, best_time = time;
+  }
+  return best;
+}
+
 static int choose_kernel(int m, int n, int k, int slices) {
   if (m <= 16 && !few_tokens_tiled(n, slices)) return 16;
   if (m <= 64 && small_matrix(n, k)) return 16;
   if (m <= 32) return 14;
-  // 33 to 64 tokens: tiles of 128 features read the tokens half as often per weight byte and stream
-  // faster once there are enough of them (32B gate-up at 64 tokens, 432 tiles: 128 to 103 us; the 7B
-  // output head 235 to 206 us; 7B gate-up, 296 tiles: 64 and 66 us)
+  // 33 to 64 tokens.  Cut along k (short runs of k per workgroup): tiles of 128 features once there
+  // are enough of them, else 64 (7B down in 8 slices 30.5 us either way, its output projection 10.6
+  // and 9.7 us; 160 features 41 and 15 us).
+  if (m <= 64 && slices == 1) return choose_mid_tiles(m, n);
   if (m <= 64) return static_cast<int64_t>((n + 127) / 128) * slices >= 384 ? 12 : 11;
   const GemmPlan plan = plan_many_tokens(m, n, k, slices);
   return plan.slices == slices ? plan.kernel : 11;
@@ -701,9 +732,10 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
     case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
     case 14: return launch_tiled<1, 1, 1, 2>(xb, wb, ep, m, n, k, slices, stream);  // 32 tokens x 64 features, two wavefronts
     case 12: return launch_tiled<1, 2, 2, 2>(xb, wb, ep, m, n, k, slices, stream);  // 64 tokens x 128 features
+    case 15: return launch_tiled<1, 5, 2, 1>(xb, wb, ep, m, n, k, slices, stream);  // 64 tokens x 160 features
     case 22: return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
     case 44: return launch_tiled<2, 2, 4, 4>(xb, wb, ep, m, n, k, slices, stream);
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 14, 12, 11, 22 or 44"); return -1;
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 22 or 44"); return -1;
   }
 }
 
@@ -742,6 +774,8 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices) {
   // unit before the cutting stops (32B down at 32 tokens: 320 workgroups 65 us, 640 workgroups 56 us)
   return choose_slices(tiles_64(m, n), (k / 8 + 3) / 4, min(max_slices, 8), 512);
 }
+
+int mlr_gemm_bf16_kernel(int m, int n, int k, int slices) { return choose_kernel(m, n, k, slices); }
 
 // y = x w^T (+ bias) in bfloat16 on the matrix cores; see mlr_gemm_simple for the
 // argument meanings.  Requires k % 8 == 0 and 16-byte aligned x and w.  With

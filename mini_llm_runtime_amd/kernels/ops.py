@@ -42,6 +42,7 @@ _SIGNATURES = {
     "mlr_gemm_residual_parts": ([_I, _I], _I),
     "mlr_gemm_residual_bf16": ([_VP, _VP, _VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _VP], _I),
     "mlr_gemm_bf16_slices": ([_I, _I, _I, _I], _I),
+    "mlr_gemm_bf16_kernel": ([_I, _I, _I, _I], _I),
     "mlr_qkv_rope_write_bf16": (
         [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP],
         _I,
@@ -412,7 +413,7 @@ class HipOps:
         accepts, instead of [M, N], a float32 stack [S, M, N] of partial sums over slices
         of k (bias in slice 0).  Narrow products of a few tokens are cut that way so that
         all compute units stream the weight; the norm kernel adds the slices in order.
-        mfma_kernel, slices: force one of the matrix-core kernels (16, 14, 12, 11, 22, 44) and a number
+        mfma_kernel, slices: force one of the matrix-core kernels (16, 15, 14, 12, 11, 22, 44) and a number
         of k slices instead of letting the shape choose; for tests and tuning.
         """
         if kernel not in ("auto", "fma"):

@@ -233,7 +233,7 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 14, 12, 11, 22, 44])
+@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 22, 44])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
@@ -251,6 +251,28 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     if kernel != 16:
         with pytest.raises(Exception, match="64 tokens"):
             ops.linear(x.cuda(), w.cuda(), mfma_kernel=16)
+
+
+@pytest.mark.parametrize("m,n,chosen", [(64, 37888, 15), (41, 37890, 15), (40, 37888, 11), (64, 27648, 12), (50, 16000, 11),
+                                        (64, 151936, 15)])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_wide_products_at_33_to_64_tokens(ops_for, m, n, chosen, swiglu):
+    """Whole-k products of 33 to 64 tokens choose their tile width (64, 128 or 160 features) by the
+    rounds their tiles make over the compute units; these widths reach each of the three, one with
+    a last tile that is not whole."""
+    ops = ops_for(torch.bfloat16)
+    k = 136
+    n = n - n % 4 if swiglu else n
+    assert ops.lib.mlr_gemm_bf16_kernel(m, n, k, 1) == chosen
+    x = _rand((m, k), torch.bfloat16, 71)
+    w = _rand((n, k), torch.bfloat16, 72, 0.05)
+    ref = x.double() @ w.double().t()
+    if swiglu:
+        quads = ref.view(m, -1, 4)
+        gate, up = quads[..., :2], quads[..., 2:]
+        ref = (gate * torch.sigmoid(gate) * up).reshape(m, -1)
+    got = ops.linear(x.cuda(), w.cuda(), None, swiglu=swiglu, out_dtype=None if swiglu else torch.float32)
+    torch.testing.assert_close(got.cpu().double(), ref, atol=2e-2 if swiglu else 2e-3, rtol=2e-2 if swiglu else 1e-4)
 
 
 @pytest.mark.parametrize("m", [17, 31, 32, 33, 50, 64])
