@@ -251,22 +251,44 @@ struct TiledShape {
 // run of the tile order, and that order walks groups of eight token tiles feature tile by
 // feature tile, so that the workgroups resident on an XCD at one time form a compact block
 // of the output and share their operands in its L2.
+// `light`: the last token tile holds so few tokens that only the first row of wavefronts has any
+// (a prompt portion of 2,048 tokens beside 32 decoding requests: the ninth tile of 256).  Such
+// tiles cost a fraction of a full one, and at the end of the order they would all land on the last
+// XCD, which would then idle while the others work: they are dealt out evenly instead, behind each
+// XCD's share of the full tiles.
 struct TileOrder {
-  int m_tiles, n_tiles, slices;
+  int m_tiles, n_tiles, slices, light;
 };
+__host__ __device__ inline TileOrder make_tile_order(int m, int n_tiles, int slices, int tile_tokens, int wave_rows) {
+  const int m_tiles = (m + tile_tokens - 1) / tile_tokens;
+  const int last = m - (m_tiles - 1) * tile_tokens;
+  return TileOrder{m_tiles, n_tiles, slices, m_tiles > 1 && last * wave_rows <= tile_tokens ? 1 : 0};
+}
 __device__ __forceinline__ void place_workgroup(const TileOrder& order, int id, int& slice, int& mt, int& nt) {
   constexpr int kXcds = 8, kGroup = 8;
-  const int tiles = order.m_tiles * order.n_tiles;
-  const int total = tiles * order.slices;
+  const int full_rows = order.m_tiles - order.light;
+  const int tiles = full_rows * order.n_tiles;  // full tiles of a slice
+  const int full = tiles * order.slices;
+  const int total = full + order.light * order.n_tiles * order.slices;
   const int q = total / kXcds, r = total % kXcds;
+  const int qf = full / kXcds, rf = full % kXcds;
   const int xcd = id % kXcds, local = id / kXcds;
-  int pos = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
+  const int full_here = qf + (xcd < rf ? 1 : 0);
+  if (local >= full_here) {  // one of this XCD's light tiles
+    const int before = (xcd * q + min(xcd, r)) - (xcd * qf + min(xcd, rf));
+    const int pos = before + local - full_here;
+    slice = pos / order.n_tiles;
+    nt = pos - slice * order.n_tiles;
+    mt = order.m_tiles - 1;
+    return;
+  }
+  int pos = xcd * qf + min(xcd, rf) + local;
   slice = pos / tiles;
   pos -= slice * tiles;
   const int per_group = kGroup * order.n_tiles;
   const int group = pos / per_group;
   const int first = group * kGroup;
-  const int size = min(order.m_tiles - first, kGroup);
+  const int size = min(full_rows - first, kGroup);
   const int in_group = pos - group * per_group;
   mt = first + in_group % size;
   nt = in_group / size;
@@ -395,7 +417,11 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) *reinterpret_cast<bf16x8_t*>(lds + buf * kBuffer + lds_off[it]) = reg[it];
   };
+  // A tile at the lower edge of the matrix may have tokens for its first rows of wavefronts only:
+  // the others skip the products and only help to stage the operands.
+  const bool idle = __builtin_amdgcn_readfirstlane(static_cast<int>(wm * 32 * WM >= x_rows)) != 0;
   auto multiply = [&](int buf) {
+    if (idle) return;
     const bf16* wt = lds + buf * kBuffer + (wn * 32 * WN + r32) * kLd + h * 8;
     const bf16* xt = lds + buf * kBuffer + (BN + wm * 32 * WM + r32) * kLd + h * 8;
 #pragma unroll
@@ -546,7 +572,7 @@ template <int WM, int WN, int GM = 2, int GN = 2>
 static int launch_tiled(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
                         hipStream_t stream) {
   using Shape = TiledShape<WM, WN, GM, GN>;
-  TileOrder order{(m + Shape::BM - 1) / Shape::BM, (n + Shape::BN - 1) / Shape::BN, slices};
+  const TileOrder order = make_tile_order(m, (n + Shape::BN - 1) / Shape::BN, slices, Shape::BM, GM);
   const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles * slices;
   if (groups >= (1ll << 31)) {
     set_error("mlr_gemm_bf16: too many tiles for one launch");
@@ -567,7 +593,7 @@ static int launch_tiled_qkv(const bf16* xb, const bf16* wb, GemmEpilogue ep, con
   const int rot_pairs = qkv.cos != nullptr ? (qkv.heads + qkv.kv_heads) * (qkv.head_dim / 2) : 0;
   const int rot_tiles = (rot_pairs + Shape::BN / 2 - 1) / (Shape::BN / 2);
   const int rest_tiles = (n - 2 * rot_pairs + Shape::BN - 1) / Shape::BN;
-  const TileOrder order{(m + Shape::BM - 1) / Shape::BM, rot_tiles + rest_tiles, 1};
+  const TileOrder order = make_tile_order(m, rot_tiles + rest_tiles, 1, Shape::BM, GM);
   const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles;
   MLR_REQUIRE(groups < (1ll << 31), "too many tiles for one launch");
   static bool prepared = false;

@@ -253,6 +253,25 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
             ops.linear(x.cuda(), w.cuda(), mfma_kernel=16)
 
 
+@pytest.mark.parametrize("kernel,m,n", [(44, 2080, 1100), (44, 530, 3000), (44, 257, 256), (22, 1050, 700), (11, 532, 2373),
+                                        (11, 90, 640), (12, 80, 1000), (44, 2112, 520), (44, 2113, 520)])
+@pytest.mark.parametrize("slices", [1, 2])
+def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
+    """A last token tile whose tokens fit the first row of wavefronts (a prompt portion beside a few
+    decoding requests) skips the matrix-core work of the others and is dealt out over the XCDs apart
+    from the full tiles: every tile of every slice is still computed exactly once.  (The last two
+    cases: 64 tokens in the last tile, which is light, and 65, which is not.)"""
+    ops = ops_for(torch.bfloat16)
+    k = 200
+    x = _rand((m, k), torch.bfloat16, 81)
+    w = _rand((n, k), torch.bfloat16, 82, 0.05)
+    b = _rand((n,), torch.float32, 83)
+    ref = x.double() @ w.double().t() + b.double()
+    got = ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, partial_sums=True, mfma_kernel=kernel, slices=slices)
+    total = got.cpu().double().sum(0) if slices > 1 else got.cpu().double()
+    torch.testing.assert_close(total, ref, atol=2e-3, rtol=1e-4)
+
+
 @pytest.mark.parametrize("m,n,chosen", [(64, 37888, 15), (41, 37890, 15), (40, 37888, 11), (64, 27648, 12), (50, 16000, 11),
                                         (64, 151936, 15)])
 @pytest.mark.parametrize("swiglu", [False, True])
