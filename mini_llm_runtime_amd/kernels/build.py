@@ -15,6 +15,7 @@ from __future__ import annotations
 import hashlib
 import json
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -149,7 +150,15 @@ def is_current(module: Module, folder: Optional[Path] = None) -> bool:
         return False
 
 
-def _run(cmd: Sequence[str], what: str) -> None:
+# The compiler reports every kernel's registers: a kernel that spills them to memory still
+# computes the right thing, ten times slower, so the build counts the spills and says so.
+RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
+_KERNEL_NAME = re.compile(r"remark: Function Name: (\S+)")
+_KERNEL_SPILL = re.compile(r"remark:\s+VGPRs Spill: (\d+)")
+
+
+def _run(cmd: Sequence[str], what: str) -> dict[str, int]:
+    """Runs a compiler command; returns {kernel: spilled vector registers} for the kernels it reported."""
     env = dict(os.environ)
     # hipcc and clang want a writable HOME/TMPDIR for their temporary files
     if not env.get("HOME") or not os.access(env.get("HOME", ""), os.W_OK):
@@ -158,9 +167,24 @@ def _run(cmd: Sequence[str], what: str) -> None:
     if proc.returncode != 0:
         raise RuntimeError(f"{what} failed (exit {proc.returncode}):\n$ {' '.join(cmd)}\n{proc.stdout}")
     noise = "is not a recognized feature for this target"
-    rest = [line for line in proc.stdout.splitlines() if line.strip() and noise not in line]
+    spills: dict[str, int] = {}
+    kernel, rest = None, []
+    for line in proc.stdout.splitlines():
+        named = _KERNEL_NAME.search(line)
+        if named:
+            kernel = named.group(1)
+            spills.setdefault(kernel, 0)
+        spilled = _KERNEL_SPILL.search(line)
+        if spilled and kernel is not None:
+            spills[kernel] = max(spills[kernel], int(spilled.group(1)))
+        if line.strip() and noise not in line and "[-Rpass-analysis=kernel-resource-usage]" not in line:
+            rest.append(line)
     if rest:
         log(f"{what}: " + "\n".join(rest))
+    for name, count in spills.items():
+        if count:
+            log(f"{what}: kernel {name} spills {count} vector registers to memory")
+    return spills
 
 
 def build_module(module: Module, *, force: bool = False, jobs: int = 8) -> Path:
@@ -184,17 +208,24 @@ def build_module(module: Module, *, force: bool = False, jobs: int = 8) -> Path:
     try:
         defines = [f"-D{d}" for d in module.defines]
 
-        def compile_one(pair: tuple[str, Path]) -> None:
+        def compile_one(pair: tuple[str, Path]) -> dict[str, int]:
             src, obj = pair
             log(f"  hipcc {src}")
-            _run([hipcc, *FLAGS, *defines, "-I", str(CSRC), "-c", str(CSRC / src), "-o", str(obj)], f"compiling {src}")
+            return _run(
+                [hipcc, *FLAGS, RESOURCE_REMARKS, *defines, "-I", str(CSRC), "-c", str(CSRC / src), "-o", str(obj)],
+                f"compiling {src}",
+            )
 
         with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(objects)))) as pool:
-            list(pool.map(compile_one, zip(module.sources, objects)))
+            reports = list(pool.map(compile_one, zip(module.sources, objects)))
+        kernels = {name: count for report in reports for name, count in report.items()}
         tmp = lib.with_suffix(f".tmp{os.getpid()}.so")
         _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objects)], f"linking {lib.name}")
         os.replace(tmp, lib)
-        lib.with_suffix(".json").write_text(json.dumps({"hash": _source_hash(module), "arch": ARCH}))
+        lib.with_suffix(".json").write_text(json.dumps({
+            "hash": _source_hash(module), "arch": ARCH, "kernels": len(kernels),
+            "spilling_kernels": {name: count for name, count in kernels.items() if count},
+        }))
     finally:
         done.set()
     log(f"built {lib.name} in {time.time() - started:.1f} s")
