@@ -37,6 +37,13 @@ around every call of an untimed extra step), and beside it what the vendor libra
 for the same shapes on the same card (torch's linear for the four products of a layer, its
 scaled_dot_product_attention for the attention): a yardstick for the hand-written kernels; none of
 those routines is on the engine's path.
+`reference`: the reference's own published measurements, run here at their parameters with the
+0.5B shape (random weights and token ids of the published lengths; its figures are of an RTX 3060
+laptop GPU in float16 and stand beside for scale): the burst of 8 short requests under continuous and
+static batching (docs/benchmarks/static-continuous.json: prompts of 3/7/4/9 tokens, 2/4/8/12 new
+tokens, 4 running requests, 64 tokens a step, block 16, 3 warm-up runs and 10 measured), the prompt step
+of 4 x 512 tokens (docs/benchmarks/prefill-4x512.json) and the decode attention at one request and a
+context of 2,048 (docs/split_kv_sweep.md:38-46).
 """
 
 from __future__ import annotations
@@ -85,7 +92,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--prompt-len", type=int, default=PROMPT_LEN)
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library"))
+    p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference"))
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
     p.add_argument("--layers-32b", type=int, default=None, help="layers of the 32B shape's points (default: all 64)")
@@ -292,6 +299,133 @@ def chunked(args, config, full_layers, model, ops, device) -> dict:
             prompt_len=long_prompt,
             portion=portion,
         ),
+    }
+
+
+def reference_measurements(args, bench) -> dict:
+    """The reference's three published measurements at their own parameters (see the module's text)."""
+    import random
+    from types import SimpleNamespace
+
+    import torch
+
+    from mini_llm_runtime_amd.engine import BatchingPolicy, ContinuousBatchEngine, PageAdmission, Scheduler
+    from mini_llm_runtime_amd.engine.factory import make_cache
+    from mini_llm_runtime_amd.engine.runner import ModelRunner, StepEntry
+    from mini_llm_runtime_amd.sampling.sampler import Sampler
+
+    config, model, ops, device = bench.config, bench.model, bench.ops, bench.device
+    published = {
+        "continuous": {"tokens_per_s": 71.70, "median_ttft_ms": 178.08, "median_tpot_ms": 25.56, "median_e2e_ms": 414.06},
+        "static": {"tokens_per_s": 65.43, "median_ttft_ms": 334.78, "median_tpot_ms": 24.06, "median_e2e_ms": 478.58},
+        "prefill_4x512_ms": 136.475,
+        "decode_attention_us": 77.0,
+        "hardware": "RTX 3060 Laptop, float16 (README.md:79-95, 114-115; docs/split_kv_sweep.md:38-46)",
+    }
+    # 1. the burst of 8 short requests, both policies
+    specs = [(3, 2), (7, 4), (4, 8), (9, 12)] * 2
+    cache = make_cache(model, block_size=16, num_blocks=64, max_requests=4)
+    runner = ModelRunner(model, cache, ops)
+    sampler = Sampler(ops, device)
+
+    def burst_of_eight(policy, seed: int) -> dict:
+        admission = PageAdmission(cache, max_step_tokens=64)
+        scheduler = Scheduler(max_running_requests=4, max_batch_tokens=64, admit=admission.admit, batching_policy=policy)
+        engine = ContinuousBatchEngine(scheduler=scheduler, runner=runner, admission=admission, sampler=sampler)
+        rng = random.Random(seed)
+        torch.cuda.synchronize(device)
+        begin = time.perf_counter()
+        for i, (prompt, new) in enumerate(specs):
+            engine.submit(f"r{i}", [rng.randrange(config.vocab_size) for _ in range(prompt)], max_new_tokens=new)
+        while engine.scheduler.busy:
+            engine.step()
+        torch.cuda.synchronize(device)
+        seconds = time.perf_counter() - begin
+        shots = engine.all_times()
+        return {
+            "tokens_per_s": sum(new for _, new in specs) / seconds,
+            "median_ttft_ms": median([t.ttft_ms for t in shots]),
+            "median_tpot_ms": median([t.median_tpot_ms for t in shots if t.median_tpot_ms is not None]),
+            "median_e2e_ms": median([t.e2e_ms for t in shots]),
+        }
+
+    policies = {"continuous": BatchingPolicy.CONTINUOUS, "static": BatchingPolicy.STATIC}
+    samples = {name: [] for name in policies}
+    for trial in range(3 + 10):  # the cases take turns, in reversed order on odd rounds, as published
+        order = list(policies) if trial % 2 == 0 else list(policies)[::-1]
+        for name in order:
+            shot = burst_of_eight(policies[name], args.seed)
+            if trial >= 3:
+                samples[name].append(shot)
+    bursts = {
+        name: {key: round(median([shot[key] for shot in shots]), 3) for key in shots[0]} for name, shots in samples.items()
+    }
+    del runner, cache
+    # 2. four prompts of 512 tokens in one step of the step function (model and cache write only)
+    cache = make_cache(model, block_size=16, num_blocks=4 * 32 + 8, max_requests=4)
+    runner = ModelRunner(model, cache, ops)
+    gen = torch.Generator().manual_seed(args.seed)
+    times = []
+    for trial in range(2 + 6):
+        entries = []
+        for i in range(4):
+            cache.create_request(f"p{i}")
+            ids = torch.randint(0, config.vocab_size, (512,), generator=gen).tolist()
+            entries.append(StepEntry.of(f"p{i}", ids, (511,)))
+        torch.cuda.synchronize(device)
+        begin = time.perf_counter()
+        runner.step(entries, borrow_logits=True)
+        torch.cuda.synchronize(device)
+        times.append((time.perf_counter() - begin) * 1e3)
+        for i in range(4):
+            cache.release_request(f"p{i}")
+    prefill_ms = median(times[2:])
+    del runner, cache
+    # 3. the decode attention alone: one request, context 2,048, on the cache's page layout
+    heads, kv, d, bs, ctx_len = config.num_attention_heads, config.num_key_value_heads, config.head_dim, 16, 2048
+    pages = ctx_len // bs
+    g = torch.Generator(device=device).manual_seed(args.seed)
+    rand = lambda *shape: torch.randn(*shape, device=device, generator=g).to(bench.dtype)  # noqa: E731
+    key_pages, value_pages, q = rand(pages, kv, bs, d), rand(pages, kv, d, bs), rand(1, heads * d)
+    table = torch.randperm(pages, device=device).to(torch.int32).view(1, pages)
+    one = lambda v: torch.tensor(v, dtype=torch.int32, device=device)  # noqa: E731
+    plan = SimpleNamespace(num_entries=1, token_entry=one([0]), positions=one([ctx_len - 1]), cu_q=one([0, 1]),
+                           context_lens=one([ctx_len]), max_context_len=ctx_len, max_q_len=1, num_query_tiles=0,
+                           num_decode_entries=1, max_decode_context=ctx_len)
+    attend = lambda: ops.paged_attention(  # noqa: E731
+        q, key_pages, value_pages, table, plan, plan=plan, num_heads=heads, num_kv_heads=kv, head_dim=d, block_size=bs,
+        scale=d ** -0.5, window=None)
+    for _ in range(3):
+        attend()
+    torch.cuda.synchronize(device)
+    graph, kept = torch.cuda.CUDAGraph(), []  # 50 calls recorded and replayed: the kernels' time, not the host's
+    with torch.cuda.graph(graph):
+        for _ in range(50):
+            kept.append(attend())
+    graph.replay()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize(device)
+    begin.record()
+    for _ in range(10):
+        graph.replay()
+    end.record()
+    torch.cuda.synchronize(device)
+    attention_us = begin.elapsed_time(end) * 1e3 / 500
+    return {
+        "metric": "the reference's published measurements at their own parameters",
+        "value": bursts["continuous"]["tokens_per_s"],
+        "unit": "tokens/s (continuous batching, burst of 8 short requests)",
+        "n_gpus": 1,
+        "higher_is_better": True,
+        "vs_baseline": round(bursts["continuous"]["tokens_per_s"] / published["continuous"]["tokens_per_s"], 1),
+        "dtype": bench.short,
+        "data": "synthetic (random weights, uniform random token ids of the published lengths)",
+        "burst_of_8": bursts,
+        "prefill_4x512_ms": round(prefill_ms, 3),
+        "decode_attention_us": round(attention_us, 2),
+        "published": published,
+        "config": dict(workload_config(args, config, bench.full_layers), requests=8, max_running_requests=4,
+                       max_batch_tokens=64, kv_block_size=16),
     }
 
 
@@ -679,8 +813,8 @@ def main() -> int:
     bench = Bench(args, args.config, args.layers, batches)
     config = bench.config
 
-    if args.workload == "library":
-        line = library_yardstick(args, bench)
+    if args.workload in ("library", "reference"):
+        line = (library_yardstick if args.workload == "library" else reference_measurements)(args, bench)
         bench.close()
         line["env"] = environment()
         print(json.dumps(line), flush=True)

@@ -49,3 +49,26 @@ def test_default_line_keeps_the_contract(tmp_path):
     assert set(line["points"]) == {"decode_b1", "decode_b64"}
     memory = line["peak_memory_gb"]  # weights (about 1 GB) and the page pool at least, the card's 288 GB at most
     assert 1.0 < memory["allocated"] <= memory["reserved"] < 288 and memory["device_in_use"] >= memory["reserved"]
+
+
+@pytest.mark.gpu
+def test_the_reference_measurements_workload_prints_its_line():
+    """The reference's published measurements at their parameters: both batching policies of the burst of
+    eight, the 4 x 512 prompt step and the decode attention, each beside the published figure."""
+    run = subprocess.run(
+        [sys.executable, str(ROOT / "bench.py"), "--workload", "reference"],
+        capture_output=True, text=True, timeout=600, cwd=str(ROOT),
+    )
+    assert run.returncode == 0, run.stderr[-2000:]
+    lines = [l for l in run.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    bursts = line["burst_of_8"]
+    assert set(bursts) == {"continuous", "static"}
+    for policy in bursts.values():
+        assert policy["tokens_per_s"] > 0 and policy["median_ttft_ms"] > 0 and policy["median_e2e_ms"] >= policy["median_ttft_ms"]
+    # a request of the second batch waits for the whole first batch under static batching
+    assert bursts["static"]["median_ttft_ms"] > bursts["continuous"]["median_ttft_ms"]
+    assert line["value"] == bursts["continuous"]["tokens_per_s"]
+    assert abs(line["vs_baseline"] - line["value"] / line["published"]["continuous"]["tokens_per_s"]) < 0.1
+    assert line["prefill_4x512_ms"] > 0 and line["decode_attention_us"] > 0
