@@ -41,7 +41,9 @@ those routines is on the engine's path.
 0.5B shape (random weights and token ids of the published lengths; its figures are of an RTX 3060
 laptop GPU in float16 and stand beside for scale): the burst of 8 short requests under continuous and
 static batching (docs/benchmarks/static-continuous.json: prompts of 3/7/4/9 tokens, 2/4/8/12 new
-tokens, 4 running requests, 64 tokens a step, block 16, 3 warm-up runs and 10 measured), the prompt step
+tokens, 4 running requests, 64 tokens a step, block 16, 3 warm-up runs and 10 measured), the time to the
+first token of a request that arrives when the first four have reserved all 28 pages or 28 of 29
+(scripts/benchmark_block_pressure_ttft.py:25-45, 170-232), the prompt step
 of 4 x 512 tokens (docs/benchmarks/prefill-4x512.json) and the decode attention at one request and a
 context of 2,048 (docs/split_kv_sweep.md:38-46).
 """
@@ -318,9 +320,10 @@ def reference_measurements(args, bench) -> dict:
     published = {
         "continuous": {"tokens_per_s": 71.70, "median_ttft_ms": 178.08, "median_tpot_ms": 25.56, "median_e2e_ms": 414.06},
         "static": {"tokens_per_s": 65.43, "median_ttft_ms": 334.78, "median_tpot_ms": 24.06, "median_e2e_ms": 478.58},
+        "late_request_ttft_ms": {"28_blocks": 76.73, "29_blocks": 52.46, "paired_difference": 23.60},
         "prefill_4x512_ms": 136.475,
         "decode_attention_us": 77.0,
-        "hardware": "RTX 3060 Laptop, float16 (README.md:79-95, 114-115; docs/split_kv_sweep.md:38-46)",
+        "hardware": "RTX 3060 Laptop, float16 (README.md:79-95, 114-115; docs/split_kv_sweep.md:38-46; docs/block_pressure_ttft_benchmark.md:38-41)",
     }
     # 1. the burst of 8 short requests, both policies
     specs = [(3, 2), (7, 4), (4, 8), (9, 12)] * 2
@@ -361,6 +364,41 @@ def reference_measurements(args, bench) -> dict:
         name: {key: round(median([shot[key] for shot in shots]), 3) for key in shots[0]} for name, shots in samples.items()
     }
     del runner, cache
+    # 1b. a request that arrives behind step 0 when the first four have reserved every page (28) or all but one (29)
+    first, late = [(128, 2), (128, 3), (128, 3), (1, 3)], (7, 2)
+    pools = {}
+    for blocks in (28, 29):
+        pool = make_cache(model, block_size=16, num_blocks=blocks, max_requests=5)
+        pools[blocks] = (pool, ModelRunner(model, pool, ops))
+
+    def late_arrival(blocks: int) -> dict:
+        pool, pool_runner = pools[blocks]
+        admission = PageAdmission(pool, max_step_tokens=sum(n for n, _ in first))
+        scheduler = Scheduler(max_running_requests=5, max_batch_tokens=sum(n for n, _ in first), admit=admission.admit)
+        engine = ContinuousBatchEngine(scheduler=scheduler, runner=pool_runner, admission=admission, sampler=sampler)
+        rng = random.Random(args.seed)
+        for i, (prompt, new) in enumerate(first):
+            engine.submit(f"first{i}", [rng.randrange(config.vocab_size) for _ in range(prompt)], max_new_tokens=new)
+        engine.step()
+        engine.submit("late", [rng.randrange(config.vocab_size) for _ in range(late[0])], max_new_tokens=late[1])
+        while engine.scheduler.busy:
+            engine.step()
+        shot = engine.times("late")
+        return {"ttft_ms": shot.ttft_ms, "queue_wait_ms": shot.queue_wait_ms}
+
+    waits = {28: [], 29: []}
+    for trial in range(3 + 10):
+        for blocks in ((28, 29) if trial % 2 == 0 else (29, 28)):
+            shot = late_arrival(blocks)
+            if trial >= 3:
+                waits[blocks].append(shot)
+    late_request = {
+        f"{blocks}_blocks": {key: round(median([shot[key] for shot in shots]), 3) for key in shots[0]}
+        for blocks, shots in waits.items()
+    }
+    late_request["paired_ttft_difference_ms"] = round(
+        median([a["ttft_ms"] - b["ttft_ms"] for a, b in zip(waits[28], waits[29])]), 3)
+    del pools
     # 2. four prompts of 512 tokens in one step of the step function (model and cache write only)
     cache = make_cache(model, block_size=16, num_blocks=4 * 32 + 8, max_requests=4)
     runner = ModelRunner(model, cache, ops)
@@ -421,6 +459,7 @@ def reference_measurements(args, bench) -> dict:
         "dtype": bench.short,
         "data": "synthetic (random weights, uniform random token ids of the published lengths)",
         "burst_of_8": bursts,
+        "late_request_under_page_pressure": late_request,
         "prefill_4x512_ms": round(prefill_ms, 3),
         "decode_attention_us": round(attention_us, 2),
         "published": published,

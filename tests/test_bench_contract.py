@@ -72,3 +72,6 @@ def test_the_reference_measurements_workload_prints_its_line():
     assert line["value"] == bursts["continuous"]["tokens_per_s"]
     assert abs(line["vs_baseline"] - line["value"] / line["published"]["continuous"]["tokens_per_s"]) < 0.1
     assert line["prefill_4x512_ms"] > 0 and line["decode_attention_us"] > 0
+    # with every page reserved the late request waits for a request to finish: one step longer in the queue
+    late = line["late_request_under_page_pressure"]
+    assert late["28_blocks"]["queue_wait_ms"] > late["29_blocks"]["queue_wait_ms"] and late["paired_ttft_difference_ms"] > 0
