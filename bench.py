@@ -16,7 +16,8 @@ second, step time, share of the HBM bound) and the prefill for the two larger sh
 7B shape's burst workload and the 32B shape's chunked workload (below) as `burst` and
 `chunked`, with the number of layers run and of the full model beside them;
 `points_ctx16k` decode at batch 8 and the prefill at a context of 16,384 tokens for the 0.5B
-and the 7B shape.  `peak_memory_gb` (per shape) is the most device memory the run held.
+and the 7B shape, `points_reference` the reference's own published measurements at their parameters
+beside its figures (`--workload reference`, below).  `peak_memory_gb` (per shape) is the most device memory the run held.
 
 How it measures (the reference's harness rules, src/mini_llm_runtime/timing.py:49-82,
 141-160 and environment.py:37-93): untimed warm-up first; the timed steps between
@@ -437,7 +438,7 @@ def reference_measurements(args, bench) -> dict:
         attend()
     torch.cuda.synchronize(device)
     graph, kept = torch.cuda.CUDAGraph(), []  # 50 calls recorded and replayed: the kernels' time, not the host's
-    with torch.cuda.graph(graph):
+    with torch.inference_mode(), torch.cuda.graph(graph):  # (as the engine records its steps)
         for _ in range(50):
             kept.append(attend())
     graph.replay()
@@ -866,6 +867,7 @@ def main() -> int:
         print(json.dumps(line), flush=True)
         return 0
 
+    default_run = not args.no_large and args.config == "qwen2.5-0.5b" and args.layers is None and args.dtype == "bfloat16"
     main_run = bench.decode(args.batch, args.warmup, args.steps)
     ms_main = main_run["ms"]
     points = {}
@@ -878,6 +880,27 @@ def main() -> int:
     kv_per_token = bench.kv_bytes_per_token()
     full_layers = bench.full_layers
     peak_memory = bench.peak_memory()
+    points_reference = None
+    if default_run:
+        # the reference's own published measurements at their parameters, compact (`--workload reference` has all)
+        ours = reference_measurements(args, bench)
+        theirs = ours["published"]
+        points_reference = {
+            "burst_of_8_continuous_tokens_per_s": ours["burst_of_8"]["continuous"]["tokens_per_s"],
+            "burst_of_8_static_tokens_per_s": ours["burst_of_8"]["static"]["tokens_per_s"],
+            "burst_of_8_continuous_median_ttft_ms": ours["burst_of_8"]["continuous"]["median_ttft_ms"],
+            "late_request_ttft_ms_28_and_29_pages": [ours["late_request_under_page_pressure"][k]["ttft_ms"] for k in ("28_blocks", "29_blocks")],
+            "prefill_4x512_ms": ours["prefill_4x512_ms"],
+            "decode_attention_us": ours["decode_attention_us"],
+            "published_rtx3060_fp16": {
+                "burst_of_8_continuous_tokens_per_s": theirs["continuous"]["tokens_per_s"],
+                "burst_of_8_static_tokens_per_s": theirs["static"]["tokens_per_s"],
+                "burst_of_8_continuous_median_ttft_ms": theirs["continuous"]["median_ttft_ms"],
+                "late_request_ttft_ms_28_and_29_pages": [theirs["late_request_ttft_ms"]["28_blocks"], theirs["late_request_ttft_ms"]["29_blocks"]],
+                "prefill_4x512_ms": theirs["prefill_4x512_ms"],
+                "decode_attention_us": theirs["decode_attention_us"],
+            },
+        }
     bench.close()
 
     line = {
@@ -921,7 +944,8 @@ def main() -> int:
     }
     if args.tuning:
         line["tuning"] = args.tuning
-    if not args.no_large and args.config == "qwen2.5-0.5b" and args.layers is None and args.dtype == "bfloat16":
+    if default_run:
+        line["points_reference"] = points_reference
         # the other configurations' measurements: decode at batch 1, 8 and 64 and the prefill for the 7B
         # shape and the whole 32B shape (64 layers, 65 GB of weights), the burst of 64 requests on the
         # 7B shape, the 8,192-token prompt in portions beside 32 decoding requests on the 32B shape
