@@ -45,7 +45,8 @@ static batching (docs/benchmarks/static-continuous.json: prompts of 3/7/4/9 toke
 tokens, 4 running requests, 64 tokens a step, block 16, 3 warm-up runs and 10 measured), the time to the
 first token of a request that arrives when the first four have reserved all 28 pages or 28 of 29
 (scripts/benchmark_block_pressure_ttft.py:25-45, 170-232), the prompt step
-of 4 x 512 tokens (docs/benchmarks/prefill-4x512.json) and the decode attention at one request and a
+of 4 x 512 and of 4 x 256 tokens (docs/benchmarks/prefill-4x512.json, docs/prefill_attention_backends.md:73-77)
+and the decode attention at one request and a
 context of 2,048 (docs/split_kv_sweep.md:38-46).
 """
 
@@ -323,8 +324,9 @@ def reference_measurements(args, bench) -> dict:
         "static": {"tokens_per_s": 65.43, "median_ttft_ms": 334.78, "median_tpot_ms": 24.06, "median_e2e_ms": 478.58},
         "late_request_ttft_ms": {"28_blocks": 76.73, "29_blocks": 52.46, "paired_difference": 23.60},
         "prefill_4x512_ms": 136.475,
+        "prefill_4x256_ms": 68.77,
         "decode_attention_us": 77.0,
-        "hardware": "RTX 3060 Laptop, float16 (README.md:79-95, 114-115; docs/split_kv_sweep.md:38-46; docs/block_pressure_ttft_benchmark.md:38-41)",
+        "hardware": "RTX 3060 Laptop, float16 (README.md:79-95, 114-115; docs/split_kv_sweep.md:38-46; docs/block_pressure_ttft_benchmark.md:38-41; docs/prefill_attention_backends.md:73-77)",
     }
     # 1. the burst of 8 short requests, both policies
     specs = [(3, 2), (7, 4), (4, 8), (9, 12)] * 2
@@ -400,25 +402,28 @@ def reference_measurements(args, bench) -> dict:
     late_request["paired_ttft_difference_ms"] = round(
         median([a["ttft_ms"] - b["ttft_ms"] for a, b in zip(waits[28], waits[29])]), 3)
     del pools
-    # 2. four prompts of 512 tokens in one step of the step function (model and cache write only)
+    # 2. four prompts of 512 (and of 256) tokens in one step of the step function (model and cache write only)
     cache = make_cache(model, block_size=16, num_blocks=4 * 32 + 8, max_requests=4)
     runner = ModelRunner(model, cache, ops)
     gen = torch.Generator().manual_seed(args.seed)
-    times = []
-    for trial in range(2 + 6):
-        entries = []
-        for i in range(4):
-            cache.create_request(f"p{i}")
-            ids = torch.randint(0, config.vocab_size, (512,), generator=gen).tolist()
-            entries.append(StepEntry.of(f"p{i}", ids, (511,)))
-        torch.cuda.synchronize(device)
-        begin = time.perf_counter()
-        runner.step(entries, borrow_logits=True)
-        torch.cuda.synchronize(device)
-        times.append((time.perf_counter() - begin) * 1e3)
-        for i in range(4):
-            cache.release_request(f"p{i}")
-    prefill_ms = median(times[2:])
+    prefill_of_four = {}
+    for length in (512, 256):
+        times = []
+        for trial in range(2 + 6):
+            entries = []
+            for i in range(4):
+                cache.create_request(f"p{i}")
+                ids = torch.randint(0, config.vocab_size, (length,), generator=gen).tolist()
+                entries.append(StepEntry.of(f"p{i}", ids, (length - 1,)))
+            torch.cuda.synchronize(device)
+            begin = time.perf_counter()
+            runner.step(entries, borrow_logits=True)
+            torch.cuda.synchronize(device)
+            times.append((time.perf_counter() - begin) * 1e3)
+            for i in range(4):
+                cache.release_request(f"p{i}")
+        prefill_of_four[length] = median(times[2:])
+    prefill_ms = prefill_of_four[512]
     del runner, cache
     # 3. the decode attention alone: one request, context 2,048, on the cache's page layout
     heads, kv, d, bs, ctx_len = config.num_attention_heads, config.num_key_value_heads, config.head_dim, 16, 2048
@@ -462,6 +467,7 @@ def reference_measurements(args, bench) -> dict:
         "burst_of_8": bursts,
         "late_request_under_page_pressure": late_request,
         "prefill_4x512_ms": round(prefill_ms, 3),
+        "prefill_4x256_ms": round(prefill_of_four[256], 3),
         "decode_attention_us": round(attention_us, 2),
         "published": published,
         "config": dict(workload_config(args, config, bench.full_layers), requests=8, max_running_requests=4,
