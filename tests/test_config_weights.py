@@ -76,6 +76,13 @@ def test_a_head_size_no_kernel_runs_is_refused_when_the_model_is_built():
         build_model(too_wide)
 
 
+def test_an_odd_intermediate_size_is_refused_when_the_model_is_built():
+    """Gate and up rows are woven in pairs for the SwiGLU epilogue: an odd number of them has no such
+    layout, and the feed-forward says so instead of computing something else."""
+    with pytest.raises(ValueError, match="intermediate size even"):
+        build_model(Qwen2Config.from_dict({**TINY_A, "intermediate_size": 129}))
+
+
 def test_random_model_is_seeded_and_loads(tmp_path):
     d1 = make_model_dir(tmp_path / "x", "A", seed=5)
     d2 = make_model_dir(tmp_path / "y", "A", seed=5)
