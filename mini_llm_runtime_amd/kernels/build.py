@@ -155,6 +155,7 @@ def is_current(module: Module, folder: Optional[Path] = None) -> bool:
 RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
 _KERNEL_NAME = re.compile(r"remark: Function Name: (\S+)")
 _KERNEL_SPILL = re.compile(r"remark:\s+VGPRs Spill: (\d+)")
+_SOURCE_CONTEXT = re.compile(r"^\s*\d*\s*\|")
 
 
 def _run(cmd: Sequence[str], what: str) -> dict[str, int]:
@@ -168,7 +169,7 @@ def _run(cmd: Sequence[str], what: str) -> dict[str, int]:
         raise RuntimeError(f"{what} failed (exit {proc.returncode}):\n$ {' '.join(cmd)}\n{proc.stdout}")
     noise = "is not a recognized feature for this target"
     spills: dict[str, int] = {}
-    kernel, rest = None, []
+    kernel, rest, in_report = None, [], False
     for line in proc.stdout.splitlines():
         named = _KERNEL_NAME.search(line)
         if named:
@@ -177,7 +178,13 @@ def _run(cmd: Sequence[str], what: str) -> dict[str, int]:
         spilled = _KERNEL_SPILL.search(line)
         if spilled and kernel is not None:
             spills[kernel] = max(spills[kernel], int(spilled.group(1)))
-        if line.strip() and noise not in line and "[-Rpass-analysis=kernel-resource-usage]" not in line:
+        if "[-Rpass-analysis=kernel-resource-usage]" in line:
+            in_report = True  # the source line and the caret under it belong to the report
+            continue
+        if in_report and _SOURCE_CONTEXT.match(line):
+            continue
+        in_report = False
+        if line.strip() and noise not in line:
             rest.append(line)
     if rest:
         log(f"{what}: " + "\n".join(rest))

@@ -13,6 +13,8 @@ from mini_llm_runtime_amd.kernels import build
 def test_spilled_registers_are_read_from_the_compiler_report(monkeypatch):
     report = "\n".join([
         "a.hip:10:1: remark: Function Name: _Zkernel_one [-Rpass-analysis=kernel-resource-usage]",
+        "   10 | __global__ void kernel_one(int n) {",
+        "      | ^",
         "a.hip:10:1: remark:     VGPRs: 128 [-Rpass-analysis=kernel-resource-usage]",
         "a.hip:10:1: remark:     VGPRs Spill: 301 [-Rpass-analysis=kernel-resource-usage]",
         "a.hip:90:1: remark: Function Name: _Zkernel_two [-Rpass-analysis=kernel-resource-usage]",
@@ -27,6 +29,7 @@ def test_spilled_registers_are_read_from_the_compiler_report(monkeypatch):
     )
     assert build._run(["hipcc"], "compiling a.hip") == {"_Zkernel_one": 301, "_Zkernel_two": 0}
     assert any("warning: something else" in line and "remark" not in line for line in logged)
+    assert not any("__global__" in line or "| ^" in line for line in logged)
     assert any("_Zkernel_one spills 301" in line for line in logged)
 
 
