@@ -19,7 +19,9 @@
 //    is the largest that still keeps the compute units busy), K in
 //    slices of 64 staged through double-buffered LDS by range-checked
 //    buffer loads (edge tiles and the tail of K read zeros, no branches),
-//    32x32x16 MFMA.  Workgroups are placed so that those resident on
+//    32x32x16 MFMA.  Beyond 64 tokens the two larger tilings run gemm_direct: the same tiles
+//    loaded straight into LDS (no registers, no LDS stores; rows swizzled instead of padded),
+//    with a step's barrier ahead of its last quarter of products.  Workgroups are placed so that those resident on
 //    one XCD share operands in its L2.  Up to 16 tokens take this kernel too once
 //    its tiles fill the compute units (it streams a wide weight fastest).
 //    With more than one K slice both kernels write float32 partial sums
@@ -544,6 +546,190 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
   }
 }
 
+// ---- tiled, tiles loaded straight into LDS ---------------------------------------------------------
+// The square tiles of gemm_tiled_kernel (64, 128 or 256 on a side, wavefronts of WM x WN blocks of 32 x 32
+// in a GM x GN arrangement) with two changes to what a step of k costs beside its products.  The tiles
+// go from memory into LDS without passing registers (a lane's 16 bytes land at wavefront base + 16 *
+// lane, so rows are 128 bytes without padding, and a row's eight 16-byte pieces are stored in the
+// order piece ^ (row % 8): the operand reads of eight consecutive rows then fall into eight different
+// piece slots).  And the barrier of a step stands before its last quarter of products: behind it every
+// wavefront first asks for the next slice's first operands and for the slice after that, then
+// multiplies the quarter it kept, so the matrix cores have work while those arrive.  (KEEP: quarters
+// kept; two cost registers and gained nothing.  Eight wavefronts of 128 x 64 or 64 x 128 on the
+// 256 x 256 tile ran like sixteen of 64 x 64; sixteen of 32 x 32 on the 128 x 128 tile slower than four.)
+// Measured against the register-staged kernel on one matrix streamed again and again: 7B gate-up at
+// 2,048 tokens 592 to 527 us (hipBLASLt: 584), 7B down in two slices 262 to 247, 32B down in three
+// slices 541 to 493, 0.5B gate-up 57 to 51 (the library: 53); on a model's weights, which come from
+// memory, 1 to 10 %.
+constexpr int direct_lds_bytes(int tile) { return 2 * 2 * tile * kBK * 2; }  // two buffers of (tile + tile) rows x 128 bytes
+
+template <int KEEP, int WM, int WN, int GM, int GN>
+__global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+                                                                  GemmEpilogue ep, TileOrder order, int M, int N, int K) {
+  constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN, WAVES = GM * GN;
+  static_assert(BM == BN, "square tiles");
+  constexpr int kRuns = (BM + BN) / 8;  // 1 KB runs (8 rows) of a buffer, dealt out to the wavefronts in turn
+  constexpr int kMostPieces = 8;        // at most this many per wavefront
+  static_assert(kRuns % WAVES == 0 && kRuns / WAVES <= kMostPieces && kRuns / 2 % WAVES == 0, "the wavefronts share a buffer's runs evenly");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int kBufferBytes = (BM + BN) * kBK * 2;
+  __shared__ float scales[BM];
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wn = wave % GN;
+  const int wm = wave / GN;
+  const int r32 = lane % 32;
+  const int h = lane / 32;
+  int slice, mt, nt;
+  place_workgroup(order, blockIdx.x, slice, mt, nt);
+  const int n0 = nt * BN;
+  const int m0 = mt * BM;
+  RowScaleLoads<1, 1> owed;
+  if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, m0, BM, M);
+  const int chunks = K / 8;
+  const int slices = order.slices;
+  const int k_slices = (K + kBK - 1) / kBK;
+  const int per = (k_slices + slices - 1) / slices;
+  const int s_begin = slice * per;
+  const int s_end = min(k_slices, s_begin + per);
+
+  const int w_rows = min(BN, N - n0), x_rows = min(BM, M - m0);
+  const __amdgpu_buffer_rsrc_t w_buf = make_buffer(w + static_cast<int64_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2u);
+  const __amdgpu_buffer_rsrc_t x_buf = make_buffer(x + static_cast<int64_t>(m0) * K, static_cast<unsigned>(x_rows) * K * 2u);
+  // piece p of this wavefront fills rows 8 * (WAVES p + wave) .. + 7 of a buffer (its first half: weights,
+  // its second: tokens): lane l brings row + l / 8, piece (l % 8) ^ (l / 8) to slot l % 8
+  const int lane_row = lane / 8;
+  const int lane_chunk = (lane % 8) ^ lane_row;
+  unsigned piece_off[kMostPieces];
+#pragma unroll
+  for (int p = 0; p < kMostPieces; ++p) {
+    const int row = 8 * (WAVES * p + wave) + lane_row;  // first half of the pieces: weight rows, second: token rows
+    piece_off[p] = static_cast<unsigned>(row % BN) * K * 2u + lane_chunk * 16u;
+  }
+  auto fetch = [&](int s, int buf) {
+    const int left = s < s_end ? chunks - s * (kBK / 8) : 0;
+    const unsigned off_ok = lane_chunk < left ? 0u : kOutOfBuffer;
+#pragma unroll
+    for (int p = 0; p < kMostPieces; ++p) {
+      if (p * WAVES >= kRuns) break;
+      __attribute__((address_space(3))) void* dst =
+          (__attribute__((address_space(3))) void*)(smem + buf * kBufferBytes + (WAVES * p + wave) * 1024);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(p * WAVES < kRuns / 2 ? w_buf : x_buf, dst, 16, (piece_off[p] + s * (kBK * 2u)) | off_ok, 0, 0, 0);
+    }
+  };
+
+  f32x16_t acc[WN][WM];
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const bool idle = __builtin_amdgcn_readfirstlane(static_cast<int>(wm * 32 * WM >= x_rows)) != 0;
+  // operand rows of this lane: weight rows (wn WN + i) * 32 + r32, token rows BN + (wm WM + j) * 32 + r32;
+  // piece kk * 2 + h of a row sits in slot (kk * 2 + h) ^ (row % 8), and row % 8 == r32 % 8 for all of them
+  const int swz = r32 % 8;
+  const int a_base = (wn * 32 * WN + r32) * 128;
+  const int b_base = (BN + wm * 32 * WM + r32) * 128;
+  struct Fragments {
+    bf16x8_t a[WN], b[WM];
+  };
+  auto read = [&](int buf, int kk) {
+    Fragments f;
+    const unsigned char* base = smem + buf * kBufferBytes + (((kk * 2 + h) ^ swz) * 16);
+#pragma unroll
+    for (int i = 0; i < WN; ++i) f.a[i] = load_bf16x8(base + a_base + i * 32 * 128);
+#pragma unroll
+    for (int j = 0; j < WM; ++j) f.b[j] = load_bf16x8(base + b_base + j * 32 * 128);
+    return f;
+  };
+  auto multiply = [&](const Fragments& f) {
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) acc[i][j] = mfma_32x32x16(f.a[i], f.b[j], acc[i][j]);
+  };
+
+  fetch(s_begin, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  fetch(s_begin + 1, 1);
+  Fragments cur = read(0, 0);
+  int buf = 0;
+  for (int s = s_begin; s < s_end; ++s, buf ^= 1) {
+    Fragments kept[KEEP];
+    if (!idle) {
+#pragma unroll
+      for (int kk = 0; kk < kBK / 16 - KEEP; ++kk) {
+        const Fragments next = read(buf, kk + 1);
+        multiply(cur);
+        cur = next;
+      }
+      kept[0] = cur;
+#pragma unroll
+      for (int e = 1; e < KEEP; ++e) kept[e] = read(buf, kBK / 16 - KEEP + e);
+    }
+    // the slice after this one has landed (this wavefront's share; the barrier answers for the others),
+    // and nobody reads this slice's buffer any more
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    fetch(s + 2, buf);
+    if (!idle) {
+      cur = read(buf ^ 1, 0);
+#pragma unroll
+      for (int e = 0; e < KEEP; ++e) multiply(kept[e]);  // the part kept for behind the barrier
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be on its way into LDS when the workgroup ends
+
+  if (ep.row_sumsq != nullptr) {
+    row_scales_finish(ep, owed, m0, BM, M, K, scales);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j) {
+      const int m = m0 + (wm * WM + j) * 32 + r32;
+      const float scale = ep.row_sumsq != nullptr ? scales[(wm * WM + j) * 32 + r32] : 1.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + (wn * WN + i) * 32 + g * 8 + h * 4;
+        const float v[4] = {acc[i][j][g * 4 + 0] * scale, acc[i][j][g * 4 + 1] * scale, acc[i][j][g * 4 + 2] * scale,
+                            acc[i][j][g * 4 + 3] * scale};
+        finish4(ep, slice, slices, m, n, M, N, v);
+      }
+    }
+}
+
+
+using DirectKernel = void (*)(const bf16*, const bf16*, GemmEpilogue, TileOrder, int, int, int);
+// `wave_rows`: rows of wavefronts in the tile (a last token tile that fills only the first is light)
+static int launch_direct(DirectKernel kernel, int tile, int threads, int wave_rows, bool& configured, const bf16* xb,
+                         const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices, hipStream_t stream) {
+  const TileOrder order = make_tile_order(m, (n + tile - 1) / tile, slices, tile, wave_rows);
+  const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles * slices;
+  if (groups >= (1ll << 31)) {
+    set_error("mlr_gemm_bf16: too many tiles for one launch");
+    return -1;
+  }
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       direct_lds_bytes(tile));
+    if (e != hipSuccess) {
+      set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
+      return -1;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups)), dim3(threads), direct_lds_bytes(tile), stream, xb, wb, ep,
+                     order, m, n, k);
+  return 0;
+}
+
 // ONCE: the tokens fit one tile, so every weight byte is read once; the kernel then loads the
 // weights with the non-temporal hint (measured on matrices far larger than the caches, as a
 // model's layers are to each other: 7B gate-up at 8 tokens 50.7 to 45.4 us, the output head 191
@@ -646,6 +832,10 @@ static bool half_rows_fill_better(int blocks16) {
 // at five model sizes (hidden 896 to 5120) and 96 to 2,048 tokens, with weights that rotate
 // through more memory than the caches hold: rms error of the estimate 8 %, the chosen pair within
 // 1 % of the best one on average, where rules on tile counts had been 8 % off and up to 76 %.
+// (Fitted with the register-staged kernels.  The two larger tilings now run gemm_direct_kernel, whose
+// steps measured 4 % shorter on such weights (128 to 2,048 tokens, 0.5B and 7B gate-up and down: 0 to
+// 10 % with 128 x 128 tiles, 1 to 7 % with 256 x 256); the 64 x 64 tiling keeps the staged kernel, which
+// has two slices of k on their way and streams weights faster at up to some 500 tokens.)
 struct GemmPlan {
   int kernel, slices;
 };
@@ -654,7 +844,7 @@ struct TilingCost {
   float alone, busy, fixed;
 };
 constexpr TilingCost kTilingCosts[] = {
-    {11, 64, 8, 0.401f, 0.251f, 6.4f}, {22, 128, 2, 0.966f, 0.603f, 6.5f}, {44, 256, 1, 1.15f, 1.937f, 10.5f}};
+    {11, 64, 8, 0.401f, 0.251f, 6.4f}, {23, 128, 2, 0.927f, 0.579f, 6.5f}, {45, 256, 1, 1.09f, 1.84f, 10.5f}};
 constexpr int kComputeUnits = 256;
 static float tiled_time_us(const TilingCost& c, int m, int n, int k, int slices) {
   const int64_t tiles = static_cast<int64_t>((m + c.tile - 1) / c.tile) * ((n + c.tile - 1) / c.tile);
@@ -689,7 +879,8 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 }
 
 // The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,
-// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 14 = gemm_tiled
+// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 13 / 23 / 45 = gemm_direct
+// with the same three, 14 = gemm_tiled
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
 // rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 12 = gemm_tiled with tiles of 64
 // tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products, 15 = gemm_tiled with
@@ -761,7 +952,19 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
     case 15: return launch_tiled<1, 5, 2, 1>(xb, wb, ep, m, n, k, slices, stream);  // 64 tokens x 160 features
     case 22: return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
     case 44: return launch_tiled<2, 2, 4, 4>(xb, wb, ep, m, n, k, slices, stream);
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 22 or 44"); return -1;
+    case 45: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 4>, 256, 1024, 4, configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 23: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 256, 2, configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 13: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 2>, 64, 256, 2, configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 13, 22, 23, 44 or 45"); return -1;
   }
 }
 

@@ -233,13 +233,13 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 22, 44])
+@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 13, 22, 23, 44, 45])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
     shorter than an LDS slice, whole and cut along k."""
     ops = ops_for(torch.bfloat16)
-    m, n, k = (13 if kernel == 16 else (300 if kernel == 44 else 150)), (203 if kernel != 44 else 530), 1208
+    m, n, k = (13 if kernel == 16 else (300 if kernel in (44, 45) else 150)), (203 if kernel not in (44, 45) else 530), 1208
     x = _rand((m, k), torch.bfloat16, 61)
     w = _rand((n, k), torch.bfloat16, 62, 0.05)
     b = _rand((n,), torch.float32, 63)
@@ -254,7 +254,9 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
 
 
 @pytest.mark.parametrize("kernel,m,n", [(44, 2080, 1100), (44, 530, 3000), (44, 257, 256), (22, 1050, 700), (11, 532, 2373),
-                                        (11, 90, 640), (12, 80, 1000), (44, 2112, 520), (44, 2113, 520)])
+                                        (11, 90, 640), (12, 80, 1000), (44, 2112, 520), (44, 2113, 520), (45, 2080, 1100),
+                                        (45, 530, 3000), (45, 257, 256), (23, 1050, 700), (13, 532, 2373), (13, 90, 640),
+                                        (45, 2112, 520), (45, 2113, 520)])
 @pytest.mark.parametrize("slices", [1, 2])
 def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
     """A last token tile whose tokens fit the first row of wavefronts (a prompt portion beside a few
