@@ -551,8 +551,9 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 // in a GM x GN arrangement) with two changes to what a step of k costs beside its products.  The tiles
 // go from memory into LDS without passing registers (a lane's 16 bytes land at wavefront base + 16 *
 // lane, so rows are 128 bytes without padding, and a row's eight 16-byte pieces are stored in the
-// order piece ^ (row % 8): the operand reads of eight consecutive rows then fall into eight different
-// piece slots).  And the barrier of a step stands before its last quarter of products: behind it every
+// order piece ^ ((row / 2) % 8): LDS serves sixteen lanes' 16 bytes a cycle from 64 banks, two rows' worth, so
+// the operand reads of sixteen consecutive rows then fall on sixteen different places; with row % 8 as
+// the key a third of the kernel's time went to bank conflicts).  And the barrier of a step stands before its last quarter of products: behind it every
 // wavefront first asks for the next slice's first operands and for the slice after that, then
 // multiplies the quarter it kept, so the matrix cores have work while those arrive.  (KEEP: quarters
 // kept; two cost registers and gained nothing.  Eight wavefronts of 128 x 64 or 64 x 128 on the
@@ -599,9 +600,9 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   const __amdgpu_buffer_rsrc_t w_buf = make_buffer(w + static_cast<int64_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2u);
   const __amdgpu_buffer_rsrc_t x_buf = make_buffer(x + static_cast<int64_t>(m0) * K, static_cast<unsigned>(x_rows) * K * 2u);
   // piece p of this wavefront fills rows 8 * (WAVES p + wave) .. + 7 of a buffer (its first half: weights,
-  // its second: tokens): lane l brings row + l / 8, piece (l % 8) ^ (l / 8) to slot l % 8
+  // its second: tokens): lane l brings row + l / 8, piece (l % 8) ^ key to slot l % 8, key = (row / 2) % 8
   const int lane_row = lane / 8;
-  const int lane_chunk = (lane % 8) ^ lane_row;
+  const int lane_chunk = (lane % 8) ^ ((4 * wave + lane_row / 2) % 8);  // ((row / 2) % 8 of the row it fills)
   unsigned piece_off[kMostPieces];
 #pragma unroll
   for (int p = 0; p < kMostPieces; ++p) {
@@ -630,8 +631,8 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
 
   const bool idle = __builtin_amdgcn_readfirstlane(static_cast<int>(wm * 32 * WM >= x_rows)) != 0;
   // operand rows of this lane: weight rows (wn WN + i) * 32 + r32, token rows BN + (wm WM + j) * 32 + r32;
-  // piece kk * 2 + h of a row sits in slot (kk * 2 + h) ^ (row % 8), and row % 8 == r32 % 8 for all of them
-  const int swz = r32 % 8;
+  // piece kk * 2 + h of a row sits in slot (kk * 2 + h) ^ ((row / 2) % 8), and that key is (r32 / 2) % 8 for all of them
+  const int swz = (r32 / 2) % 8;
   const int a_base = (wn * 32 * WN + r32) * 128;
   const int b_base = (BN + wm * 32 * WM + r32) * 128;
   struct Fragments {
