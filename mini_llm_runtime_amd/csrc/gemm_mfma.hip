@@ -556,24 +556,35 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 // the key a third of the kernel's time went to bank conflicts).  And the barrier of a step stands before its last quarter of products: behind it every
 // wavefront first asks for the next slice's first operands and for the slice after that, then
 // multiplies the quarter it kept, so the matrix cores have work while those arrive.  (KEEP: quarters
-// kept; two cost registers and gained nothing.  Eight wavefronts of 128 x 64 or 64 x 128 on the
+// kept; two cost registers and gained nothing.  BKT, NBUF: width of a slice and LDS buffers, NBUF - 1
+// slices on their way; slices of 32 in four buffers, or of 64 in three on the 128 x 128 tile, were 5 to
+// 25 % slower from 512 tokens on and up to 16 % faster at 128 to 256, where other tilings are chosen.
+// A 64 x 64 tile this way was 7 to 15 % slower than the staged kernel at up to 512 tokens of weights
+// that come from memory, equal beyond.  Eight wavefronts of 128 x 64 or 64 x 128 on the
 // 256 x 256 tile ran like sixteen of 64 x 64; sixteen of 32 x 32 on the 128 x 128 tile slower than four.)
 // Measured against the register-staged kernel on one matrix streamed again and again: 7B gate-up at
 // 2,048 tokens 592 to 527 us (hipBLASLt: 584), 7B down in two slices 262 to 247, 32B down in three
 // slices 541 to 493, 0.5B gate-up 57 to 51 (the library: 53); on a model's weights, which come from
 // memory, 1 to 10 %.
-constexpr int direct_lds_bytes(int tile) { return 2 * 2 * tile * kBK * 2; }  // two buffers of (tile + tile) rows x 128 bytes
+constexpr int direct_lds_bytes(int tile, int bk, int buffers) { return buffers * 2 * tile * bk * 2; }  // (tile + tile) rows of bk
 
-template <int KEEP, int WM, int WN, int GM, int GN>
+template <int KEEP, int WM, int WN, int GM, int GN, int BKT = kBK, int NBUF = 2>
 __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                                   GemmEpilogue ep, TileOrder order, int M, int N, int K) {
   constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN, WAVES = GM * GN;
   static_assert(BM == BN, "square tiles");
-  constexpr int kRuns = (BM + BN) / 8;  // 1 KB runs (8 rows) of a buffer, dealt out to the wavefronts in turn
-  constexpr int kMostPieces = 8;        // at most this many per wavefront
+  constexpr int kRowBytes = BKT * 2;            // 128 or 64
+  constexpr int kRowPieces = BKT / 8;           // 16-byte pieces of a row
+  constexpr int kRunRows = 1024 / kRowBytes;    // rows of a 1 KB run, the unit a wavefront loads
+  constexpr int kBankRows = 256 / kRowBytes;    // rows that LDS serves side by side in one cycle
+  constexpr int kRuns = (BM + BN) / kRunRows;   // dealt out to the wavefronts in turn
+  constexpr int kMostPieces = 8;                // at most this many per wavefront
+  constexpr int kSteps = BKT / 16;              // products of k = 16 per slice
   static_assert(kRuns % WAVES == 0 && kRuns / WAVES <= kMostPieces && kRuns / 2 % WAVES == 0, "the wavefronts share a buffer's runs evenly");
+  static_assert(WAVES % 2 == 0 && KEEP >= 1 && KEEP < kSteps + 1 && NBUF >= 2, "see the swizzle key and the loop");
+  constexpr int kInFlight = (NBUF - 2) * (kRuns / WAVES);  // loads of this wavefront that may still be out when a slice is needed
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  constexpr int kBufferBytes = (BM + BN) * kBK * 2;
+  constexpr int kBufferBytes = (BM + BN) * kRowBytes;
   __shared__ float scales[BM];
 
   const int tid = threadIdx.x;
@@ -591,7 +602,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, m0, BM, M);
   const int chunks = K / 8;
   const int slices = order.slices;
-  const int k_slices = (K + kBK - 1) / kBK;
+  const int k_slices = (K + BKT - 1) / BKT;
   const int per = (k_slices + slices - 1) / slices;
   const int s_begin = slice * per;
   const int s_end = min(k_slices, s_begin + per);
@@ -599,25 +610,26 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   const int w_rows = min(BN, N - n0), x_rows = min(BM, M - m0);
   const __amdgpu_buffer_rsrc_t w_buf = make_buffer(w + static_cast<int64_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2u);
   const __amdgpu_buffer_rsrc_t x_buf = make_buffer(x + static_cast<int64_t>(m0) * K, static_cast<unsigned>(x_rows) * K * 2u);
-  // piece p of this wavefront fills rows 8 * (WAVES p + wave) .. + 7 of a buffer (its first half: weights,
-  // its second: tokens): lane l brings row + l / 8, piece (l % 8) ^ key to slot l % 8, key = (row / 2) % 8
-  const int lane_row = lane / 8;
-  const int lane_chunk = (lane % 8) ^ ((4 * wave + lane_row / 2) % 8);  // ((row / 2) % 8 of the row it fills)
+  // piece p of this wavefront fills the run of rows kRunRows * (WAVES p + wave) .. of a buffer (its first
+  // half: weights, its second: tokens): lane l brings row + l / kRowPieces, piece (l % kRowPieces) ^ key to
+  // slot l % kRowPieces, key = (row / kBankRows) % kRowPieces (the same for every p)
+  const int lane_row = lane / kRowPieces;
+  const int lane_chunk = (lane % kRowPieces) ^ (((kRunRows / kBankRows) * wave + lane_row / kBankRows) % kRowPieces);
   unsigned piece_off[kMostPieces];
 #pragma unroll
   for (int p = 0; p < kMostPieces; ++p) {
-    const int row = 8 * (WAVES * p + wave) + lane_row;  // first half of the pieces: weight rows, second: token rows
+    const int row = kRunRows * (WAVES * p + wave) + lane_row;  // first half of the pieces: weight rows, second: token rows
     piece_off[p] = static_cast<unsigned>(row % BN) * K * 2u + lane_chunk * 16u;
   }
   auto fetch = [&](int s, int buf) {
-    const int left = s < s_end ? chunks - s * (kBK / 8) : 0;
+    const int left = s < s_end ? chunks - s * kRowPieces : 0;
     const unsigned off_ok = lane_chunk < left ? 0u : kOutOfBuffer;
 #pragma unroll
     for (int p = 0; p < kMostPieces; ++p) {
       if (p * WAVES >= kRuns) break;
       __attribute__((address_space(3))) void* dst =
           (__attribute__((address_space(3))) void*)(smem + buf * kBufferBytes + (WAVES * p + wave) * 1024);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(p * WAVES < kRuns / 2 ? w_buf : x_buf, dst, 16, (piece_off[p] + s * (kBK * 2u)) | off_ok, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(p * WAVES < kRuns / 2 ? w_buf : x_buf, dst, 16, (piece_off[p] + s * (BKT * 2u)) | off_ok, 0, 0, 0);
     }
   };
 
@@ -631,10 +643,10 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
 
   const bool idle = __builtin_amdgcn_readfirstlane(static_cast<int>(wm * 32 * WM >= x_rows)) != 0;
   // operand rows of this lane: weight rows (wn WN + i) * 32 + r32, token rows BN + (wm WM + j) * 32 + r32;
-  // piece kk * 2 + h of a row sits in slot (kk * 2 + h) ^ ((row / 2) % 8), and that key is (r32 / 2) % 8 for all of them
-  const int swz = (r32 / 2) % 8;
-  const int a_base = (wn * 32 * WN + r32) * 128;
-  const int b_base = (BN + wm * 32 * WM + r32) * 128;
+  // piece kk * 2 + h of a row sits in slot (kk * 2 + h) ^ key, and the key is (r32 / kBankRows) % kRowPieces for all of them
+  const int swz = (r32 / kBankRows) % kRowPieces;
+  const int a_base = (wn * 32 * WN + r32) * kRowBytes;
+  const int b_base = (BN + wm * 32 * WM + r32) * kRowBytes;
   struct Fragments {
     bf16x8_t a[WN], b[WM];
   };
@@ -642,9 +654,9 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
     Fragments f;
     const unsigned char* base = smem + buf * kBufferBytes + (((kk * 2 + h) ^ swz) * 16);
 #pragma unroll
-    for (int i = 0; i < WN; ++i) f.a[i] = load_bf16x8(base + a_base + i * 32 * 128);
+    for (int i = 0; i < WN; ++i) f.a[i] = load_bf16x8(base + a_base + i * 32 * kRowBytes);
 #pragma unroll
-    for (int j = 0; j < WM; ++j) f.b[j] = load_bf16x8(base + b_base + j * 32 * 128);
+    for (int j = 0; j < WM; ++j) f.b[j] = load_bf16x8(base + b_base + j * 32 * kRowBytes);
     return f;
   };
   auto multiply = [&](const Fragments& f) {
@@ -654,35 +666,38 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
       for (int j = 0; j < WM; ++j) acc[i][j] = mfma_32x32x16(f.a[i], f.b[j], acc[i][j]);
   };
 
-  fetch(s_begin, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // NBUF - 1 slices are on their way or in LDS ahead of the one that is multiplied
+#pragma unroll
+  for (int b = 0; b < NBUF; ++b) fetch(s_begin + b, b);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 1) * (kRuns / WAVES)) : "memory");
   __syncthreads();
-  fetch(s_begin + 1, 1);
   Fragments cur = read(0, 0);
   int buf = 0;
-  for (int s = s_begin; s < s_end; ++s, buf ^= 1) {
+  for (int s = s_begin; s < s_end; ++s) {
     Fragments kept[KEEP];
     if (!idle) {
 #pragma unroll
-      for (int kk = 0; kk < kBK / 16 - KEEP; ++kk) {
+      for (int kk = 0; kk < kSteps - KEEP; ++kk) {
         const Fragments next = read(buf, kk + 1);
         multiply(cur);
         cur = next;
       }
       kept[0] = cur;
 #pragma unroll
-      for (int e = 1; e < KEEP; ++e) kept[e] = read(buf, kBK / 16 - KEEP + e);
+      for (int e = 1; e < KEEP; ++e) kept[e] = read(buf, kSteps - KEEP + e);
     }
     // the slice after this one has landed (this wavefront's share; the barrier answers for the others),
     // and nobody reads this slice's buffer any more
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kInFlight) : "memory");
     __syncthreads();
-    fetch(s + 2, buf);
+    fetch(s + NBUF, buf);
+    const int next_buf = buf + 1 == NBUF ? 0 : buf + 1;
     if (!idle) {
-      cur = read(buf ^ 1, 0);
+      cur = read(next_buf, 0);
 #pragma unroll
       for (int e = 0; e < KEEP; ++e) multiply(kept[e]);  // the part kept for behind the barrier
     }
+    buf = next_buf;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be on its way into LDS when the workgroup ends
 
@@ -706,11 +721,11 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
     }
 }
 
-
 using DirectKernel = void (*)(const bf16*, const bf16*, GemmEpilogue, TileOrder, int, int, int);
 // `wave_rows`: rows of wavefronts in the tile (a last token tile that fills only the first is light)
-static int launch_direct(DirectKernel kernel, int tile, int threads, int wave_rows, bool& configured, const bf16* xb,
-                         const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices, hipStream_t stream) {
+static int launch_direct(DirectKernel kernel, int tile, int threads, int wave_rows, int lds_bytes, bool& configured,
+                         const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
+                         hipStream_t stream) {
   const TileOrder order = make_tile_order(m, (n + tile - 1) / tile, slices, tile, wave_rows);
   const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles * slices;
   if (groups >= (1ll << 31)) {
@@ -718,16 +733,14 @@ static int launch_direct(DirectKernel kernel, int tile, int threads, int wave_ro
     return -1;
   }
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       direct_lds_bytes(tile));
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) {
       set_error(std::string("mlr_gemm_bf16: cannot raise the LDS limit: ") + hipGetErrorString(e));
       return -1;
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups)), dim3(threads), direct_lds_bytes(tile), stream, xb, wb, ep,
-                     order, m, n, k);
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups)), dim3(threads), lds_bytes, stream, xb, wb, ep, order, m, n, k);
   return 0;
 }
 
@@ -880,8 +893,8 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 }
 
 // The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,
-// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 13 / 23 / 45 = gemm_direct
-// with the same three, 14 = gemm_tiled
+// 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 23 / 45 = gemm_direct
+// with the two larger ones, 14 = gemm_tiled
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
 // rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 12 = gemm_tiled with tiles of 64
 // tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products, 15 = gemm_tiled with
@@ -955,17 +968,15 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
     case 44: return launch_tiled<2, 2, 4, 4>(xb, wb, ep, m, n, k, slices, stream);
     case 45: {
       static bool configured = false;
-      return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 4>, 256, 1024, 4, configured, xb, wb, ep, m, n, k, slices, stream);
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 4>, 256, 1024, 4, direct_lds_bytes(256, 64, 2), configured, xb, wb, ep,
+                           m, n, k, slices, stream);
     }
     case 23: {
       static bool configured = false;
-      return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 256, 2, configured, xb, wb, ep, m, n, k, slices, stream);
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 256, 2, direct_lds_bytes(128, 64, 2), configured, xb, wb, ep,
+                           m, n, k, slices, stream);
     }
-    case 13: {
-      static bool configured = false;
-      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 2>, 64, 256, 2, configured, xb, wb, ep, m, n, k, slices, stream);
-    }
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 13, 22, 23, 44 or 45"); return -1;
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 22, 23, 44 or 45"); return -1;
   }
 }
 

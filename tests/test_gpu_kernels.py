@@ -233,7 +233,7 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 13, 22, 23, 44, 45])
+@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 22, 23, 44, 45])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
@@ -255,7 +255,7 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
 
 @pytest.mark.parametrize("kernel,m,n", [(44, 2080, 1100), (44, 530, 3000), (44, 257, 256), (22, 1050, 700), (11, 532, 2373),
                                         (11, 90, 640), (12, 80, 1000), (44, 2112, 520), (44, 2113, 520), (45, 2080, 1100),
-                                        (45, 530, 3000), (45, 257, 256), (23, 1050, 700), (13, 532, 2373), (13, 90, 640),
+                                        (45, 530, 3000), (45, 257, 256), (23, 1050, 700), (23, 532, 2373), (23, 140, 640),
                                         (45, 2112, 520), (45, 2113, 520)])
 @pytest.mark.parametrize("slices", [1, 2])
 def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
