@@ -547,25 +547,26 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 }
 
 // ---- tiled, tiles loaded straight into LDS ---------------------------------------------------------
-// The square tiles of gemm_tiled_kernel (64, 128 or 256 on a side, wavefronts of WM x WN blocks of 32 x 32
-// in a GM x GN arrangement) with two changes to what a step of k costs beside its products.  The tiles
-// go from memory into LDS without passing registers (a lane's 16 bytes land at wavefront base + 16 *
-// lane, so rows are 128 bytes without padding, and a row's eight 16-byte pieces are stored in the
-// order piece ^ ((row / 2) % 8): LDS serves sixteen lanes' 16 bytes a cycle from 64 banks, two rows' worth, so
-// the operand reads of sixteen consecutive rows then fall on sixteen different places; with row % 8 as
-// the key a third of the kernel's time went to bank conflicts).  And the barrier of a step stands before its last quarter of products: behind it every
-// wavefront first asks for the next slice's first operands and for the slice after that, then
-// multiplies the quarter it kept, so the matrix cores have work while those arrive.  (KEEP: quarters
-// kept; two cost registers and gained nothing.  BKT, NBUF: width of a slice and LDS buffers, NBUF - 1
-// slices on their way; slices of 32 in four buffers, or of 64 in three on the 128 x 128 tile, were 5 to
-// 25 % slower from 512 tokens on and up to 16 % faster at 128 to 256, where other tilings are chosen.
-// A 64 x 64 tile this way was 7 to 15 % slower than the staged kernel at up to 512 tokens of weights
-// that come from memory, equal beyond.  Eight wavefronts of 128 x 64 or 64 x 128 on the
-// 256 x 256 tile ran like sixteen of 64 x 64; sixteen of 32 x 32 on the 128 x 128 tile slower than four.)
+// The square tiles of gemm_tiled_kernel (wavefronts of WM x WN blocks of 32 x 32 in a GM x GN arrangement)
+// with two changes to what a step of k costs beside its products.
+//  * The tiles go from memory into LDS without passing registers.  A lane's 16 bytes land at wavefront
+//    base + 16 * lane, so a row of a slice (BKT * 2 bytes) has no padding; instead its 16-byte pieces
+//    are stored in the order piece ^ key.  LDS serves sixteen lanes' 16 bytes a cycle from 64 banks
+//    (256 bytes: two rows of a 64-wide slice), so the key is (row / 2) % 8 there: the operand reads of
+//    sixteen consecutive rows fall on sixteen different places.  (With row % 8 as the key the bank
+//    conflict counter showed a third of the kernel's cycles.)
+//  * The one barrier of a step stands before its last quarter of products: behind it every wavefront
+//    first asks for the next slice's first operands and for the slice NBUF slices on, then multiplies
+//    the quarter it kept, so the matrix cores have work while those arrive.
 // Measured against the register-staged kernel on one matrix streamed again and again: 7B gate-up at
-// 2,048 tokens 592 to 527 us (hipBLASLt: 584), 7B down in two slices 262 to 247, 32B down in three
-// slices 541 to 493, 0.5B gate-up 57 to 51 (the library: 53); on a model's weights, which come from
-// memory, 1 to 10 %.
+// 2,048 tokens 592 to 527 us (the vendor library: 584), 7B down in two slices 262 to 247, 32B down in
+// three slices 541 to 493, 0.5B gate-up 57 to 51 (the library: 53); on a model's weights, which come
+// from memory, 1 to 10 %.  Variants that lost: two quarters kept (KEEP 2: spills a register, no gain);
+// slices of 32 in four buffers or of 64 in three (BKT, NBUF; NBUF - 1 slices on their way: 5 to 25 %
+// slower from 512 tokens on, up to 16 % faster at 128 to 256, where other tilings are chosen); a 64 x 64
+// tile (7 to 15 % slower than the staged kernel, which has two slices on their way, at up to 512 tokens
+// of weights that come from memory; equal beyond); eight wavefronts of 128 x 64 or 64 x 128 on the
+// 256 x 256 tile (like sixteen of 64 x 64); sixteen of 32 x 32 on the 128 x 128 tile (slower than four).
 constexpr int direct_lds_bytes(int tile, int bk, int buffers) { return buffers * 2 * tile * bk * 2; }  // (tile + tile) rows of bk
 
 template <int KEEP, int WM, int WN, int GM, int GN, int BKT = kBK, int NBUF = 2>
@@ -578,6 +579,8 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   constexpr int kRunRows = 1024 / kRowBytes;    // rows of a 1 KB run, the unit a wavefront loads
   constexpr int kBankRows = 256 / kRowBytes;    // rows that LDS serves side by side in one cycle
   constexpr int kRuns = (BM + BN) / kRunRows;   // dealt out to the wavefronts in turn
+  // (loops over a wavefront's runs go to this fixed bound and break: with a bound that depends on the
+  // template's parameters the host pass left the kernel uninstantiated, without a message)
   constexpr int kMostPieces = 8;                // at most this many per wavefront
   constexpr int kSteps = BKT / 16;              // products of k = 16 per slice
   static_assert(kRuns % WAVES == 0 && kRuns / WAVES <= kMostPieces && kRuns / 2 % WAVES == 0, "the wavefronts share a buffer's runs evenly");
