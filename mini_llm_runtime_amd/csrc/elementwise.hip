@@ -5,6 +5,7 @@
 #define MLR_ERROR_CHANNEL
 #include "api.h"
 #include "common.h"
+#include "mfma.h"
 
 namespace mlr {
 
@@ -280,6 +281,69 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   }
 }
 
+// The same for bfloat16 with the whole head rotated and a head size that is a multiple of 16: a thread
+// takes 8 dims of the first half of a head and their 8 partners in 16-byte loads and stores (2,048 tokens
+// of the 7B shape: 17.7 to 15.6 us; what is left is the values' scatter into their transposed pages,
+// 2 bytes at a stride of a page row).
+__global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(
+    bf16* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ slots, bf16* __restrict__ key_pages, bf16* __restrict__ value_pages, int heads, int kv_heads,
+    int head_dim, int block_size, int num_pages, int write) {
+  const int t = blockIdx.x;
+  const int half = head_dim / 2;
+  const int per_head = half / 8;  // pairs of 16-byte pieces
+  const int64_t width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  bf16* q = qkv + t * width;
+  bf16* v = q + static_cast<int64_t>(heads + kv_heads) * head_dim;
+  const float* cs = cos_t + static_cast<int64_t>(t) * half;
+  const float* sn = sin_t + static_cast<int64_t>(t) * half;
+
+  int64_t page_base = -1, value_base = -1;  // as in rope_kv_write_kernel
+  const int64_t head_stride = static_cast<int64_t>(block_size) * head_dim;
+  if (write) {
+    const int slot = slots[t];
+    if (slot >= 0) {
+      const int page = slot / block_size;
+      const int off = slot - page * block_size;
+      if (page < num_pages) {
+        page_base = (static_cast<int64_t>(page) * kv_heads * block_size + off) * head_dim;
+        value_base = static_cast<int64_t>(page) * kv_heads * head_stride + off;
+      }
+    }
+  }
+  for (int i = threadIdx.x; i < (heads + kv_heads) * per_head; i += blockDim.x) {
+    const int h = i / per_head;  // query heads first, then key heads: they lie behind one another in the row
+    const int j = (i - h * per_head) * 8;
+    bf16* p = q + static_cast<int64_t>(h) * head_dim;
+    const u16x8_t lo = *reinterpret_cast<const u16x8_t*>(p + j);
+    const u16x8_t hi = *reinterpret_cast<const u16x8_t*>(p + j + half);
+    const f32x4_t c0 = *reinterpret_cast<const f32x4_t*>(cs + j), c1 = *reinterpret_cast<const f32x4_t*>(cs + j + 4);
+    const f32x4_t s0 = *reinterpret_cast<const f32x4_t*>(sn + j), s1 = *reinterpret_cast<const f32x4_t*>(sn + j + 4);
+    u16x8_t out_lo, out_hi;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float a = to_f32(bf16{lo[e]}), b = to_f32(bf16{hi[e]});
+      const float c = e < 4 ? c0[e] : c1[e - 4], sv = e < 4 ? s0[e] : s1[e - 4];
+      out_lo[e] = f32_to_bf16(a * c - b * sv).bits;
+      out_hi[e] = f32_to_bf16(b * c + a * sv).bits;
+    }
+    *reinterpret_cast<u16x8_t*>(p + j) = out_lo;
+    *reinterpret_cast<u16x8_t*>(p + j + half) = out_hi;
+    if (h >= heads && page_base >= 0) {
+      bf16* dst = key_pages + page_base + (h - heads) * head_stride;
+      *reinterpret_cast<u16x8_t*>(dst + j) = out_lo;
+      *reinterpret_cast<u16x8_t*>(dst + j + half) = out_hi;
+    }
+  }
+  if (page_base >= 0) {
+    for (int i = threadIdx.x; i < kv_heads * head_dim; i += blockDim.x) {
+      const int h = i / head_dim;
+      const int j = i - h * head_dim;
+      value_pages[value_base + h * head_stride + static_cast<int64_t>(j) * block_size] = v[h * head_dim + j];
+    }
+  }
+}
+
 // ---- the query/key/value product that came as K slices -----------------------------------------
 // A wide product of few tokens streams its weights fastest through the LDS-tiled kernel cut
 // along K, which leaves float32 partial sums [slice, token, width] (the bias in slice 0).  This
@@ -476,6 +540,12 @@ int mlr_rope_kv_write(void* qkv, int dtype, const float* cos, const float* sin, 
     rope_kv_write_kernel<float><<<tokens, 256, 0, stream>>>(
         static_cast<float*>(qkv), cos, sin, slots, static_cast<float*>(key_pages),
         static_cast<float*>(value_pages), heads, kv_heads, head_dim, rotary_dim, block_size, num_pages, write);
+  else if (rotary_dim == head_dim && head_dim % 16 == 0 && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(cos) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(sin) % 16 == 0)
+    rope_kv_write_bf16x8_kernel<<<tokens, 256, 0, stream>>>(
+        static_cast<bf16*>(qkv), cos, sin, slots, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages), heads,
+        kv_heads, head_dim, block_size, num_pages, write);
   else
     rope_kv_write_kernel<bf16><<<tokens, 256, 0, stream>>>(
         static_cast<bf16*>(qkv), cos, sin, slots, static_cast<bf16*>(key_pages),

@@ -336,7 +336,8 @@ def test_rope_table(ops_for):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary", [(4, 2, 16, 16), (3, 1, 32, 32), (14, 2, 64, 64), (8, 8, 128, 64), (2, 1, 48, 48)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary", [(4, 2, 16, 16), (3, 1, 32, 32), (14, 2, 64, 64), (8, 8, 128, 64), (2, 1, 48, 48),
+                                                         (28, 4, 128, 128), (5, 1, 80, 80), (3, 2, 20, 20)])
 def test_rope_kv_write(ops_for, dtype, heads, kv_heads, head_dim, rotary):
     ops = ops_for(dtype)
     tokens, bs, pages = 11, 8, 9
