@@ -567,27 +567,36 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 // tile (7 to 15 % slower than the staged kernel, which has two slices on their way, at up to 512 tokens
 // of weights that come from memory; equal beyond); eight wavefronts of 128 x 64 or 64 x 128 on the
 // 256 x 256 tile (like sixteen of 64 x 64); sixteen of 32 x 32 on the 128 x 128 tile (slower than four).
-constexpr int direct_lds_bytes(int tile, int bk, int buffers) { return buffers * 2 * tile * bk * 2; }  // (tile + tile) rows of bk
+// LDS of a tile of `tokens` x `features` under `waves` wavefronts: every wavefront fills the same number
+// of 1 KB runs per buffer, so a buffer has room for whole rounds of them.
+constexpr int direct_lds_bytes(int tokens, int features, int waves, int bk, int buffers) {
+  const int runs = (tokens + features) * bk * 2 / 1024;
+  return buffers * ((runs + waves - 1) / waves) * waves * 1024;
+}
 
 template <int KEEP, int WM, int WN, int GM, int GN, int BKT = kBK, int NBUF = 2>
 __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                                   GemmEpilogue ep, TileOrder order, int M, int N, int K) {
   constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN, WAVES = GM * GN;
-  static_assert(BM == BN, "square tiles");
   constexpr int kRowBytes = BKT * 2;            // 128 or 64
   constexpr int kRowPieces = BKT / 8;           // 16-byte pieces of a row
   constexpr int kRunRows = 1024 / kRowBytes;    // rows of a 1 KB run, the unit a wavefront loads
   constexpr int kBankRows = 256 / kRowBytes;    // rows that LDS serves side by side in one cycle
   constexpr int kRuns = (BM + BN) / kRunRows;   // dealt out to the wavefronts in turn
+  constexpr int kWeightRuns = BN / kRunRows;    // the first of them are weight rows, the others token rows
+  // Every wavefront issues kPieces loads per slice (the wait counters count instructions); where the
+  // runs do not go round, the last wavefronts' surplus loads are out of range and bring zeros to slots
+  // of their own behind the tile.
+  constexpr int kPieces = (kRuns + WAVES - 1) / WAVES;
   // (loops over a wavefront's runs go to this fixed bound and break: with a bound that depends on the
   // template's parameters the host pass left the kernel uninstantiated, without a message)
   constexpr int kMostPieces = 8;                // at most this many per wavefront
   constexpr int kSteps = BKT / 16;              // products of k = 16 per slice
-  static_assert(kRuns % WAVES == 0 && kRuns / WAVES <= kMostPieces && kRuns / 2 % WAVES == 0, "the wavefronts share a buffer's runs evenly");
+  static_assert(kPieces <= kMostPieces && BN % 32 == 0 && BM % 32 == 0, "whole runs of weight rows and of token rows");
   static_assert(WAVES % 2 == 0 && KEEP >= 1 && KEEP < kSteps + 1 && NBUF >= 2, "see the swizzle key and the loop");
-  constexpr int kInFlight = (NBUF - 2) * (kRuns / WAVES);  // loads of this wavefront that may still be out when a slice is needed
+  constexpr int kInFlight = (NBUF - 2) * kPieces;  // loads of this wavefront that may still be out when a slice is needed
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  constexpr int kBufferBytes = (BM + BN) * kRowBytes;
+  constexpr int kBufferBytes = kPieces * WAVES * 1024;
   __shared__ float scales[BM];
 
   const int tid = threadIdx.x;
@@ -621,18 +630,20 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   unsigned piece_off[kMostPieces];
 #pragma unroll
   for (int p = 0; p < kMostPieces; ++p) {
-    const int row = kRunRows * (WAVES * p + wave) + lane_row;  // first half of the pieces: weight rows, second: token rows
-    piece_off[p] = static_cast<unsigned>(row % BN) * K * 2u + lane_chunk * 16u;
+    const int run = WAVES * p + wave;
+    const int row = kRunRows * run + lane_row;  // rows of the buffer: BN weight rows, then BM token rows
+    piece_off[p] = run >= kRuns ? kOutOfBuffer : static_cast<unsigned>(row < BN ? row : row - BN) * K * 2u + lane_chunk * 16u;
   }
   auto fetch = [&](int s, int buf) {
     const int left = s < s_end ? chunks - s * kRowPieces : 0;
     const unsigned off_ok = lane_chunk < left ? 0u : kOutOfBuffer;
 #pragma unroll
     for (int p = 0; p < kMostPieces; ++p) {
-      if (p * WAVES >= kRuns) break;
+      if (p >= kPieces) break;
       __attribute__((address_space(3))) void* dst =
           (__attribute__((address_space(3))) void*)(smem + buf * kBufferBytes + (WAVES * p + wave) * 1024);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(p * WAVES < kRuns / 2 ? w_buf : x_buf, dst, 16, (piece_off[p] + s * (BKT * 2u)) | off_ok, 0, 0, 0);
+      const bool weights = (p + 1) * WAVES <= kWeightRuns || (p * WAVES < kWeightRuns && WAVES * p + wave < kWeightRuns);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(weights ? w_buf : x_buf, dst, 16, (piece_off[p] + s * (BKT * 2u)) | off_ok, 0, 0, 0);
     }
   };
 
@@ -672,7 +683,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   // NBUF - 1 slices are on their way or in LDS ahead of the one that is multiplied
 #pragma unroll
   for (int b = 0; b < NBUF; ++b) fetch(s_begin + b, b);
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 1) * (kRuns / WAVES)) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 1) * kPieces) : "memory");
   __syncthreads();
   Fragments cur = read(0, 0);
   int buf = 0;
@@ -726,10 +737,10 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
 
 using DirectKernel = void (*)(const bf16*, const bf16*, GemmEpilogue, TileOrder, int, int, int);
 // `wave_rows`: rows of wavefronts in the tile (a last token tile that fills only the first is light)
-static int launch_direct(DirectKernel kernel, int tile, int threads, int wave_rows, int lds_bytes, bool& configured,
-                         const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
-                         hipStream_t stream) {
-  const TileOrder order = make_tile_order(m, (n + tile - 1) / tile, slices, tile, wave_rows);
+static int launch_direct(DirectKernel kernel, int tile_tokens, int tile_features, int threads, int wave_rows, int lds_bytes,
+                         bool& configured, const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k,
+                         int slices, hipStream_t stream) {
+  const TileOrder order = make_tile_order(m, (n + tile_features - 1) / tile_features, slices, tile_tokens, wave_rows);
   const int64_t groups = static_cast<int64_t>(order.m_tiles) * order.n_tiles * slices;
   if (groups >= (1ll << 31)) {
     set_error("mlr_gemm_bf16: too many tiles for one launch");
@@ -857,14 +868,24 @@ struct GemmPlan {
   int kernel, slices;
 };
 struct TilingCost {
-  int kernel, tile, resident;
+  int kernel, tile_tokens, tile_features, resident;
   float alone, busy, fixed;
 };
-constexpr TilingCost kTilingCosts[] = {
-    {11, 64, 8, 0.401f, 0.251f, 6.4f}, {23, 128, 2, 0.927f, 0.579f, 6.5f}, {45, 256, 1, 1.09f, 1.84f, 10.5f}};
+// The narrower tiles of 256 tokens (gemm_direct; a step of k costs 7.2 ns per feature of the tile at 256
+// features, 7.6 at 192, 8.4 at 160) are there for products whose 256 x 256 tiles leave compute units
+// without work or make a round for a few tiles.  Weights from memory, 2,048 tokens: 7B query/key/value
+// (4,608 features: 144 tiles, or 232 of 160 features) 92 to 80 us, 32B output projection (160 or 256
+// tiles) 130 to 112, 1.5B gate-up 139 to 132; 7B gate-up at 512 tokens 199 to 165.  Over the four
+// products of four model sizes at 256 to 4,096 tokens the chosen pairs add up to 0.6 % more than the
+// best pairs.  (256 x 224 by fourteen wavefronts was level with 256 x 256 and is not built.)
+constexpr TilingCost kTilingCosts[] = {{11, 64, 64, 8, 0.401f, 0.251f, 6.4f},
+                                       {23, 128, 128, 2, 0.927f, 0.579f, 6.5f},
+                                       {45, 256, 256, 1, 1.09f, 1.84f, 10.5f},
+                                       {46, 256, 192, 1, 0.86f, 1.45f, 10.5f},
+                                       {47, 256, 160, 1, 0.79f, 1.34f, 10.5f}};
 constexpr int kComputeUnits = 256;
 static float tiled_time_us(const TilingCost& c, int m, int n, int k, int slices) {
-  const int64_t tiles = static_cast<int64_t>((m + c.tile - 1) / c.tile) * ((n + c.tile - 1) / c.tile);
+  const int64_t tiles = static_cast<int64_t>((m + c.tile_tokens - 1) / c.tile_tokens) * ((n + c.tile_features - 1) / c.tile_features);
   const int64_t groups = tiles * slices;
   const int ksteps = (k + kBK - 1) / kBK;
   const float per = static_cast<float>((ksteps + slices - 1) / slices);
@@ -897,7 +918,8 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 
 // The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,
 // 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 23 / 45 = gemm_direct
-// with the two larger ones, 14 = gemm_tiled
+// with the two larger ones, 46 / 47 = gemm_direct with tiles of 256 tokens x 192 features (twelve
+// wavefronts of 64 x 64) and x 160 features (ten of 128 x 32), 14 = gemm_tiled
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
 // rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 12 = gemm_tiled with tiles of 64
 // tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products, 15 = gemm_tiled with
@@ -971,15 +993,25 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
     case 44: return launch_tiled<2, 2, 4, 4>(xb, wb, ep, m, n, k, slices, stream);
     case 45: {
       static bool configured = false;
-      return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 4>, 256, 1024, 4, direct_lds_bytes(256, 64, 2), configured, xb, wb, ep,
-                           m, n, k, slices, stream);
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 4>, 256, 256, 1024, 4, direct_lds_bytes(256, 256, 16, 64, 2), configured,
+                           xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 46: {  // 256 tokens x 192 features, twelve wavefronts of 64 x 64
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 3>, 256, 192, 768, 4, direct_lds_bytes(256, 192, 12, 64, 2), configured,
+                           xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 47: {  // 256 tokens x 160 features, ten wavefronts of 128 x 32
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 4, 1, 2, 5>, 256, 160, 640, 2, direct_lds_bytes(256, 160, 10, 64, 2), configured,
+                           xb, wb, ep, m, n, k, slices, stream);
     }
     case 23: {
       static bool configured = false;
-      return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 256, 2, direct_lds_bytes(128, 64, 2), configured, xb, wb, ep,
-                           m, n, k, slices, stream);
+      return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 128, 256, 2, direct_lds_bytes(128, 128, 4, 64, 2), configured,
+                           xb, wb, ep, m, n, k, slices, stream);
     }
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 22, 23, 44 or 45"); return -1;
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 22, 23, 44, 45, 46 or 47"); return -1;
   }
 }
 

@@ -233,13 +233,13 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 22, 23, 44, 45])
+@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 22, 23, 44, 45, 46, 47])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
     shorter than an LDS slice, whole and cut along k."""
     ops = ops_for(torch.bfloat16)
-    m, n, k = (13 if kernel == 16 else (300 if kernel in (44, 45) else 150)), (203 if kernel not in (44, 45) else 530), 1208
+    m, n, k = (13 if kernel == 16 else (300 if kernel >= 44 else 150)), (203 if kernel < 44 else 530), 1208
     x = _rand((m, k), torch.bfloat16, 61)
     w = _rand((n, k), torch.bfloat16, 62, 0.05)
     b = _rand((n,), torch.float32, 63)
@@ -256,13 +256,15 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
 @pytest.mark.parametrize("kernel,m,n", [(44, 2080, 1100), (44, 530, 3000), (44, 257, 256), (22, 1050, 700), (11, 532, 2373),
                                         (11, 90, 640), (12, 80, 1000), (44, 2112, 520), (44, 2113, 520), (45, 2080, 1100),
                                         (45, 530, 3000), (45, 257, 256), (23, 1050, 700), (23, 532, 2373), (23, 140, 640),
-                                        (45, 2112, 520), (45, 2113, 520)])
+                                        (45, 2112, 520), (45, 2113, 520), (46, 2080, 1100), (46, 257, 192), (46, 2112, 520),
+                                        (46, 2113, 400), (47, 2080, 1100), (47, 530, 3000), (47, 2176, 330), (47, 2177, 330)])
 @pytest.mark.parametrize("slices", [1, 2])
 def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
     """A last token tile whose tokens fit the first row of wavefronts (a prompt portion beside a few
     decoding requests) skips the matrix-core work of the others and is dealt out over the XCDs apart
-    from the full tiles: every tile of every slice is still computed exactly once.  (The last two
-    cases: 64 tokens in the last tile, which is light, and 65, which is not.)"""
+    from the full tiles: every tile of every slice is still computed exactly once.  (Beside them: 64
+    tokens in the last tile, which is light where a row of wavefronts has 64 tokens, and 65, which is
+    not; 128 and 129 where it has 128.)"""
     ops = ops_for(torch.bfloat16)
     k = 200
     x = _rand((m, k), torch.bfloat16, 81)
@@ -272,6 +274,21 @@ def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
     got = ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, partial_sums=True, mfma_kernel=kernel, slices=slices)
     total = got.cpu().double().sum(0) if slices > 1 else got.cpu().double()
     torch.testing.assert_close(total, ref, atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("m,n,k,chosen", [(2048, 4608, 200, 47), (2048, 17920, 896, 46), (2048, 5120, 264, 47)])
+def test_narrower_tiles_where_square_ones_leave_units_idle(ops_for, m, n, k, chosen):
+    """Products whose 256 x 256 tiles would not go round the compute units take tiles of 192 or 160
+    features by themselves (the 7B query/key/value width, a gate-up width, the 32B output width); the
+    result is the float64 product, and the same bits as when that kernel is forced."""
+    ops = ops_for(torch.bfloat16)
+    assert ops.lib.mlr_gemm_bf16_kernel(m, n, k, 1) == chosen
+    x = _rand((m, k), torch.bfloat16, 91)
+    w = _rand((n, k), torch.bfloat16, 92, 0.05)
+    b = _rand((n,), torch.float32, 93)
+    got = ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32)
+    torch.testing.assert_close(got.cpu().double(), x.double() @ w.double().t() + b.double(), atol=2e-3, rtol=1e-4)
+    assert torch.equal(got, ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, mfma_kernel=chosen))
 
 
 @pytest.mark.parametrize("m,n,chosen", [(64, 37888, 15), (41, 37890, 15), (40, 37888, 11), (64, 27648, 12), (50, 16000, 11),
