@@ -547,8 +547,9 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 }
 
 // ---- tiled, tiles loaded straight into LDS ---------------------------------------------------------
-// The square tiles of gemm_tiled_kernel (wavefronts of WM x WN blocks of 32 x 32 in a GM x GN arrangement)
-// with two changes to what a step of k costs beside its products.
+// The tiles of gemm_tiled_kernel (wavefronts of WM x WN blocks of 32 x 32 in a GM x GN arrangement; square
+// ones and, for products whose square tiles would not go round the compute units, 256 tokens x 192 or
+// x 160 features) with two changes to what a step of k costs beside its products.
 //  * The tiles go from memory into LDS without passing registers.  A lane's 16 bytes land at wavefront
 //    base + 16 * lane, so a row of a slice (BKT * 2 bytes) has no padding; instead its 16-byte pieces
 //    are stored in the order piece ^ key.  LDS serves sixteen lanes' 16 bytes a cycle from 64 banks
@@ -566,7 +567,9 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 // slower from 512 tokens on, up to 16 % faster at 128 to 256, where other tilings are chosen); a 64 x 64
 // tile (7 to 15 % slower than the staged kernel, which has two slices on their way, at up to 512 tokens
 // of weights that come from memory; equal beyond); eight wavefronts of 128 x 64 or 64 x 128 on the
-// 256 x 256 tile (like sixteen of 64 x 64); sixteen of 32 x 32 on the 128 x 128 tile (slower than four).
+// 256 x 256 tile (like sixteen of 64 x 64), four of 128 x 128 (7B gate-up 791 us against 571: one wavefront
+// per SIMD has nobody to fill its waits); sixteen of 32 x 32 on the 128 x 128 tile (slower than four).
+
 // LDS of a tile of `tokens` x `features` under `waves` wavefronts: every wavefront fills the same number
 // of 1 KB runs per buffer, so a buffer has room for whole rounds of them.
 constexpr int direct_lds_bytes(int tokens, int features, int waves, int bk, int buffers) {
