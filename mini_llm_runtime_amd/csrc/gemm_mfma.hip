@@ -242,10 +242,8 @@ struct TiledShape {
   static constexpr int kLds = 2 * (BM + BN) * kLd * 2;              // bytes, two buffers
   // slices of K in flight ahead of the one in LDS: one for the large tiles, two for the small ones
   // (a slice of their work is shorter than a trip to memory; four were no faster, also for the
-  // tile of few tokens, which only streams weights), three for the tile of 160 features, which has
-  // its compute unit to itself and two wavefronts to keep the loads going (7B gate-up at 64 tokens:
-  // one slice ahead 70 us, three 58, four 60)
-  static constexpr int kDepth = WN == 5 ? 3 : (WM * WN >= 4 || GM * GN > 4 ? 1 : 2);
+  // tile of few tokens, which only streams weights)
+  static constexpr int kDepth = WM * WN >= 4 || GM * GN > 4 ? 1 : 2;
 };
 
 // Workgroup -> (slice, token tile, feature tile).  Consecutive workgroups go to the eight
@@ -577,7 +575,7 @@ constexpr int direct_lds_bytes(int tokens, int features, int waves, int bk, int 
   return buffers * ((runs + waves - 1) / waves) * waves * 1024;
 }
 
-template <int KEEP, int WM, int WN, int GM, int GN, int BKT = kBK, int NBUF = 2>
+template <int KEEP, int WM, int WN, int GM, int GN, int BKT = kBK, int NBUF = 2, bool ONCE = false>
 __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                                   GemmEpilogue ep, TileOrder order, int M, int N, int K) {
   constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN, WAVES = GM * GN;
@@ -593,7 +591,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   constexpr int kPieces = (kRuns + WAVES - 1) / WAVES;
   // (loops over a wavefront's runs go to this fixed bound and break: with a bound that depends on the
   // template's parameters the host pass left the kernel uninstantiated, without a message)
-  constexpr int kMostPieces = 8;                // at most this many per wavefront
+  constexpr int kMostPieces = 16;               // at most this many per wavefront
   constexpr int kSteps = BKT / 16;              // products of k = 16 per slice
   static_assert(kPieces <= kMostPieces && BN % 32 == 0 && BM % 32 == 0, "whole runs of weight rows and of token rows");
   static_assert(WAVES % 2 == 0 && KEEP >= 1 && KEEP < kSteps + 1 && NBUF >= 2, "see the swizzle key and the loop");
@@ -646,7 +644,9 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
       __attribute__((address_space(3))) void* dst =
           (__attribute__((address_space(3))) void*)(smem + buf * kBufferBytes + (WAVES * p + wave) * 1024);
       const bool weights = (p + 1) * WAVES <= kWeightRuns || (p * WAVES < kWeightRuns && WAVES * p + wave < kWeightRuns);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(weights ? w_buf : x_buf, dst, 16, (piece_off[p] + s * (BKT * 2u)) | off_ok, 0, 0, 0);
+      const unsigned off = (piece_off[p] + s * (BKT * 2u)) | off_ok;
+      if (ONCE && weights) __builtin_amdgcn_raw_ptr_buffer_load_lds(w_buf, dst, 16, off, 0, 0, 2);  // read once: non-temporal
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(weights ? w_buf : x_buf, dst, 16, off, 0, 0, 0);
     }
   };
 
@@ -924,10 +924,8 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 // with the two larger ones, 46 / 47 = gemm_direct with tiles of 256 tokens x 192 features (twelve
 // wavefronts of 64 x 64) and x 160 features (ten of 128 x 32), 14 = gemm_tiled
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
-// rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 12 = gemm_tiled with tiles of 64
-// tokens x 128 features (four wavefronts) for 33 to 64 tokens of wide products, 15 = gemm_tiled with
-// tiles of 64 tokens x 160 features (two wavefronts) for 41 to 64 tokens of products whose tiles then
-// make whole rounds over the compute units.
+// rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 62 to 68 = gemm_direct with tiles of
+// 64 tokens x 64, 96, ... 256 features for up to 64 tokens (see choose_few_token_tiles).
 // A small matrix (an output projection of a narrow model) at 17 to 64 tokens: the tiled kernels have
 // too few tiles of it to keep the compute units busy, the row-splitting kernel with its 16 features a
 // workgroup has four times as many workgroups (0.5B output projection with the norm behind it, in a
@@ -935,28 +933,48 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 // Larger matrices read the tokens too often that way (0.5B gate-up at 64 tokens: 10 us tiled, 16).
 static bool small_matrix(int n, int k) { return static_cast<int64_t>(n) * k * 2 <= (4ll << 20); }
 
-// 33 to 64 tokens, whole K (gate-up, the output head): such a product streams its weight once, and
-// it is done when the busiest compute unit has streamed its share.  Per tiling, that share is the
-// rows of the tiles that land on one compute unit, and the rate is what a compute unit takes in
-// with that tiling, measured in a replayed graph at 64 tokens (GB/s; `alone`: one tile per unit):
-//   64 features: 21;  128 features: 23 alone, 26 beside another;  160 features: 20 alone, 27.
-// 7B gate-up (37,888 rows): 592 / 296 / 237 tiles -> 64 / 68 / 58 us; a 27,648-row gate-up with k
-// 5,120: 66 / 58 / 78; 32B gate-up: 128 / 105 / 120; the 7B output head: 238 / 211 / 198.  Up to
-// 40 tokens the 160-feature tile was never ahead.
-static int choose_mid_tiles(int m, int n) {
-  struct Tiling {
-    int kernel, features;
-    float alone, beside;
-  };
-  constexpr Tiling kTilings[] = {{11, 64, 21.f, 21.f}, {12, 128, 23.f, 26.f}, {15, 160, 20.f, 27.f}};
-  int best = 11;
+// Up to 64 tokens through tiles: such a product streams its weights once and is done when the busiest
+// compute unit has streamed its share, so what counts is how the tiles go round the 256 units and what
+// a unit takes in.  Fitted to replayed graphs over weights that come from memory (the five products of
+// seven model sizes at 8 to 64 tokens, 1,500 timings, rms error 9 %): a unit takes in 44 GB/s through the
+// tiles of gemm_direct and 37 through the register-staged ones, tokens included (a tile of 64 tokens x
+// 64 features reads as many token bytes as weight bytes, one of 256 features a fifth of that), all
+// units together 6.1 TB/s of weights (23.8 GB/s each), a launch costs 3.7 us and a round of tiles that
+// have their unit to themselves 2 us until their first bytes arrive (0.8 where two share a unit).
+// The tiles of 64 tokens x 64 ... 256 features of gemm_direct (a wavefront per 32 x 32 block; as many
+// slices of k in LDS as fit, 3 to 6, where the staged kernels have 2 on their way) are there so that some
+// width makes one round that fills the units: 7B gate-up (37,888 rows) at 64 tokens 67 us in staged
+// 64-feature tiles, 48.8 in 237 tiles of 160; 32B gate-up 130 to 92 (247 tiles of 224; at 8 tokens 101
+// to 92, 6.2 TB/s); cut along k in 8: 7B down 31.8 to 28.4, 32B down 69.6 to 50.1; the 7B output head
+// 244 to 212; 0.5B gate-up 10.3 to 8.9.  Over the sweep the chosen tilings add up to 1.4 % more than the
+// best ones, and to 7 % less than the staged 64-feature tiles everywhere.
+struct FewTokenTiling {
+  int kernel, tokens, features;
+  bool direct;
+  float round_us;  // per round of tiles
+};
+constexpr FewTokenTiling kFewTokenTilings[] = {
+    {62, 64, 64, true, 0.77f},  {63, 64, 96, true, 2.f},  {64, 64, 128, true, 2.f}, {65, 64, 160, true, 2.f}, {66, 64, 192, true, 2.f},
+    {67, 64, 224, true, 2.f},   {68, 64, 256, true, 2.f}, {14, 32, 64, false, 0.f}, {11, 64, 64, false, 0.f}};
+static float few_token_time_us(const FewTokenTiling& t, int m, int n, int k, int slices) {
+  constexpr float kDirectIntake = 44.f, kStagedIntake = 37.f, kUnitShare = 23.8f, kLaunch = 3.7f;  // GB/s, GB/s, GB/s, us
+  const int64_t groups = static_cast<int64_t>((n + t.features - 1) / t.features) * slices;
+  const float tile_kb = static_cast<float>(t.features) * ((k + slices - 1) / slices) * 2.f / 1e3f;
+  const float unit = (t.direct ? kDirectIntake : kStagedIntake) * t.features / (t.features + min(m, t.tokens));
+  const int64_t full = groups / kComputeUnits, rest = groups % kComputeUnits;
+  float time = kLaunch + full * (tile_kb / fminf(unit, kUnitShare) + t.round_us);
+  if (rest > 0) time += tile_kb / fminf(unit, kUnitShare * kComputeUnits / rest) + t.round_us;
+  return time;
+}
+static int choose_few_token_tiles(int m, int n, int k, int slices) {
+  int best = 0;
   float best_time = 0.f;
-  for (const Tiling& t : kTilings) {
-    if (t.kernel == 15 && m <= 40) continue;
-    const int64_t tiles = (n + t.features - 1) / t.features;
-    const int64_t per_unit = (tiles + kComputeUnits - 1) / kComputeUnits;
-    const float time = static_cast<float>(per_unit * t.features) / (per_unit > 1 ? t.beside : t.alone);
-    if (best_time == 0.f || time < best_time) best = t.kernel, best_time = time;
+  // narrow tiles first (at a tie the one that fills more units), the staged ones last and only when
+  // clearly ahead: where the estimate has them level the direct tile measured 10 to 20 % faster
+  for (const FewTokenTiling& t : kFewTokenTilings) {
+    if (m > t.tokens || (t.kernel == 11 && m <= 32)) continue;
+    const float time = few_token_time_us(t, m, n, k, slices);
+    if (best == 0 || time < (t.direct ? 0.99f : 0.97f) * best_time) best = t.kernel, best_time = time;
   }
   return best;
 }
@@ -964,12 +982,7 @@ static int choose_mid_tiles(int m, int n) {
 static int choose_kernel(int m, int n, int k, int slices) {
   if (m <= 16 && !few_tokens_tiled(n, slices)) return 16;
   if (m <= 64 && small_matrix(n, k)) return 16;
-  if (m <= 32) return 14;
-  // 33 to 64 tokens.  Cut along k (short runs of k per workgroup): tiles of 128 features once there
-  // are enough of them, else 64 (7B down in 8 slices 30.5 us either way, its output projection 10.6
-  // and 9.7 us; 160 features 41 and 15 us).
-  if (m <= 64 && slices == 1) return choose_mid_tiles(m, n);
-  if (m <= 64) return static_cast<int64_t>((n + 127) / 128) * slices >= 384 ? 12 : 11;
+  if (m <= 64) return choose_few_token_tiles(m, n, k, slices);
   const GemmPlan plan = plan_many_tokens(m, n, k, slices);
   return plan.slices == slices ? plan.kernel : 11;
 }
@@ -990,14 +1003,48 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
     }
     case 11: return launch_tiled<1, 1>(xb, wb, ep, m, n, k, slices, stream);
     case 14: return launch_tiled<1, 1, 1, 2>(xb, wb, ep, m, n, k, slices, stream);  // 32 tokens x 64 features, two wavefronts
-    case 12: return launch_tiled<1, 2, 2, 2>(xb, wb, ep, m, n, k, slices, stream);  // 64 tokens x 128 features
-    case 15: return launch_tiled<1, 5, 2, 1>(xb, wb, ep, m, n, k, slices, stream);  // 64 tokens x 160 features
     case 22: return launch_tiled<2, 2>(xb, wb, ep, m, n, k, slices, stream);
     case 44: return launch_tiled<2, 2, 4, 4>(xb, wb, ep, m, n, k, slices, stream);
     case 45: {
       static bool configured = false;
       return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 4>, 256, 256, 1024, 4, direct_lds_bytes(256, 256, 16, 64, 2), configured,
                            xb, wb, ep, m, n, k, slices, stream);
+    }
+    // 64 tokens x 64 to 256 features, a wavefront per 32 x 32 block, as many slices of k in LDS as fit
+    case 62: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 2, 64, 4, true>, 64, 64, 256, 2, direct_lds_bytes(64, 64, 4, 64, 4),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 63: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 3, 64, 6, true>, 64, 96, 384, 2, direct_lds_bytes(64, 96, 6, 64, 6),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 64: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 4, 64, 6, true>, 64, 128, 512, 2, direct_lds_bytes(64, 128, 8, 64, 6),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 65: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 5, 64, 5, true>, 64, 160, 640, 2, direct_lds_bytes(64, 160, 10, 64, 5),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 66: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 6, 64, 4, true>, 64, 192, 768, 2, direct_lds_bytes(64, 192, 12, 64, 4),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 67: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 7, 64, 3, true>, 64, 224, 896, 2, direct_lds_bytes(64, 224, 14, 64, 3),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
+    }
+    case 68: {
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 8, 64, 3, true>, 64, 256, 1024, 2, direct_lds_bytes(64, 256, 16, 64, 3),
+                           configured, xb, wb, ep, m, n, k, slices, stream);
     }
     case 46: {  // 256 tokens x 192 features, twelve wavefronts of 64 x 64
       static bool configured = false;
@@ -1014,7 +1061,7 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
       return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 128, 256, 2, direct_lds_bytes(128, 128, 4, 64, 2), configured,
                            xb, wb, ep, m, n, k, slices, stream);
     }
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 15, 14, 12, 11, 22, 23, 44, 45, 46 or 47"); return -1;
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 14, 11, 22, 23, 44 to 47 or 62 to 68"); return -1;
   }
 }
 

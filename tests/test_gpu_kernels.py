@@ -233,13 +233,13 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 15, 14, 12, 11, 22, 23, 44, 45, 46, 47])
+@pytest.mark.parametrize("kernel", [16, 14, 11, 22, 23, 44, 45, 46, 47, 62, 63, 64, 65, 66, 67, 68])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
     shorter than an LDS slice, whole and cut along k."""
     ops = ops_for(torch.bfloat16)
-    m, n, k = (13 if kernel == 16 else (300 if kernel >= 44 else 150)), (203 if kernel < 44 else 530), 1208
+    m, n, k = (13 if kernel == 16 else (300 if 44 <= kernel < 60 else 150)), (203 if kernel < 44 else 530), 1208
     x = _rand((m, k), torch.bfloat16, 61)
     w = _rand((n, k), torch.bfloat16, 62, 0.05)
     b = _rand((n,), torch.float32, 63)
@@ -254,7 +254,7 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
 
 
 @pytest.mark.parametrize("kernel,m,n", [(44, 2080, 1100), (44, 530, 3000), (44, 257, 256), (22, 1050, 700), (11, 532, 2373),
-                                        (11, 90, 640), (12, 80, 1000), (44, 2112, 520), (44, 2113, 520), (45, 2080, 1100),
+                                        (11, 90, 640), (44, 2112, 520), (44, 2113, 520), (45, 2080, 1100),
                                         (45, 530, 3000), (45, 257, 256), (23, 1050, 700), (23, 532, 2373), (23, 140, 640),
                                         (45, 2112, 520), (45, 2113, 520), (46, 2080, 1100), (46, 257, 192), (46, 2112, 520),
                                         (46, 2113, 400), (47, 2080, 1100), (47, 530, 3000), (47, 2176, 330), (47, 2177, 330)])
@@ -291,26 +291,33 @@ def test_narrower_tiles_where_square_ones_leave_units_idle(ops_for, m, n, k, cho
     assert torch.equal(got, ops.linear(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, mfma_kernel=chosen))
 
 
-@pytest.mark.parametrize("m,n,chosen", [(64, 37888, 15), (41, 37890, 15), (40, 37888, 11), (64, 27648, 12), (50, 16000, 11),
-                                        (64, 151936, 15)])
+@pytest.mark.parametrize("m,n,k,slices,chosen", [
+    (64, 37888, 512, 1, 65), (41, 37890, 512, 1, 65), (64, 27648, 512, 1, 64), (50, 16000, 1024, 1, 62), (64, 55296, 512, 1, 67),
+    (20, 55296, 1024, 1, 67), (8, 37888, 1024, 1, 65), (8, 37888, 512, 1, 14), (48, 59136, 512, 1, 68), (64, 17920, 512, 1, 63),
+    (33, 24000, 512, 1, 11), (64, 3584, 18944, 8, 64), (32, 5120, 5120, 8, 65), (40, 896, 4864, 8, 11),
+])
 @pytest.mark.parametrize("swiglu", [False, True])
-def test_wide_products_at_33_to_64_tokens(ops_for, m, n, chosen, swiglu):
-    """Whole-k products of 33 to 64 tokens choose their tile width (64, 128 or 160 features) by the
-    rounds their tiles make over the compute units; these widths reach each of the three, one with
-    a last tile that is not whole."""
+def test_tiles_for_up_to_64_tokens_chosen_by_rounds(ops_for, m, n, k, slices, chosen, swiglu):
+    """Products of up to 64 tokens through tiles choose the tile width (64 to 256 features, straight
+    into LDS, or the register-staged tiles of 64) by how the tiles go round the compute units and
+    what a unit takes in; these shapes reach every width, whole and cut along k, some with a last
+    tile that is not whole."""
+    if swiglu and slices > 1:
+        pytest.skip("partial sums have no SwiGLU")
     ops = ops_for(torch.bfloat16)
-    k = 136
     n = n - n % 4 if swiglu else n
-    assert ops.lib.mlr_gemm_bf16_kernel(m, n, k, 1) == chosen
+    assert ops.lib.mlr_gemm_bf16_kernel(m, n, k, slices) == chosen
     x = _rand((m, k), torch.bfloat16, 71)
-    w = _rand((n, k), torch.bfloat16, 72, 0.05)
-    ref = x.double() @ w.double().t()
+    w = (torch.randn((n, k), generator=torch.Generator(device="cuda").manual_seed(72), device="cuda") * 0.05).to(torch.bfloat16)
+    ref = x.cuda().double() @ w.double().t()
     if swiglu:
         quads = ref.view(m, -1, 4)
         gate, up = quads[..., :2], quads[..., 2:]
         ref = (gate * torch.sigmoid(gate) * up).reshape(m, -1)
-    got = ops.linear(x.cuda(), w.cuda(), None, swiglu=swiglu, out_dtype=None if swiglu else torch.float32)
-    torch.testing.assert_close(got.cpu().double(), ref, atol=2e-2 if swiglu else 2e-3, rtol=2e-2 if swiglu else 1e-4)
+    got = ops.linear(x.cuda(), w, None, swiglu=swiglu, out_dtype=None if swiglu else torch.float32, partial_sums=slices > 1, slices=slices if slices > 1 else None)
+    total = got.double().sum(0) if got.dim() == 3 else got.double()
+    scale = float(ref.abs().max())
+    torch.testing.assert_close(total, ref, atol=(2e-2 if swiglu else 2e-3) * max(1.0, scale), rtol=2e-2 if swiglu else 1e-4)
 
 
 @pytest.mark.parametrize("m", [17, 31, 32, 33, 50, 64])
