@@ -83,8 +83,8 @@ int mlr_gemm_bf16_slices(int m, int n, int k, int max_slices);
 int mlr_gemm_bf16_kernel(int m, int n, int k, int slices);
 // `kernel` 0 lets the shape choose; 16 (streaming, up to 64 tokens), 14 (LDS-tiled, tiles of 32
 // tokens x 64 features), 11, 22, 44 (LDS-tiled with 64 x 64, 128 x 128, 256 x 256 tiles), 23, 45 (the
-// two larger tiles loaded straight into LDS), 46, 47 (the same with tiles of 256 tokens x 192 and
-// x 160 features), 62 to 68 (64 tokens x 64, 96, ... 256 features straight into LDS, for up to 64
+// two larger tiles loaded straight into LDS), 46, 47, 48 (the same with tiles of 256 tokens x 192,
+// x 160 and x 320 features), 62 to 68 (64 tokens x 64, 96, ... 256 features straight into LDS, for up to 64
 // tokens) force one, for tests and tuning.
 // Any `slices` within
 // 1..64 is accepted with a float32 [slices, m, n] output.

@@ -568,11 +568,11 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_tiled_kernel(const bf16* __
 // 256 x 256 tile (like sixteen of 64 x 64), four of 128 x 128 (7B gate-up 791 us against 571: one wavefront
 // per SIMD has nobody to fill its waits); sixteen of 32 x 32 on the 128 x 128 tile (slower than four).
 
-// LDS of a tile of `tokens` x `features` under `waves` wavefronts: every wavefront fills the same number
-// of 1 KB runs per buffer, so a buffer has room for whole rounds of them.
+// LDS of a tile of `tokens` x `features` under `waves` wavefronts: a buffer holds the tile's 1 KB runs
+// and, where they do not go round the wavefronts, one more for the surplus loads (see kPieces).
 constexpr int direct_lds_bytes(int tokens, int features, int waves, int bk, int buffers) {
   const int runs = (tokens + features) * bk * 2 / 1024;
-  return buffers * ((runs + waves - 1) / waves) * waves * 1024;
+  return buffers * (runs + (runs % waves != 0 ? 1 : 0)) * 1024;
 }
 
 template <int KEEP, int WM, int WN, int GM, int GN, int BKT = kBK, int NBUF = 2, bool ONCE = false>
@@ -586,8 +586,8 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   constexpr int kRuns = (BM + BN) / kRunRows;   // dealt out to the wavefronts in turn
   constexpr int kWeightRuns = BN / kRunRows;    // the first of them are weight rows, the others token rows
   // Every wavefront issues kPieces loads per slice (the wait counters count instructions); where the
-  // runs do not go round, the last wavefronts' surplus loads are out of range and bring zeros to slots
-  // of their own behind the tile.
+  // runs do not go round, the last wavefronts' surplus loads are out of range and bring zeros to one
+  // spare run behind the tile, which nobody reads.
   constexpr int kPieces = (kRuns + WAVES - 1) / WAVES;
   // (loops over a wavefront's runs go to this fixed bound and break: with a bound that depends on the
   // template's parameters the host pass left the kernel uninstantiated, without a message)
@@ -597,7 +597,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
   static_assert(WAVES % 2 == 0 && KEEP >= 1 && KEEP < kSteps + 1 && NBUF >= 2, "see the swizzle key and the loop");
   constexpr int kInFlight = (NBUF - 2) * kPieces;  // loads of this wavefront that may still be out when a slice is needed
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  constexpr int kBufferBytes = kPieces * WAVES * 1024;
+  constexpr int kBufferBytes = (kRuns + (kRuns % WAVES != 0 ? 1 : 0)) * 1024;
   __shared__ float scales[BM];
 
   const int tid = threadIdx.x;
@@ -642,7 +642,7 @@ __global__ __launch_bounds__(64 * GM * GN) void gemm_direct_kernel(const bf16* _
     for (int p = 0; p < kMostPieces; ++p) {
       if (p >= kPieces) break;
       __attribute__((address_space(3))) void* dst =
-          (__attribute__((address_space(3))) void*)(smem + buf * kBufferBytes + (WAVES * p + wave) * 1024);
+          (__attribute__((address_space(3))) void*)(smem + buf * kBufferBytes + min(WAVES * p + wave, kRuns) * 1024);
       const bool weights = (p + 1) * WAVES <= kWeightRuns || (p * WAVES < kWeightRuns && WAVES * p + wave < kWeightRuns);
       const unsigned off = (piece_off[p] + s * (BKT * 2u)) | off_ok;
       if (ONCE && weights) __builtin_amdgcn_raw_ptr_buffer_load_lds(w_buf, dst, 16, off, 0, 0, 2);  // read once: non-temporal
@@ -881,11 +881,17 @@ struct TilingCost {
 // tiles) 130 to 112, 1.5B gate-up 139 to 132; 7B gate-up at 512 tokens 199 to 165.  Over the four
 // products of four model sizes at 256 to 4,096 tokens the chosen pairs add up to 0.6 % more than the
 // best pairs.  (256 x 224 by fourteen wavefronts was level with 256 x 256 and is not built.)
+// 256 x 320 by eight wavefronts of 64 x 160 (ten wavefronts have too few registers each) needs 0.7
+// operand reads per product where the square tile needs 1, and makes one round where the others make
+// two: 0.5B gate-up (248 tiles) 53 to 49 us, 7B gate-up at 512 tokens 168 to 135, 7B query/key/value at
+// 4,096 tokens 159 to 134, 32B down at 4,096 tokens 1,084 to 938; level or behind where the square
+// tiles already go round (7B gate-up at 2,048 tokens 533 against 517 on weights from memory).
 constexpr TilingCost kTilingCosts[] = {{11, 64, 64, 8, 0.401f, 0.251f, 6.4f},
                                        {23, 128, 128, 2, 0.927f, 0.579f, 6.5f},
                                        {45, 256, 256, 1, 1.09f, 1.84f, 10.5f},
                                        {46, 256, 192, 1, 0.86f, 1.45f, 10.5f},
-                                       {47, 256, 160, 1, 0.79f, 1.34f, 10.5f}};
+                                       {47, 256, 160, 1, 0.79f, 1.34f, 10.5f},
+                                       {48, 256, 320, 1, 1.39f, 2.35f, 12.f}};
 constexpr int kComputeUnits = 256;
 static float tiled_time_us(const TilingCost& c, int m, int n, int k, int slices) {
   const int64_t tiles = static_cast<int64_t>((m + c.tile_tokens - 1) / c.tile_tokens) * ((n + c.tile_features - 1) / c.tile_features);
@@ -921,8 +927,8 @@ static GemmPlan plan_many_tokens(int m, int n, int k, int max_slices) {
 
 // The kernel for a shape: 16 = gemm_skinny_split, 11 / 22 / 44 = gemm_tiled with 64 x 64,
 // 128 x 128 (four wavefronts each) and 256 x 256 (sixteen wavefronts) tiles, 23 / 45 = gemm_direct
-// with the two larger ones, 46 / 47 = gemm_direct with tiles of 256 tokens x 192 features (twelve
-// wavefronts of 64 x 64) and x 160 features (ten of 128 x 32), 14 = gemm_tiled
+// with the two larger ones, 46 / 47 / 48 = gemm_direct with tiles of 256 tokens x 192 features (twelve
+// wavefronts of 64 x 64), x 160 features (ten of 128 x 32) and x 320 features (eight of 64 x 160), 14 = gemm_tiled
 // with tiles of 32 tokens x 64 features (two wavefronts): for up to 32 tokens it stages half the
 // rows of the 64 x 64 tile and streams weights 5 to 15 % faster, 62 to 68 = gemm_direct with tiles of
 // 64 tokens x 64, 96, ... 256 features for up to 64 tokens (see choose_few_token_tiles).
@@ -1046,6 +1052,11 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
       return launch_direct(gemm_direct_kernel<1, 1, 1, 2, 8, 64, 3, true>, 64, 256, 1024, 2, direct_lds_bytes(64, 256, 16, 64, 3),
                            configured, xb, wb, ep, m, n, k, slices, stream);
     }
+    case 48: {  // 256 tokens x 320 features, eight wavefronts of 64 x 160
+      static bool configured = false;
+      return launch_direct(gemm_direct_kernel<1, 2, 5, 4, 2>, 256, 320, 512, 4, direct_lds_bytes(256, 320, 8, 64, 2), configured,
+                           xb, wb, ep, m, n, k, slices, stream);
+    }
     case 46: {  // 256 tokens x 192 features, twelve wavefronts of 64 x 64
       static bool configured = false;
       return launch_direct(gemm_direct_kernel<1, 2, 2, 4, 3>, 256, 192, 768, 4, direct_lds_bytes(256, 192, 12, 64, 2), configured,
@@ -1061,7 +1072,7 @@ static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int
       return launch_direct(gemm_direct_kernel<1, 2, 2, 2, 2>, 128, 128, 256, 2, direct_lds_bytes(128, 128, 4, 64, 2), configured,
                            xb, wb, ep, m, n, k, slices, stream);
     }
-    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 14, 11, 22, 23, 44 to 47 or 62 to 68"); return -1;
+    default: set_error("mlr_gemm_bf16: kernel must be 0 (chosen by shape), 16, 14, 11, 22, 23, 44 to 48 or 62 to 68"); return -1;
   }
 }
 

@@ -413,7 +413,7 @@ class HipOps:
         accepts, instead of [M, N], a float32 stack [S, M, N] of partial sums over slices
         of k (bias in slice 0).  Narrow products of a few tokens are cut that way so that
         all compute units stream the weight; the norm kernel adds the slices in order.
-        mfma_kernel, slices: force one of the matrix-core kernels (16, 14, 11, 22, 23, 44 to 47, 62 to 68) and a number
+        mfma_kernel, slices: force one of the matrix-core kernels (16, 14, 11, 22, 23, 44 to 48, 62 to 68) and a number
         of k slices instead of letting the shape choose; for tests and tuning.
         """
         if kernel not in ("auto", "fma"):

@@ -308,7 +308,7 @@ def test_product_that_finishes_the_stream(gpu_device, m, n, k, bias, weight_f32)
     gate, up = quads[..., :2], quads[..., 2:]
     torch.testing.assert_close(glu.cpu().double(), (gate * torch.sigmoid(gate) * up).reshape(m, -1), atol=2e-2, rtol=3e-2)
     # every matrix-core kernel that takes these tokens pays the factor the same way
-    for kernel in (16, 14, 11, 23, 45, 46, 47, 62, 65, 68):
+    for kernel in (16, 14, 11, 23, 45, 46, 47, 48, 62, 65, 68):
         if (kernel == 14 and m > 32) or n % 8:
             continue
         forced = ops.linear(owed, w2.cuda(), b2.cuda(), out_dtype=torch.float32, mfma_kernel=kernel)

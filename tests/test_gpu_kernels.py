@@ -233,7 +233,7 @@ def test_k_slices_chosen_for_many_tokens(ops_for):
     assert lib.mlr_gemm_bf16_slices(96, 3584, 18944, 8) > 1
 
 
-@pytest.mark.parametrize("kernel", [16, 14, 11, 22, 23, 44, 45, 46, 47, 62, 63, 64, 65, 66, 67, 68])
+@pytest.mark.parametrize("kernel", [16, 14, 11, 22, 23, 44, 45, 46, 47, 48, 62, 63, 64, 65, 66, 67, 68])
 @pytest.mark.parametrize("slices", [1, 3])
 def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
     """Every bfloat16 kernel forced at sizes that are no multiple of its tile, with a tail of k
@@ -257,7 +257,8 @@ def test_each_matrix_core_kernel_at_odd_sizes(ops_for, kernel, slices):
                                         (11, 90, 640), (44, 2112, 520), (44, 2113, 520), (45, 2080, 1100),
                                         (45, 530, 3000), (45, 257, 256), (23, 1050, 700), (23, 532, 2373), (23, 140, 640),
                                         (45, 2112, 520), (45, 2113, 520), (46, 2080, 1100), (46, 257, 192), (46, 2112, 520),
-                                        (46, 2113, 400), (47, 2080, 1100), (47, 530, 3000), (47, 2176, 330), (47, 2177, 330)])
+                                        (46, 2113, 400), (47, 2080, 1100), (47, 530, 3000), (47, 2176, 330), (47, 2177, 330), (48, 2080, 1100),
+                                        (48, 2112, 700), (48, 2113, 330)])
 @pytest.mark.parametrize("slices", [1, 2])
 def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
     """A last token tile whose tokens fit the first row of wavefronts (a prompt portion beside a few
@@ -276,10 +277,11 @@ def test_tiles_with_few_tokens_at_the_lower_edge(ops_for, kernel, m, n, slices):
     torch.testing.assert_close(total, ref, atol=2e-3, rtol=1e-4)
 
 
-@pytest.mark.parametrize("m,n,k,chosen", [(2048, 4608, 200, 47), (2048, 17920, 896, 46), (2048, 5120, 264, 47)])
+@pytest.mark.parametrize("m,n,k,chosen", [(2048, 4608, 200, 47), (2048, 9728, 264, 48), (2048, 5120, 264, 47), (512, 37888, 520, 48)])
 def test_narrower_tiles_where_square_ones_leave_units_idle(ops_for, m, n, k, chosen):
-    """Products whose 256 x 256 tiles would not go round the compute units take tiles of 192 or 160
-    features by themselves (the 7B query/key/value width, a gate-up width, the 32B output width); the
+    """Products whose 256 x 256 tiles would not go round the compute units take tiles of 160, 192 or
+    320 features by themselves (the 7B query/key/value width, the 0.5B gate-up width, the 32B output
+    width, the 7B gate-up at 512 tokens); the
     result is the float64 product, and the same bits as when that kernel is forced."""
     ops = ops_for(torch.bfloat16)
     assert ops.lib.mlr_gemm_bf16_kernel(m, n, k, 1) == chosen
