@@ -964,12 +964,15 @@ constexpr FewTokenTiling kFewTokenTilings[] = {
     {67, 64, 224, true, 2.f},   {68, 64, 256, true, 2.f}, {14, 32, 64, false, 0.f}, {11, 64, 64, false, 0.f}};
 static float few_token_time_us(const FewTokenTiling& t, int m, int n, int k, int slices) {
   constexpr float kDirectIntake = 44.f, kStagedIntake = 37.f, kUnitShare = 23.8f, kLaunch = 3.7f;  // GB/s, GB/s, GB/s, us
-  const int64_t groups = static_cast<int64_t>((n + t.features - 1) / t.features) * slices;
+  // more tokens than a tile: every tile of tokens streams the weights again, but only the first from memory
+  const int token_tiles = (m + t.tokens - 1) / t.tokens;
+  const int64_t groups = static_cast<int64_t>((n + t.features - 1) / t.features) * slices * token_tiles;
   const float tile_kb = static_cast<float>(t.features) * ((k + slices - 1) / slices) * 2.f / 1e3f;
   const float unit = (t.direct ? kDirectIntake : kStagedIntake) * t.features / (t.features + min(m, t.tokens));
+  const float share = kUnitShare * token_tiles;
   const int64_t full = groups / kComputeUnits, rest = groups % kComputeUnits;
-  float time = kLaunch + full * (tile_kb / fminf(unit, kUnitShare) + t.round_us);
-  if (rest > 0) time += tile_kb / fminf(unit, kUnitShare * kComputeUnits / rest) + t.round_us;
+  float time = kLaunch + full * (tile_kb / fminf(unit, share) + t.round_us);
+  if (rest > 0) time += tile_kb / fminf(unit, share * kComputeUnits / rest) + t.round_us;
   return time;
 }
 static int choose_few_token_tiles(int m, int n, int k, int slices) {
@@ -978,7 +981,7 @@ static int choose_few_token_tiles(int m, int n, int k, int slices) {
   // narrow tiles first (at a tie the one that fills more units), the staged ones last and only when
   // clearly ahead: where the estimate has them level the direct tile measured 10 to 20 % faster
   for (const FewTokenTiling& t : kFewTokenTilings) {
-    if (m > t.tokens || (t.kernel == 11 && m <= 32)) continue;
+    if ((t.kernel == 14 && m > t.tokens) || (t.kernel == 11 && m <= 32)) continue;
     const float time = few_token_time_us(t, m, n, k, slices);
     if (best == 0 || time < (t.direct ? 0.99f : 0.97f) * best_time) best = t.kernel, best_time = time;
   }
@@ -990,7 +993,13 @@ static int choose_kernel(int m, int n, int k, int slices) {
   if (m <= 64 && small_matrix(n, k)) return 16;
   if (m <= 64) return choose_few_token_tiles(m, n, k, slices);
   const GemmPlan plan = plan_many_tokens(m, n, k, slices);
-  return plan.slices == slices ? plan.kernel : 11;
+  const int kernel = plan.slices == slices ? plan.kernel : 11;
+  // up to 256 tokens in tiles of 64: the same choice of widths as for one tile of tokens (7B down at 128
+  // tokens in 4 slices: 50.6 us staged, 41.8 in tiles of 128 features; 32B down at 192 tokens 131 and
+  // 106).  Not for small matrices: the staged tiles, four workgroups to a compute unit, share the weights
+  // of neighbouring token tiles (1.5B query/key/value, 6 MB, at 192 tokens: 7.4 us against 9.1).
+  if (kernel == 11 && m <= 256 && static_cast<int64_t>(n) * k * 2 >= (16ll << 20)) return choose_few_token_tiles(m, n, k, slices);
+  return kernel;
 }
 
 static int gemm_bf16(const bf16* xb, const bf16* wb, const GemmEpilogue& ep, int m, int n, int k, int slices,
