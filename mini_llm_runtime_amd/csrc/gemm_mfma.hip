@@ -54,7 +54,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   __shared__ float red[WAVES][MT][kWave][4];
   __shared__ float scales[MT * 16];
   RowScaleLoads<MT * 16 / WAVES, 4 / MT> owed;  // up to 256 partial sums a row for 16 tokens, 64 for 64 tokens
-  if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, 0, min(M, MT * 16), M);
+  const int token0 = blockIdx.z * (MT * 16);  // grid.z: further groups of MT slabs, a workgroup each
+  if (ep.row_sumsq != nullptr) row_scales_issue(ep, owed, token0, min(M - token0, MT * 16), M);
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int r = lane % 16;
@@ -85,8 +86,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   f32x4_t acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    xp[mt] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(mt * 16 + r, M - 1)) * K);
-    xok[mt] = mt * 16 + r < M;
+    xp[mt] = reinterpret_cast<const bf16x8_t*>(x + static_cast<int64_t>(min(token0 + mt * 16 + r, M - 1)) * K);
+    xok[mt] = token0 + mt * 16 + r < M;
     acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][mt][lane][i] = acc[mt][i];
-  if (ep.row_sumsq != nullptr) row_scales_finish(ep, owed, 0, min(M, MT * 16), M, K, scales);
+  if (ep.row_sumsq != nullptr) row_scales_finish(ep, owed, token0, min(M - token0, MT * 16), M, K, scales);
   __syncthreads();
   // Slab mt is finished by wavefront mt % WAVES: the epilogue of a slab waits for memory more than once
   // (rotation tables, cache slots, the stores), and one wavefront doing four slabs in turn was a third
@@ -128,9 +129,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_split_kernel(const bf1
     for (int ww = 0; ww < WAVES; ++ww)
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] += red[ww][mt][lane][i];
-    const int token = mt * 16 + r;
+    const int token = token0 + mt * 16 + r;
     if (ep.row_sumsq != nullptr && token < M) {
-      const float scale = scales[token];
+      const float scale = scales[mt * 16 + r];
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= scale;
     }
@@ -1201,6 +1202,12 @@ int mlr_qkv_rope_write_bf16(const void* x, const void* w, const void* bias, int 
       gemm_skinny_qkv8_kernel<4><<<dim3(static_cast<unsigned>(n / 8)), 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
     else if (m <= 16)
       gemm_skinny_split_kernel<4, true, 1><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
+    else if (n * k * 2 <= (8ll << 20))
+      // a small matrix: a workgroup per slab of 16 tokens reads a quarter of the tokens and the weights
+      // again from L2, where one workgroup for all slabs is held up by the tokens it takes in (0.5B at
+      // 64 tokens 8.4 to 6.8 us, at 48 7.7 to 5.2; 1.5B at 64 12.0 to 10.1; a 10 MB matrix: 14.6 to 16.1).
+      // The same sums in the same order either way.
+      gemm_skinny_split_kernel<4, true, 1><<<dim3(grid.x, 1, (m + 15) / 16), 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
     else if (m <= 32)
       gemm_skinny_split_kernel<4, true, 2><<<grid, 256, 0, stream>>>(xb, wb, ep, target, m, static_cast<int>(n), k);
     else
